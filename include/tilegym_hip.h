@@ -1,0 +1,156 @@
+/*
+ * tilegym_hip.h -- C ABI of libtilegym_hip.so: FP8 (OCP e4m3fn) GEMM for AMD gfx950 (MI355X).
+ *
+ * One shared library, plain pointers and sizes, no framework types.  Every entry point
+ *   - borrows the memory it is given (never frees, never keeps a pointer),
+ *   - validates its arguments on the host BEFORE touching the device (so argument errors
+ *     are reported without a GPU),
+ *   - enqueues its kernels on the given HIP stream and returns without synchronising,
+ *   - returns an int32 code: 0 = ok, negative = error (see tg_rc_message).
+ *
+ * The tensor descriptor and the return codes keep the layout / numbering of the
+ * reference's own C-ABI precedent (TensorDesc: src/tilegym/ops/cutile_rs/ffi_util.rs:26-35,
+ * rc codes: src/tilegym/ops/cutile_rs/ffi_util.rs:108-122).
+ */
+#ifndef TILEGYM_HIP_H
+#define TILEGYM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TG_ABI_VERSION 1
+#define TG_MAX_DIMS 5
+
+/* dtype codes (src/tilegym/ops/cutile_rs/ffi_util.rs:32-34) */
+enum {
+    TG_F32 = 0,
+    TG_F16 = 1,
+    TG_BF16 = 2,
+    TG_I32 = 3,
+    TG_I64 = 4,
+    TG_F8E5M2 = 5,
+    TG_F8E4M3FN = 7
+};
+
+/* return codes (src/tilegym/ops/cutile_rs/ffi_util.rs:108-122); -1 is reserved as the
+ * "auto" sentinel of the cfg array and is never returned. */
+enum {
+    TG_OK = 0,
+    TG_ERR_DTYPE = -2,
+    TG_ERR_LAUNCH = -3,
+    TG_ERR_DEVICE = -4,
+    TG_ERR_NULL = -5,
+    TG_ERR_INVALID = -6
+};
+
+/* Borrowed view of a device tensor.  Strides are in ELEMENTS. */
+typedef struct tg_tensor {
+    uint64_t ptr;
+    int32_t ndim;
+    int64_t shape[TG_MAX_DIMS];
+    int64_t strides[TG_MAX_DIMS];
+    int32_t dtype;
+} tg_tensor;
+
+/* cfg[] slots: tile / schedule overrides, -1 (or a short array) = choose automatically.
+ * This is the C form of the reference's per-call `kernel_configs={...}` override
+ * (src/tilegym/kernel_utils.py:14-36). */
+enum {
+    TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (weight-streaming) kernel */
+    TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (64/128/256)            */
+    TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (128/256)               */
+    TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
+    TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4)         */
+    TG_CFG_COUNT = 8
+};
+
+/*
+ * Dense FP8 GEMM:  C <- alpha * (sa * op(A)) @ (sb * op(B)) + beta * C
+ *
+ * Replaces, for e4m3 inputs, the launch half of
+ *   tilegym.ops.matmul                      src/tilegym/ops/cutile/matmul.py:421-455
+ *   flashinfer gemm_alpha_beta              src/tilegym/suites/flashinfer/cutile/gemm/gemm_alpha_beta.py:336-504
+ *   unsloth w8a8_block_fp8_matmul           src/tilegym/suites/unsloth/cutile/fp8.py:388-446
+ *
+ * a: (M,K), or (K,M) when trans_a;  b: (K,N), or (N,K) when trans_b;  both e4m3fn, contiguous.
+ * c: (M,N) contiguous, dtype bf16 / f32 / f16.  beta != 0 reads c.
+ * scale_a / scale_b (f32, device memory):
+ *     NULL                     -> 1.0
+ *     1 element                -> per-tensor scale
+ *     scale_a (M, ceil(K/128)) and scale_b (ceil(N/128), ceil(K/128)) -> block scaled:
+ *        C[m,n] = sum_kb scale_a[m,kb] * scale_b[n/128,kb] * sum_{k in kb} A[m,k] * B[n,k]
+ *     (both must be of the same kind; block form requires the NT layout.)
+ * workspace: NULL, or a u8/any-dtype 1-D buffer of at least tg_fp8_gemm_workspace_bytes()
+ *     bytes that was ZERO-FILLED when allocated; the library leaves its counter region
+ *     zeroed on return, so one buffer can serve every later call on the same stream.
+ *     Calls that share a workspace must not overlap in time.  Without a workspace the
+ *     split-K schedules are not used.
+ */
+int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                    const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
+                    int32_t trans_b, float alpha, float beta, const tg_tensor* workspace,
+                    const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream);
+
+/* Bytes of workspace that let tg_fp8_gemm use every schedule for this problem
+ * (trans_b == 0 adds room for a K-contiguous copy of B).  Never fails; returns 0 for
+ * non-positive sizes. */
+int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t trans_b,
+                                    const int32_t* cfg, int32_t ncfg);
+
+/*
+ * Grouped (expert-offset) block-scaled FP8 GEMM, NT layout:
+ *   for q in [0,Q):  C[m_indptr[q]:m_indptr[q+1]] = (A[rows] * a_scale) @ (B[q] * b_scale[q])^T
+ *
+ * Replaces the launch half of flashinfer ragged_block_scaled_bmm
+ *   src/tilegym/suites/flashinfer/cutile/gemm/ragged_block_scaled_bmm.py:497-616
+ * a (total_m,K) e4m3; b (Q,N,K) e4m3; a_scale (total_m, ceil(K/128)) f32 or NULL (ones);
+ * b_scale (Q, ceil(N/128), ceil(K/128)) f32, or NULL (ones);
+ * m_indptr (Q+1) i32 DEVICE memory, non-decreasing, m_indptr[Q] <= total_m; segments need no
+ * alignment and may be empty.  Rows at or past m_indptr[Q] are not written.
+ * c (total_m,N) bf16/f32/f16.
+ */
+int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                           const tg_tensor* a_scale, const tg_tensor* b_scale,
+                           const tg_tensor* m_indptr, const int32_t* cfg, int32_t ncfg,
+                           int32_t device_id, uint64_t hip_stream);
+
+/*
+ * Token-gather MoE GEMM (block-scaled FP8, NT):
+ *   for every slot r < num_tokens_post_padded with id = sorted_token_ids[r] < num_valid:
+ *       C[id] = (A[id / top_k] * a_scale) @ (B[expert_ids[r / block_m]] * b_scale)^T  (* topk_weights[id])
+ *
+ * Replaces the launch half of invoke_fused_moe_kernel's use_fp8_w8a8 path
+ *   src/tilegym/ops/tilecpp/moe.py:241-310, kernel src/tilegym/ops/tilecpp/moe.cuh:72-225
+ * a (T,K) e4m3; b (E,N,K) e4m3; c (num_valid, N) bf16/f32/f16 (the (T,top_k,N) cache, flattened);
+ * a_scale (T, ceil(K/128)) or NULL; b_scale (E, ceil(N/128), ceil(K/128)) or NULL;
+ * topk_weights (num_valid) f32 or NULL (required when mul_routed_weight != 0);
+ * sorted_token_ids (EM) i32, expert_ids (>= EM/block_m) i32, num_tokens_post_padded (1) i32,
+ * all DEVICE memory, as produced by moe_align_block_size with block size block_m
+ * (src/tilegym/ops/cutile/moe_align_block.py:205-268); block_m must be a multiple of 16.
+ */
+int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                        const tg_tensor* a_scale, const tg_tensor* b_scale,
+                        const tg_tensor* topk_weights, const tg_tensor* sorted_token_ids,
+                        const tg_tensor* expert_ids, const tg_tensor* num_tokens_post_padded,
+                        int32_t mul_routed_weight, int32_t top_k, int32_t block_m,
+                        const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream);
+
+/* The schedule the most recent GEMM call on this host thread chose: fills out[0..n) with the
+ * TG_CFG_* slots (kernel, BLOCK_M, BLOCK_N, SPLIT_K, ROW_GROUPS).  Returns slots written. */
+int32_t tg_last_config(int32_t* out, int32_t n);
+
+/* Static message for a return code (src/tilegym/ops/cutile_rs/ffi_util.rs:125-135). */
+const char* tg_rc_message(int32_t rc);
+
+/* Detail text of the most recent error on this host thread ("" if none). */
+const char* tg_last_error(void);
+
+int32_t tg_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TILEGYM_HIP_H */

@@ -1,0 +1,234 @@
+"""ctypes binding of libtilegym_hip.so: tensor descriptors, return-code checks, workspaces.
+
+This is the only module that touches the shared library.  It never falls back to another
+implementation: if the library is missing or a call fails, it raises.
+
+The descriptor / return-code conventions follow the reference's own C-ABI precedent
+(src/tilegym/backend/cutile_rs/utils.py:268-290 ``make_tensor_desc``, :353-370 ``check_rc``).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Dict, Optional, Sequence, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_ENV = "TILEGYM_HIP_LIB"
+DEFAULT_LIB_PATH = os.path.join(_HERE, "libtilegym_hip.so")
+
+TG_MAX_DIMS = 5
+TG_CFG_COUNT = 8
+CFG_SLOTS = {"KERNEL": 0, "BLOCK_M": 1, "BLOCK_N": 2, "SPLIT_K": 3, "ROW_GROUPS": 4}
+KERNEL_NAMES = {0: "fallback", 1: "tiled", 2: "skinny"}
+
+# dtype codes of the ABI (include/tilegym_hip.h)
+_DTYPE_CODES = {
+    torch.float32: 0,
+    torch.float16: 1,
+    torch.bfloat16: 2,
+    torch.int32: 3,
+    torch.int64: 4,
+    torch.float8_e5m2: 5,
+    torch.uint8: 6,
+    torch.float8_e4m3fn: 7,
+}
+
+_RC_NAMES = {0: "ok", -2: "unsupported dtype", -3: "kernel launch failed", -4: "device init failed",
+             -5: "null tensor pointer", -6: "invalid arguments"}
+
+
+class TgTensor(ctypes.Structure):
+    _fields_ = [
+        ("ptr", ctypes.c_uint64),
+        ("ndim", ctypes.c_int32),
+        ("shape", ctypes.c_int64 * TG_MAX_DIMS),
+        ("strides", ctypes.c_int64 * TG_MAX_DIMS),
+        ("dtype", ctypes.c_int32),
+    ]
+
+
+class TileGymHipError(RuntimeError):
+    def __init__(self, rc: int, where: str, detail: str):
+        self.rc = rc
+        msg = f"{where}: rc={rc} ({_RC_NAMES.get(rc, 'unknown error')})"
+        if detail:
+            msg += f": {detail}"
+        super().__init__(msg)
+
+
+_lib = None
+
+
+def lib_path() -> str:
+    return os.environ.get(LIB_ENV, DEFAULT_LIB_PATH)
+
+
+def is_built() -> bool:
+    return os.path.exists(lib_path())
+
+
+def load():
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"libtilegym_hip.so not found at {path}; build it with "
+            f"`python -m tilegym_amd.build` (hipcc, gfx950). There is no fallback implementation.")
+    L = ctypes.CDLL(path)
+    P = ctypes.POINTER(TgTensor)
+    I32P = ctypes.POINTER(ctypes.c_int32)
+    L.tg_abi_version.restype = ctypes.c_int32
+    L.tg_rc_message.restype = ctypes.c_char_p
+    L.tg_rc_message.argtypes = [ctypes.c_int32]
+    L.tg_last_error.restype = ctypes.c_char_p
+    L.tg_last_config.restype = ctypes.c_int32
+    L.tg_last_config.argtypes = [I32P, ctypes.c_int32]
+    L.tg_fp8_gemm_workspace_bytes.restype = ctypes.c_int64
+    L.tg_fp8_gemm_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                              ctypes.c_int32, I32P, ctypes.c_int32]
+    L.tg_fp8_gemm.restype = ctypes.c_int32
+    L.tg_fp8_gemm.argtypes = [P, P, P, P, P, ctypes.c_int32, ctypes.c_int32, ctypes.c_float,
+                              ctypes.c_float, P, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_ragged_gemm.restype = ctypes.c_int32
+    L.tg_fp8_ragged_gemm.argtypes = [P, P, P, P, P, P, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_moe_gemm.restype = ctypes.c_int32
+    L.tg_fp8_moe_gemm.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_int32, ctypes.c_int32,
+                                  ctypes.c_int32, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    if L.tg_abi_version() != 1:
+        raise RuntimeError(f"libtilegym_hip.so ABI version {L.tg_abi_version()} != 1")
+    _lib = L
+    return L
+
+
+def make_tensor_desc(t: Optional[torch.Tensor]) -> Optional[TgTensor]:
+    """Borrowed descriptor of a torch tensor (strides in elements); ``None`` -> ``None``."""
+    if t is None:
+        return None
+    if t.dim() > TG_MAX_DIMS:
+        raise ValueError(f"tensor rank {t.dim()} exceeds {TG_MAX_DIMS}")
+    code = _DTYPE_CODES.get(t.dtype)
+    if code is None:
+        raise TypeError(f"dtype {t.dtype} has no ABI code")
+    d = TgTensor()
+    d.ptr = t.data_ptr()
+    d.ndim = t.dim()
+    for i, (s, st) in enumerate(zip(t.shape, t.stride())):
+        d.shape[i] = s
+        d.strides[i] = st
+    d.dtype = code
+    return d
+
+
+def _ref(d: Optional[TgTensor]):
+    return None if d is None else ctypes.byref(d)
+
+
+def make_cfg(kernel_configs: Optional[dict]):
+    """``kernel_configs={...}`` (the reference's per-call override, src/tilegym/kernel_utils.py:14-36)
+    -> (int32 array, length).  Keys: KERNEL ('fallback'|'tiled'|'skinny' or 0/1/2), BLOCK_M, BLOCK_N,
+    SPLIT_K, ROW_GROUPS; unknown keys (e.g. num_ctas, occupancy) are ignored."""
+    arr = (ctypes.c_int32 * TG_CFG_COUNT)(*([-1] * TG_CFG_COUNT))
+    if kernel_configs:
+        for key, val in kernel_configs.items():
+            slot = CFG_SLOTS.get(str(key).upper())
+            if slot is None or val is None:
+                continue
+            if slot == 0 and isinstance(val, str):
+                val = {v: k for k, v in KERNEL_NAMES.items()}[val]
+            arr[slot] = int(val)
+    return arr, TG_CFG_COUNT
+
+
+def check_rc(rc: int, where: str) -> None:
+    if rc != 0:
+        detail = load().tg_last_error().decode("utf-8", "replace")
+        raise TileGymHipError(rc, where, detail)
+
+
+def last_config() -> Dict[str, int]:
+    """Schedule chosen by the most recent GEMM call on this thread."""
+    out = (ctypes.c_int32 * TG_CFG_COUNT)()
+    load().tg_last_config(out, TG_CFG_COUNT)
+    d = {name: int(out[slot]) for name, slot in CFG_SLOTS.items()}
+    d["KERNEL_NAME"] = KERNEL_NAMES.get(d["KERNEL"], "?")
+    return d
+
+
+# ---------------------------------------------------------------------------- workspaces
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def workspace_for(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    """Zero-initialised scratch buffer for the current stream of ``device`` (grown on demand).
+    One buffer per (device, stream): calls on one stream are ordered, so they can share it."""
+    if nbytes <= 0:
+        return None
+    stream = torch.cuda.current_stream(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(int(nbytes), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def workspace_bytes(M: int, N: int, K: int, trans_b: bool, cfg, ncfg) -> int:
+    return int(load().tg_fp8_gemm_workspace_bytes(M, N, K, 1 if trans_b else 0, cfg, ncfg))
+
+
+def _device_index(t: torch.Tensor) -> int:
+    if not t.is_cuda:
+        raise RuntimeError("tilegym_amd FP8 GEMM needs tensors on a HIP device (got a CPU tensor); "
+                           "there is no CPU implementation")
+    return t.device.index if t.device.index is not None else torch.cuda.current_device()
+
+
+def _stream_handle(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+# ---------------------------------------------------------------------------- raw calls
+def fp8_gemm(c, a, b, scale_a=None, scale_b=None, trans_a=False, trans_b=True, alpha=1.0, beta=0.0,
+             kernel_configs=None, use_workspace=True) -> None:
+    L = load()
+    dev = _device_index(a)
+    cfg, ncfg = make_cfg(kernel_configs)
+    M = a.shape[1] if trans_a else a.shape[0]
+    K = a.shape[0] if trans_a else a.shape[1]
+    N = b.shape[0] if trans_b else b.shape[1]
+    ws = None
+    if use_workspace and M > 0 and N > 0 and K > 0:
+        ws = workspace_for(a.device, workspace_bytes(M, N, K, trans_b, cfg, ncfg))
+    dc, da, db = make_tensor_desc(c), make_tensor_desc(a), make_tensor_desc(b)
+    dsa, dsb, dws = make_tensor_desc(scale_a), make_tensor_desc(scale_b), make_tensor_desc(ws)
+    rc = L.tg_fp8_gemm(_ref(dc), _ref(da), _ref(db), _ref(dsa), _ref(dsb), int(bool(trans_a)),
+                       int(bool(trans_b)), float(alpha), float(beta), _ref(dws), cfg, ncfg, dev,
+                       _stream_handle(a))
+    check_rc(rc, "tg_fp8_gemm")
+
+
+def fp8_ragged_gemm(c, a, b, a_scale, b_scale, m_indptr, kernel_configs=None) -> None:
+    L = load()
+    dev = _device_index(a)
+    cfg, ncfg = make_cfg(kernel_configs)
+    ds = [make_tensor_desc(t) for t in (c, a, b, a_scale, b_scale, m_indptr)]
+    rc = L.tg_fp8_ragged_gemm(*[_ref(d) for d in ds], cfg, ncfg, dev, _stream_handle(a))
+    check_rc(rc, "tg_fp8_ragged_gemm")
+
+
+def fp8_moe_gemm(c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids, expert_ids,
+                 num_tokens_post_padded, mul_routed_weight, top_k, block_m, kernel_configs=None) -> None:
+    L = load()
+    dev = _device_index(a)
+    cfg, ncfg = make_cfg(kernel_configs)
+    ds = [make_tensor_desc(t) for t in (c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids,
+                                        expert_ids, num_tokens_post_padded)]
+    rc = L.tg_fp8_moe_gemm(*[_ref(d) for d in ds], int(bool(mul_routed_weight)), int(top_k),
+                           int(block_m), cfg, ncfg, dev, _stream_handle(a))
+    check_rc(rc, "tg_fp8_moe_gemm")

@@ -1,0 +1,99 @@
+// Layout-agnostic FP8 GEMM fallback (any strides, any K, all row modes) and a byte transpose.
+// These are correctness paths for operand layouts the MFMA kernels do not take (K not a
+// multiple of 16, unaligned bases, transposed A); they decode e4m3 in software and use no
+// matrix instructions.
+#include "tg_host.h"
+
+namespace tg {
+
+__global__ void __launch_bounds__(256) fp8_gemm_generic_kernel(const GenericParams q) {
+    const GemmParams& p = q.g;
+    const int n = blockIdx.x * 64 + threadIdx.x;
+    const int r = blockIdx.y * 4 + threadIdx.y;
+    if (n >= p.N || r >= q.rows) return;
+    int arow = r, crow = r, e = 0;
+    if (q.group == GROUP_RAGGED) {
+        e = -1;
+        for (int i = 0; i < p.E; ++i)
+            if (r >= p.m_indptr[i] && r < p.m_indptr[i + 1]) { e = i; break; }
+        if (e < 0) return;
+    } else if (q.group == GROUP_GATHER) {
+        const int post = min(p.num_post_pad[0], p.em_capacity);
+        if (r >= post) return;
+        const int id = p.sorted_ids[r];
+        if (id < 0 || id >= p.num_valid) return;
+        arow = id / p.top_k;
+        crow = id;
+        e = p.expert_ids[r / p.block_m];
+        if (e < 0 || e >= p.E) return;
+    }
+    const uint8_t* a = p.A + (int64_t)arow * q.a_sm;
+    const uint8_t* b = p.B + (int64_t)e * q.b_se + (int64_t)n * q.b_sn;
+    float acc = 0.f;
+    for (int kb = 0; kb < p.kblocks; ++kb) {
+        const int k_hi = min((kb + 1) * kKBlock, p.K);
+        float part = 0.f;
+        for (int k = kb * kKBlock; k < k_hi; ++k)
+            part += e4m3_to_f32(a[(int64_t)k * q.a_sk]) * e4m3_to_f32(b[(int64_t)k * q.b_sk]);
+        float s = 1.0f;
+        if (q.block_scaled) {
+            if (p.As) s *= p.As[(int64_t)arow * p.kblocks + kb];
+            if (p.Bs) s *= p.Bs[((int64_t)e * p.nblocks + n / 128) * p.kblocks + kb];
+        }
+        acc += part * s;
+    }
+    float scale = p.alpha;
+    if (!q.block_scaled) {
+        if (p.As) scale *= p.As[0];
+        if (p.Bs) scale *= p.Bs[0];
+    }
+    if (q.group == GROUP_GATHER && p.row_weight) scale *= p.row_weight[crow];
+    float v = acc * scale;
+    const int64_t at = (int64_t)crow * p.N + n;
+    if (p.out_type == OUT_BF16) {
+        __bf16* c = reinterpret_cast<__bf16*>(p.C) + at;
+        if (p.beta != 0.f) v += p.beta * (float)(*c);
+        *c = (__bf16)v;
+    } else if (p.out_type == OUT_F32) {
+        float* c = reinterpret_cast<float*>(p.C) + at;
+        if (p.beta != 0.f) v += p.beta * (*c);
+        *c = v;
+    } else {
+        _Float16* c = reinterpret_cast<_Float16*>(p.C) + at;
+        if (p.beta != 0.f) v += p.beta * (float)(*c);
+        *c = (_Float16)v;
+    }
+}
+
+hipError_t run_generic(const GenericParams& q, hipStream_t s) {
+    if (q.rows <= 0 || q.g.N <= 0) return hipSuccess;
+    dim3 grid((q.g.N + 63) / 64, (q.rows + 3) / 4, 1);
+    hipLaunchKernelGGL(fp8_gemm_generic_kernel, grid, dim3(64, 4, 1), 0, s, q);
+    return hipGetLastError();
+}
+
+__global__ void __launch_bounds__(256) transpose_u8_kernel(const uint8_t* __restrict__ src,
+                                                           uint8_t* __restrict__ dst, int rows,
+                                                           int cols) {
+    __shared__ uint8_t t[64][65];
+    const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {
+        const int r = r0 + i, c = c0 + tx;
+        t[i][tx] = (r < rows && c < cols) ? src[(int64_t)r * cols + c] : 0;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const int c = c0 + i, r = r0 + tx;
+        if (c < cols && r < rows) dst[(int64_t)c * rows + r] = t[tx][i];
+    }
+}
+
+hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s) {
+    if (rows <= 0 || cols <= 0) return hipSuccess;
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64, 1);
+    hipLaunchKernelGGL(transpose_u8_kernel, grid, dim3(256, 1, 1), 0, s, src, dst, rows, cols);
+    return hipGetLastError();
+}
+
+}  // namespace tg

@@ -1,0 +1,473 @@
+// LDS-tiled FP8 GEMM for gfx950: C[m,n] = sum_k A[m,k] * B[n,k]  (both operands K-contiguous).
+//
+// One workgroup (4 or 8 waves) computes a BM x BN tile of C.  Per K step of 128 bytes it stages a
+// BM x 128 slab of A and a BN x 128 slab of B in LDS with direct global->LDS loads (16 bytes
+// per lane, no staging registers, double buffered), and every wave runs 16x16x128 e4m3 MFMAs
+// over its (BM/WGM) x (BN/WGN) sub-tile with fp32 accumulators.  A direct load writes lane l
+// of a wave to LDS byte 16*l of the wave's 1 KiB destination, so the XOR swizzle that keeps
+// the fragment reads bank-conflict free is applied on the global side: each lane fetches the
+// 16-byte chunk that belongs at its LDS position.  The two stages are separate LDS objects so
+// that the compiler can tell a load into one from a read of the other.
+//
+// The MFMA "row" operand is fed from B (weights) and the "column" operand from A
+// (activations): a lane then owns, for one activation row m, four consecutive n, so a
+// per-token scale is one register per lane.
+//
+// Epilogue: each wave passes its accumulators through the (now idle) LDS in 64-column slices
+// and writes C with one 16-byte store per lane, rows contiguous; scaling, beta, routed weights
+// and the output cast happen in that short rolled loop.
+//
+// Scale modes:  per-tensor (one multiply in the epilogue) or block-scaled (every K step's
+// 16x16 product is multiplied by As[m,kb] * Bs[n/128,kb] while it is added to the
+// accumulator, the arithmetic of src/tilegym/suites/unsloth/cutile/fp8.py:282-323).
+// Row modes: dense, ragged (expert segments from m_indptr, the schedule of
+// src/tilegym/suites/flashinfer/cutile/gemm/ragged_block_scaled_bmm.py:71-91) and gather
+// (sorted_token_ids / expert_ids, the contract of src/tilegym/ops/tilecpp/moe.cuh:72-225).
+#pragma once
+#include "tg_device.h"
+
+namespace tg {
+
+#if defined(__HIP_DEVICE_COMPILE__)
+// Raw buffer descriptor over [base, base + 2 GiB): byte offsets, no format conversion.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), (short)0, 0x7FFFFFFF, 0x00020000);
+}
+#endif
+
+__device__ __forceinline__ int swz16(int r) { return ((r & 7) + ((r >> 3) & 1)) & 7; }
+
+// Number of BM-row tiles over all experts (every lane returns the same value).
+__device__ __forceinline__ int ragged_count_tiles(const int* indptr, int E, int BM, int lane) {
+    int total = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+        int e = e0 + lane, cnt = 0;
+        if (e < E) {
+            int rows = indptr[e + 1] - indptr[e];
+            cnt = rows > 0 ? (rows + BM - 1) / BM : 0;
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) cnt += __shfl_xor(cnt, d);
+        total += cnt;
+    }
+    return total;
+}
+
+// Expert that owns m-tile `mt`, and the index of that tile inside the expert.
+__device__ __forceinline__ void ragged_find(const int* indptr, int E, int BM, int lane, int mt,
+                                            int& expert, int& tile_in_expert) {
+    int base = 0;
+    expert = -1;
+    tile_in_expert = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+        int e = e0 + lane, cnt = 0;
+        if (e < E) {
+            int rows = indptr[e + 1] - indptr[e];
+            cnt = rows > 0 ? (rows + BM - 1) / BM : 0;
+        }
+        int incl = cnt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int t = __shfl_up(incl, d);
+            if (lane >= d) incl += t;
+        }
+        int excl = base + incl - cnt;
+        unsigned long long hit = __ballot(mt >= excl && mt < excl + cnt);
+        if (hit) {
+            int src = __ffsll((long long)hit) - 1;
+            expert = e0 + src;
+            tile_in_expert = mt - __shfl(excl, src);
+            return;
+        }
+        base += __shfl(incl, 63);
+    }
+}
+
+// Write 8 consecutive outputs C[row][col..col+7] = v (+ beta * old), masked against N.
+__device__ __forceinline__ void store8(void* C, int out_type, int64_t row, int col, int N,
+                                       v4f lo, v4f hi, float beta, bool vec_ok) {
+    const int64_t base = row * (int64_t)N + col;
+    if (vec_ok && col + 7 < N) {
+        if (out_type == OUT_F32) {
+            v4f* p = reinterpret_cast<v4f*>(reinterpret_cast<float*>(C) + base);
+            if (beta != 0.0f) {
+                lo += beta * p[0];
+                hi += beta * p[1];
+            }
+            p[0] = lo;
+            p[1] = hi;
+        } else if (out_type == OUT_BF16) {
+            typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+            typedef float v8f __attribute__((ext_vector_type(8)));
+            bf16x8* p = reinterpret_cast<bf16x8*>(reinterpret_cast<__bf16*>(C) + base);
+            v8f v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            if (beta != 0.0f) v += beta * __builtin_convertvector(*p, v8f);
+            *p = __builtin_convertvector(v, bf16x8);
+        } else {
+            typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+            typedef float v8f __attribute__((ext_vector_type(8)));
+            f16x8* p = reinterpret_cast<f16x8*>(reinterpret_cast<_Float16*>(C) + base);
+            v8f v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            if (beta != 0.0f) v += beta * __builtin_convertvector(*p, v8f);
+            *p = __builtin_convertvector(v, f16x8);
+        }
+        return;
+    }
+    for (int q = 0; q < 8; ++q) {
+        if (col + q >= N) break;
+        float x = q < 4 ? lo[q & 3] : hi[q & 3];
+        if (out_type == OUT_BF16) {
+            __bf16* p = reinterpret_cast<__bf16*>(C) + base + q;
+            if (beta != 0.0f) x += beta * (float)(*p);
+            *p = (__bf16)x;
+        } else if (out_type == OUT_F32) {
+            float* p = reinterpret_cast<float*>(C) + base + q;
+            if (beta != 0.0f) x += beta * (*p);
+            *p = x;
+        } else {
+            _Float16* p = reinterpret_cast<_Float16*>(C) + base + q;
+            if (beta != 0.0f) x += beta * (float)(*p);
+            *p = (_Float16)x;
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>
+__global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_gemm_tile_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only types; the host pass only needs the stub
+    constexpr int NT = 64 * WGM * WGN;
+    constexpr int NW = WGM * WGN;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 16, TN = WTN / 16;
+    constexpr int RPP = 8 * NW;  // slab rows filled per pass of the whole workgroup
+    constexpr int A_IT = BM / RPP, B_IT = BN / RPP;
+    // epilogue slices: PCOLS columns of the wave tile at a time, fp32, through one LDS object
+    constexpr int OBJ = (BM < BN ? BM : BN) * kKBlock;  // bytes of the smaller stage object
+    constexpr int PC0 = WTN < 64 ? WTN : 64;
+    constexpr int PCOLS = (WTM * PC0 * 4 * (NW / 4) <= OBJ) ? PC0 : PC0 / 2;
+    constexpr int TNG = PCOLS / 16, PASSES = TN / TNG;
+    constexpr int UNITS = PCOLS / 4;  // 16-byte units per staged row
+    static_assert(NW == 4 || NW == 8, "epilogue staging: NW/4 waves share one LDS object");
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "loader shape");
+    static_assert(WTM % 16 == 0 && WTN % 16 == 0 && TN % TNG == 0, "wave tile");
+    static_assert(WTM * PCOLS * 4 * (NW / 4) <= OBJ && PCOLS >= 16, "epilogue slice fits");
+    static_assert(!BLOCKSCALE || (WTN <= 128 && 128 % WTN == 0), "one weight scale per wave");
+    static_assert(!SPLIT || GROUP == GROUP_DENSE, "split-K is dense only");
+
+    __shared__ __align__(1024) uint8_t sA0[BM * kKBlock];
+    __shared__ __align__(1024) uint8_t sA1[BM * kKBlock];
+    __shared__ __align__(1024) uint8_t sB0[BN * kKBlock];
+    __shared__ __align__(1024) uint8_t sB1[BN * kKBlock];
+    __shared__ int s_src[GROUP == GROUP_DENSE ? 1 : BM];
+    __shared__ int s_dst[GROUP == GROUP_DENSE ? 1 : BM];
+    __shared__ int s_flag;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int tiles_n = (p.N + BN - 1) / BN;
+    const int K = p.K;
+
+    // ---------------------------------------------------------------- which tile
+    int tile_m = 0, tile_n = 0, m0 = 0, rows_valid = BM;
+    const uint8_t* Bbase = p.B;
+    const float* Bsbase = p.Bs;
+    int post_pad = 0;
+    if constexpr (GROUP == GROUP_DENSE) {
+        const int tiles_m = (p.M + BM - 1) / BM;
+        const int pid = xcd_remap(blockIdx.x, tiles_m * tiles_n);
+        constexpr int GM = 8;
+        const int width = GM * tiles_n;
+        const int group = pid / width, first_m = group * GM;
+        const int gsz = min(tiles_m - first_m, GM);
+        tile_m = first_m + (pid % width) % gsz;
+        tile_n = (pid % width) / gsz;
+        m0 = tile_m * BM;
+        rows_valid = min(BM, p.M - m0);
+    } else if constexpr (GROUP == GROUP_RAGGED) {
+        const int total_mt = ragged_count_tiles(p.m_indptr, p.E, BM, lane);
+        const int nblk = total_mt * tiles_n;
+        if ((int)blockIdx.x >= nblk) return;
+        const int pid = xcd_remap(blockIdx.x, nblk);
+        tile_m = pid / tiles_n;
+        tile_n = pid % tiles_n;
+        int e, t_in_e;
+        ragged_find(p.m_indptr, p.E, BM, lane, tile_m, e, t_in_e);
+        e = __builtin_amdgcn_readfirstlane(e);
+        t_in_e = __builtin_amdgcn_readfirstlane(t_in_e);
+        if (e < 0) return;
+        const int lo = p.m_indptr[e], hi = min(p.m_indptr[e + 1], p.M);
+        m0 = lo + t_in_e * BM;
+        rows_valid = min(BM, hi - m0);
+        if (rows_valid <= 0 || lo < 0) return;
+        Bbase += (int64_t)e * p.N * K;
+        if (Bsbase) Bsbase += (int64_t)e * p.nblocks * p.kblocks;
+    } else {
+        post_pad = min(p.num_post_pad[0], p.em_capacity);
+        const int total_mt = (post_pad + BM - 1) / BM;
+        const int nblk = total_mt * tiles_n;
+        if ((int)blockIdx.x >= nblk) return;
+        const int pid = xcd_remap(blockIdx.x, nblk);
+        tile_m = pid / tiles_n;
+        tile_n = pid % tiles_n;
+        m0 = tile_m * BM;  // position in the sorted slot sequence
+        const int e = p.expert_ids[m0 / p.block_m];
+        if (e < 0 || e >= p.E) return;
+        Bbase += (int64_t)e * p.N * K;
+        if (Bsbase) Bsbase += (int64_t)e * p.nblocks * p.kblocks;
+    }
+    const int n0 = tile_n * BN;
+
+    if constexpr (GROUP != GROUP_DENSE) {
+        for (int r = tid; r < BM; r += NT) {
+            int src, dst;
+            if constexpr (GROUP == GROUP_RAGGED) {
+                src = m0 + min(r, rows_valid - 1);
+                dst = r < rows_valid ? m0 + r : -1;
+            } else {
+                const int idx = m0 + r;
+                const int id = idx < post_pad ? p.sorted_ids[idx] : p.num_valid;
+                const bool ok = id >= 0 && id < p.num_valid;
+                src = ok ? id / p.top_k : 0;
+                dst = ok ? id : -1;
+            }
+            s_src[r] = src;
+            s_dst[r] = dst;
+        }
+        __syncthreads();
+    }
+
+    // ---------------------------------------------------------------- loader set-up
+    // Pass i of wave w fills the 8-row group g = i*NW + w: lane l lands at row 8g + l/8, chunk
+    // position l%8, and therefore fetches logical chunk (l%8) ^ swz16(row%16).  NW is even, so
+    // row%16 = 8*(w&1) + l/8 for every pass.
+    const int lrow = lane >> 3;
+    const int lj = (lane & 7) ^ swz16(((wave & 1) << 3) + lrow);
+    uint32_t a_off[A_IT], b_off[B_IT];
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+        const int r = (i * NW + wave) * 8 + lrow;
+        int src;
+        if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
+        else src = s_src[r];
+        a_off[i] = (uint32_t)src * (uint32_t)K + lj * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) {
+        const int n = min(n0 + (i * NW + wave) * 8 + lrow, p.N - 1);
+        b_off[i] = (uint32_t)n * (uint32_t)K + lj * 16;
+    }
+
+    const int li = lane & 15, lg = lane >> 4;
+    const uint32_t frag0 = li * kKBlock + ((lg ^ swz16(li)) << 4);
+    const uint32_t frag1 = frag0 ^ 64;
+    const uint32_t a_frag_base = wm * WTM * kKBlock, b_frag_base = wn * WTN * kKBlock;
+
+    // block scales: one activation scale per (lane, tm), one weight scale per wave
+    int srow[TM];
+    const float* bs_ptr = nullptr;
+    if constexpr (BLOCKSCALE) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const int r = wm * WTM + tm * 16 + li;
+            if constexpr (GROUP == GROUP_DENSE) srow[tm] = m0 + min(r, rows_valid - 1);
+            else srow[tm] = s_src[r];
+        }
+        const int nb = min((n0 + wn * WTN) / 128, p.nblocks - 1);
+        if (Bsbase) bs_ptr = Bsbase + (int64_t)nb * p.kblocks;
+    }
+
+    int ks = 0, ks_end = p.kblocks;
+    if constexpr (SPLIT) {
+        ks = blockIdx.y * p.ksteps_per_split;
+        ks_end = min(ks + p.ksteps_per_split, p.kblocks);
+    }
+
+    v4f acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    float sc_next[TM];
+
+    // Direct global->LDS load of one K step into (dA, dB), as buffer loads: 32-bit per-lane
+    // offset + scalar K offset, no 64-bit address arithmetic in the loop.  K is a multiple of
+    // 128 here (the host sends other K to the fallback kernel), so every lane's 16 bytes are
+    // in range.
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(Bbase);
+    auto issue_loads = [&](int kstep, uint8_t* dA, uint8_t* dB) {
+        const int k0 = kstep * kKBlock;
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rsrc_a, (__attribute__((address_space(3))) void*)(dA + (i * NW + wave) * 1024), 16,
+                a_off[i], k0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rsrc_b, (__attribute__((address_space(3))) void*)(dB + (i * NW + wave) * 1024), 16,
+                b_off[i], k0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto load_scales = [&](int kstep) {
+        if constexpr (BLOCKSCALE) {
+            const float bs = bs_ptr ? bs_ptr[kstep] : 1.0f;
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                const float as = p.As ? p.As[(int64_t)srow[tm] * p.kblocks + kstep] : 1.0f;
+                sc_next[tm] = as * bs;
+            }
+        }
+    };
+    auto compute = [&](const uint8_t* cA, const uint8_t* cB, const float* sc) {
+        v8i af[TM];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const uint8_t* base = cA + a_frag_base + tm * 16 * kKBlock;
+            af[tm] = join(*reinterpret_cast<const v4i*>(base + frag0),
+                          *reinterpret_cast<const v4i*>(base + frag1));
+        }
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
+            const v8i wf = join(*reinterpret_cast<const v4i*>(base + frag0),
+                                *reinterpret_cast<const v4i*>(base + frag1));
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                if constexpr (BLOCKSCALE) {
+                    const v4f part = mfma_e4m3(wf, af[tm], v4f{0.f, 0.f, 0.f, 0.f});
+                    acc[tn][tm] += part * sc[tm];
+                } else {
+                    acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
+                }
+            }
+        }
+    };
+    // All of this wave's direct loads have landed in LDS; then every wave's have.
+    auto stage_ready = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+        __syncthreads();
+    };
+
+    // ---------------------------------------------------------------- main loop
+    // Two K steps per trip (stage 0 then stage 1); an odd last step is peeled.
+    float sc_cur[TM];
+    const int nsteps = ks_end - ks;
+    issue_loads(ks, sA0, sB0);
+    load_scales(ks);
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = BLOCKSCALE ? sc_next[tm] : 1.0f;
+    stage_ready();
+    int i = 0;
+    for (; i + 1 < nsteps; i += 2) {
+        issue_loads(ks + i + 1, sA1, sB1);
+        load_scales(ks + i + 1);
+        compute(sA0, sB0, sc_cur);
+        if constexpr (BLOCKSCALE) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = sc_next[tm];
+        }
+        stage_ready();
+        if (i + 2 < nsteps) {
+            issue_loads(ks + i + 2, sA0, sB0);
+            load_scales(ks + i + 2);
+        }
+        compute(sA1, sB1, sc_cur);
+        if constexpr (BLOCKSCALE) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = sc_next[tm];
+        }
+        stage_ready();
+    }
+    if (i < nsteps) {
+        compute(sA0, sB0, sc_cur);
+        __syncthreads();
+    }
+
+    // ---------------------------------------------------------------- epilogue
+    // Every wave is past the last barrier, so the stage buffers are free: wave w stages through
+    // the w-th of them.  A staged row holds PCOLS fp32; 16-byte unit u of row r sits at unit
+    // position u ^ (r % UNITS) so that both the accumulator writes (16 lanes = 16 rows, same
+    // unit) and the row-wise reads spread over the banks.
+    float scale = p.alpha;
+    if constexpr (!BLOCKSCALE) {
+        if (p.As) scale *= p.As[0];
+        if (p.Bs) scale *= p.Bs[0];
+    }
+    const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;  // 8-wide rows stay 16-byte aligned
+    uint8_t* stage_buf = (wave & 3) == 0 ? sA0 : (wave & 3) == 1 ? sA1 : (wave & 3) == 2 ? sB0 : sB1;
+    stage_buf += (wave >> 2) * (WTM * PCOLS * 4);
+    const int64_t MN = (int64_t)p.M * p.N;
+
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+#pragma unroll
+        for (int t = 0; t < TNG; ++t)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                const int r = tm * 16 + li;
+                const int u = (t * 4 + lg) ^ (r & (UNITS - 1));
+                *reinterpret_cast<v4f*>(stage_buf + r * (PCOLS * 4) + u * 16) = acc[ps * TNG + t][tm];
+            }
+        // rolled: 8 columns per lane, PCOLS/8 lanes per row
+        constexpr int LPR = PCOLS / 8, RPI = 64 / LPR;
+        const int rr = lane / LPR, c8 = (lane % LPR) * 8;
+        const int col = n0 + wn * WTN + ps * PCOLS + c8;
+        for (int it = 0; it < WTM / RPI; ++it) {
+            const int r = it * RPI + rr;
+            const int rt = wm * WTM + r;  // row inside the workgroup tile
+            const int u0 = (c8 >> 2) ^ (r & (UNITS - 1)), u1 = ((c8 >> 2) + 1) ^ (r & (UNITS - 1));
+            v4f lo = *reinterpret_cast<const v4f*>(stage_buf + r * (PCOLS * 4) + u0 * 16);
+            v4f hi = *reinterpret_cast<const v4f*>(stage_buf + r * (PCOLS * 4) + u1 * 16);
+            int dst;
+            if constexpr (GROUP == GROUP_DENSE) dst = rt < rows_valid ? m0 + rt : -1;
+            else dst = s_dst[rt];
+            if (dst < 0 || col >= p.N) continue;
+            if constexpr (SPLIT) {
+                store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, dst, col, p.N, lo, hi, 0.f, vec_ok);
+            } else {
+                float rs = scale;
+                if constexpr (GROUP == GROUP_GATHER) {
+                    if (p.row_weight) rs *= p.row_weight[dst];
+                }
+                store8(p.C, p.out_type, dst, col, p.N, lo * rs, hi * rs, p.beta, vec_ok);
+            }
+        }
+    }
+
+    if constexpr (SPLIT) {
+        if (!splitk_arrive(p.counters, tile_m * tiles_n + tile_n, p.split_k, &s_flag)) return;
+        // last workgroup for this tile: add the partial tiles in a fixed order
+        for (int idx = tid; idx < BM * (BN / 8); idx += NT) {
+            const int r = idx / (BN / 8), col = n0 + (idx % (BN / 8)) * 8;
+            if (r >= rows_valid || col >= p.N) continue;
+            const int64_t at = (int64_t)(m0 + r) * p.N + col;
+            v4f lo = v4f{0.f, 0.f, 0.f, 0.f}, hi = lo;
+            for (int z = 0; z < p.split_k; ++z) {
+                const float* src = p.partials + z * MN + at;
+                if (vec_ok && col + 7 < p.N) {
+                    lo += reinterpret_cast<const v4f*>(src)[0];
+                    hi += reinterpret_cast<const v4f*>(src)[1];
+                } else {
+                    for (int q = 0; q < 8 && col + q < p.N; ++q) {
+                        if (q < 4) lo[q & 3] += src[q];
+                        else hi[q & 3] += src[q];
+                    }
+                }
+            }
+            store8(p.C, p.out_type, m0 + r, col, p.N, lo * scale, hi * scale, p.beta, vec_ok);
+        }
+    }
+#endif
+}
+
+template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>
+inline hipError_t launch_tile(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
+    auto kern = fp8_gemm_tile_kernel<BM, BN, WGM, WGN, BLOCKSCALE, GROUP, SPLIT>;
+    hipLaunchKernelGGL(kern, dim3(grid_x, grid_y, 1), dim3(64 * WGM * WGN, 1, 1), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace tg

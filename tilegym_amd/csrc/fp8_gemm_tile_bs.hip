@@ -1,0 +1,20 @@
+// Instantiations of the LDS-tiled kernel: block scales (1x128 activations, 128x128 weights), dense rows.
+#include "fp8_gemm_tile.h"
+#include "tg_host.h"
+
+namespace tg {
+
+hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s) {
+#define TG_CASE(BM, BN, WGM, WGN)                                                               \
+    if (bm == BM && bn == BN) {                                                                  \
+        return split ? launch_tile<BM, BN, WGM, WGN, true, GROUP_DENSE, true>(p, gx, gy, s)      \
+                     : launch_tile<BM, BN, WGM, WGN, true, GROUP_DENSE, false>(p, gx, gy, s);    \
+    }
+    TG_CASE(128, 128, 2, 2)
+    TG_CASE(128, 256, 2, 4)
+    TG_CASE(64, 128, 1, 4)
+#undef TG_CASE
+    return hipErrorInvalidConfiguration;
+}
+
+}  // namespace tg

@@ -1,0 +1,150 @@
+// Device-side building blocks shared by the FP8 GEMM kernels (gfx950 / CDNA4 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+namespace tg {
+
+constexpr int kKBlock = 128;    // bytes of K consumed by one 16x16x128 MFMA = the quant block
+constexpr int kCounterSlots = 16384;  // ints at the start of a workspace (split-K arrival counters)
+
+enum OutType { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2 };  // same numbering as the ABI dtype codes
+
+// How rows of the activation operand are found.
+enum GroupMode { GROUP_DENSE = 0, GROUP_RAGGED = 1, GROUP_GATHER = 2 };
+
+struct GemmParams {
+    const uint8_t* A;   // activations, (M,K) row-major, e4m3
+    const uint8_t* B;   // weights, (N,K) row-major (or (E,N,K)), e4m3
+    void* C;            // (M,N) row-major
+    const float* As;    // per-tensor: 1 float or null.  block: (M, kblocks)
+    const float* Bs;    // per-tensor: 1 float or null.  block: ([E,] nblocks, kblocks)
+    int M, N, K;
+    int kblocks, nblocks;  // ceil(K/128), ceil(N/128)
+    float alpha, beta;
+    int out_type;
+    int vec_store;      // 1 when N % 4 == 0 and C is 16-byte aligned: 4-wide stores allowed
+    // split-K
+    int split_k;        // >= 1
+    int ksteps_per_split;
+    float* partials;    // [split_k][M][N] fp32
+    int* counters;      // one per output tile, zero on entry, zero on exit
+    // grouped forms
+    const int* m_indptr;   // ragged: (E+1)
+    int E;
+    const int* sorted_ids; // gather: (EM)
+    const int* expert_ids; // gather: (EM / block_m)
+    const int* num_post_pad;  // gather: (1)
+    const float* row_weight;  // gather: (num_valid) or null
+    int top_k, num_valid, block_m, em_capacity;
+};
+
+// One 16x16x128 e4m3 x e4m3 MFMA with fp32 accumulation.  `w` supplies the 16 rows of the
+// result (lane l: row l%16, K bytes of K-group l/16), `x` supplies the 16 columns; lane l
+// receives column l%16, rows 4*(l/16)..+3.  With both scale operands zero the compiler
+// selects the unscaled instruction.
+__device__ __forceinline__ v4f mfma_e4m3(v8i w, v8i x, v4f acc) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, x, acc, 0, 0, 0, 0, 0, 0);
+}
+
+__device__ __forceinline__ v8i join(v4i lo, v4i hi) {
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Exact software decode of one e4m3fn code (used only by the generic fallback kernel).
+__device__ __forceinline__ float e4m3_to_f32(uint8_t c) {
+    uint32_t s = (uint32_t)(c & 0x80) << 24;
+    uint32_t e = (c >> 3) & 0xF, m = c & 7;
+    if (e == 0xF && m == 7) return __uint_as_float(s | 0x7FC00000u);
+    if (e == 0) {
+        float v = (float)m * 0.001953125f;  // m * 2^-9
+        return __uint_as_float(__float_as_uint(v) | s);
+    }
+    return __uint_as_float(s | ((e + 120u) << 23) | (m << 20));
+}
+
+// Store 4 consecutive outputs C[row][col..col+3] = v (+ beta * old), masked against ncols.
+__device__ __forceinline__ void store4(void* C, int out_type, int64_t row, int col, int N, v4f v,
+                                       float beta, bool vec_ok) {
+    int64_t base = row * (int64_t)N + col;
+    if (vec_ok && col + 3 < N) {
+        if (out_type == OUT_BF16) {
+            bf16x4* p = reinterpret_cast<bf16x4*>(reinterpret_cast<__bf16*>(C) + base);
+            if (beta != 0.0f) {
+                bf16x4 o = *p;
+                v4f of = __builtin_convertvector(o, v4f);
+                v = v + beta * of;
+            }
+            *p = __builtin_convertvector(v, bf16x4);
+        } else if (out_type == OUT_F32) {
+            v4f* p = reinterpret_cast<v4f*>(reinterpret_cast<float*>(C) + base);
+            if (beta != 0.0f) v = v + beta * (*p);
+            *p = v;
+        } else {
+            f16x4* p = reinterpret_cast<f16x4*>(reinterpret_cast<_Float16*>(C) + base);
+            if (beta != 0.0f) {
+                f16x4 o = *p;
+                v4f of = __builtin_convertvector(o, v4f);
+                v = v + beta * of;
+            }
+            *p = __builtin_convertvector(v, f16x4);
+        }
+        return;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (col + r >= N) break;
+        float x = v[r];
+        if (out_type == OUT_BF16) {
+            __bf16* p = reinterpret_cast<__bf16*>(C) + base + r;
+            if (beta != 0.0f) x += beta * (float)(*p);
+            *p = (__bf16)x;
+        } else if (out_type == OUT_F32) {
+            float* p = reinterpret_cast<float*>(C) + base + r;
+            if (beta != 0.0f) x += beta * (*p);
+            *p = x;
+        } else {
+            _Float16* p = reinterpret_cast<_Float16*>(C) + base + r;
+            if (beta != 0.0f) x += beta * (float)(*p);
+            *p = (_Float16)x;
+        }
+    }
+}
+
+// Split-K arrival: every workgroup that worked on `tile` calls this after writing its partial
+// sums.  Returns true in exactly one workgroup -- the last to arrive -- which then owns the
+// reduction.  The counter is returned to zero by that workgroup.
+__device__ __forceinline__ bool splitk_arrive(int* counters, int tile, int split_k, int* s_flag) {
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int old = __hip_atomic_fetch_add(&counters[tile], 1, __ATOMIC_ACQ_REL,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+        int last = (old == split_k - 1);
+        if (last)
+            __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_flag = last;
+    }
+    __syncthreads();
+    bool last = (*s_flag != 0);
+    if (last) __threadfence();
+    return last;
+}
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  Re-number them so that each
+// XCD (own L2) works on a contiguous range of the tile sequence.
+__device__ __forceinline__ int xcd_remap(int pid, int nblk) {
+    constexpr int X = 8;
+    int q = nblk / X, r = nblk % X;
+    int x = pid % X, idx = pid / X;
+    return x * q + (x < r ? x : r) + idx;
+}
+
+}  // namespace tg

@@ -1,0 +1,30 @@
+// Host-side declarations shared by the C-ABI translation unit and the kernel instantiation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "tg_device.h"
+
+namespace tg {
+
+// Arguments of the layout-agnostic fallback kernel: any strides, any K.
+struct GenericParams {
+    GemmParams g;            // pointers, sizes, scales, grouping (A/B strides below override NT)
+    int64_t a_sm, a_sk;      // element strides of A along m and k
+    int64_t b_sn, b_sk;      // element strides of B along n and k
+    int64_t b_se;            // element stride between experts
+    int group;               // GroupMode
+    int block_scaled;        // 0 per-tensor, 1 block
+    int rows;                // row slots to visit (M, or the sorted-slot capacity in gather mode)
+};
+
+struct TileShape { int bm, bn; };
+
+// Launchers return hipErrorInvalidConfiguration when the combination is not instantiated.
+hipError_t run_tile_per_tensor(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
+hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
+hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p, int gx, hipStream_t s);
+hipError_t run_skinny(int mt, int rg, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
+hipError_t run_generic(const GenericParams& p, hipStream_t s);
+// dst (cols, rows) <- transpose of src (rows, cols), one byte per element
+hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s);
+
+}  // namespace tg

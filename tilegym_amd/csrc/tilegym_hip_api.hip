@@ -1,0 +1,556 @@
+// C ABI of libtilegym_hip.so (declared in include/tilegym_hip.h): argument validation on the
+// host, schedule selection, kernel launches.  No allocation, no synchronisation, no global
+// mutable state apart from two thread-local diagnostics (last error text, last schedule).
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/tilegym_hip.h"
+#include "tg_host.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+thread_local int32_t g_last_cfg[TG_CFG_COUNT] = {-1, -1, -1, -1, -1, -1, -1, -1};
+
+int32_t fail(int32_t rc, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return rc;
+}
+
+int64_t numel(const tg_tensor* t) {
+    int64_t n = 1;
+    for (int i = 0; i < t->ndim; ++i) n *= t->shape[i];
+    return n;
+}
+
+bool contiguous(const tg_tensor* t) {
+    int64_t expect = 1;
+    for (int i = t->ndim - 1; i >= 0; --i) {
+        if (t->shape[i] != 1 && t->strides[i] != expect) return false;
+        expect *= t->shape[i];
+    }
+    return true;
+}
+
+int32_t check_tensor(const tg_tensor* t, const char* name, int ndim) {
+    if (!t) return fail(TG_ERR_NULL, "%s: null tensor descriptor", name);
+    if (t->ndim < 0 || t->ndim > TG_MAX_DIMS) return fail(TG_ERR_INVALID, "%s: ndim %d out of range", name, t->ndim);
+    if (ndim >= 0 && t->ndim != ndim) return fail(TG_ERR_INVALID, "%s: expected %d dims, got %d", name, ndim, t->ndim);
+    for (int i = 0; i < t->ndim; ++i)
+        if (t->shape[i] < 0) return fail(TG_ERR_INVALID, "%s: negative extent", name);
+    if (!contiguous(t)) return fail(TG_ERR_INVALID, "%s: must be contiguous", name);
+    if (numel(t) > 0 && t->ptr == 0) return fail(TG_ERR_NULL, "%s: null data pointer", name);
+    return TG_OK;
+}
+
+int32_t out_type_of(int32_t dtype) {
+    switch (dtype) {
+        case TG_F32: return tg::OUT_F32;
+        case TG_F16: return tg::OUT_F16;
+        case TG_BF16: return tg::OUT_BF16;
+        default: return -1;
+    }
+}
+
+int64_t elem_size(int32_t dtype) {
+    switch (dtype) {
+        case TG_F32: case TG_I32: return 4;
+        case TG_F16: case TG_BF16: return 2;
+        case TG_I64: return 8;
+        default: return 1;
+    }
+}
+
+inline int cfg_get(const int32_t* cfg, int32_t ncfg, int slot) {
+    return (cfg && slot < ncfg) ? cfg[slot] : -1;
+}
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
+
+constexpr int64_t kCounterBytes = (int64_t)tg::kCounterSlots * 4;
+constexpr int64_t kOffsetLimit = (int64_t)1 << 31;  // kernels index operands with 32-bit byte offsets
+constexpr int kTargetWorkgroups = 1024;             // 4 per CU on 256 CUs
+
+// Switches to the caller's device for the lifetime of a call.
+struct DeviceGuard {
+    int prev = -1;
+    bool ok = false, switched = false;
+    explicit DeviceGuard(int dev) {
+        int count = 0;
+        if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) { (void)hipGetLastError(); return; }
+        if (dev < 0 || dev >= count) return;
+        if (hipGetDevice(&prev) != hipSuccess) return;
+        if (prev != dev) {
+            if (hipSetDevice(dev) != hipSuccess) return;
+            switched = true;
+        }
+        ok = true;
+    }
+    ~DeviceGuard() {
+        if (switched) (void)hipSetDevice(prev);
+    }
+};
+
+struct Schedule {
+    int kernel;  // 0 fallback, 1 tiled, 2 skinny
+    int bm, bn, split_k, row_groups, mt;
+};
+
+void remember(const Schedule& s) {
+    for (int i = 0; i < TG_CFG_COUNT; ++i) g_last_cfg[i] = -1;
+    g_last_cfg[TG_CFG_KERNEL] = s.kernel;
+    g_last_cfg[TG_CFG_BLOCK_M] = s.bm;
+    g_last_cfg[TG_CFG_BLOCK_N] = s.bn;
+    g_last_cfg[TG_CFG_SPLIT_K] = s.split_k;
+    g_last_cfg[TG_CFG_ROW_GROUPS] = s.row_groups;
+}
+
+bool tile_exists(int bm, int bn, bool block_scaled) {
+    if (bm == 128 && bn == 128) return true;
+    if (bm == 128 && bn == 256) return true;
+    if (bm == 64 && bn == 128) return true;
+    if (bm == 256 && bn == 256) return !block_scaled;
+    return false;
+}
+
+// Split-K factor: enough workgroups to fill the chip, at least `min_steps` K steps per split,
+// partial sums must fit the workspace.
+int pick_split(int64_t workgroups, int64_t kblocks, int min_steps, int64_t M, int64_t N,
+               int64_t partial_bytes_avail, int want) {
+    int64_t split = want > 0 ? want : cdiv(kTargetWorkgroups, workgroups > 0 ? workgroups : 1);
+    if (want <= 0) split = split > 16 ? 16 : split;
+    const int64_t by_k = kblocks / min_steps > 0 ? kblocks / min_steps : 1;
+    if (split > by_k) split = by_k;
+    const int64_t per = M * N * 4;
+    if (per > 0 && split > 1 && split * per > partial_bytes_avail) split = partial_bytes_avail / per;
+    if (split < 1) split = 1;
+    // every split must own at least one K step
+    const int64_t kps = cdiv(kblocks, split);
+    split = cdiv(kblocks, kps);
+    return (int)split;
+}
+
+Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
+                      const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
+    Schedule s{0, -1, -1, 1, -1, -1};
+    const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
+    const int64_t kblocks = cdiv(K, 128);
+    if (!fast_layout || want_kernel == 0 || K == 0) return s;
+    const bool tile_ok = (K % 128) == 0;
+    bool skinny = M <= 64;
+    if (want_kernel == 1 && tile_ok) skinny = false;
+    if (want_kernel == 2 && M <= 64) skinny = true;
+    if (!skinny && !tile_ok) return s;
+    const int want_split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
+    if (skinny) {
+        s.kernel = 2;
+        s.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+        int rg = cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS);
+        if (rg != 1 && rg != 2 && rg != 4) {
+            rg = 1;
+            if (cdiv(N, 32) >= 768) rg = 2;
+            if (cdiv(N, 64) >= 1024 && s.mt <= 2) rg = 4;
+        }
+        s.row_groups = rg;
+        const int64_t wgs = cdiv(N, 16 * rg);
+        s.split_k = wgs > tg::kCounterSlots ? 1 : pick_split(wgs, kblocks, 8, M, N, partial_bytes_avail, want_split);
+        return s;
+    }
+    s.kernel = 1;
+    int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
+    if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, block_scaled))) {
+        auto tiles = [&](int64_t a, int64_t b) { return cdiv(M, a) * cdiv(N, b); };
+        if (!block_scaled && tiles(256, 256) >= 200) { bm = 256; bn = 256; }
+        else if (tiles(128, 256) >= 200) { bm = 128; bn = 256; }
+        else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
+        else { bm = 64; bn = 128; }
+    }
+    s.bm = bm;
+    s.bn = bn;
+    const int64_t wgs = cdiv(M, bm) * cdiv(N, bn);
+    s.split_k = 1;
+    if (wgs <= tg::kCounterSlots && (want_split > 1 || (want_split < 0 && wgs < 192)))
+        s.split_k = pick_split(wgs * 4, kblocks, 8, M, N, partial_bytes_avail, want_split);
+    return s;
+}
+
+struct Resolved {
+    int64_t M, N, K;
+    bool block_scaled;
+    const float* As;
+    const float* Bs;
+};
+
+}  // namespace
+
+extern "C" {
+
+int32_t tg_abi_version(void) { return TG_ABI_VERSION; }
+
+const char* tg_rc_message(int32_t rc) {
+    switch (rc) {
+        case TG_OK: return "ok";
+        case TG_ERR_DTYPE: return "unsupported dtype";
+        case TG_ERR_LAUNCH: return "kernel launch failed";
+        case TG_ERR_DEVICE: return "device init failed";
+        case TG_ERR_NULL: return "null tensor pointer";
+        case TG_ERR_INVALID: return "invalid arguments";
+        default: return "unknown error";
+    }
+}
+
+const char* tg_last_error(void) { return g_err; }
+
+int32_t tg_last_config(int32_t* out, int32_t n) {
+    if (!out || n <= 0) return 0;
+    const int32_t m = n < TG_CFG_COUNT ? n : TG_CFG_COUNT;
+    for (int32_t i = 0; i < m; ++i) out[i] = g_last_cfg[i];
+    return m;
+}
+
+int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t trans_b,
+                                    const int32_t* cfg, int32_t ncfg) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    int64_t split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
+    if (split <= 0) split = 16;
+    int64_t bytes = kCounterBytes;
+    // partial sums are only used while they stay a modest part of the traffic
+    int64_t partial = split * M * N * 4;
+    const int64_t cap = (int64_t)256 << 20;
+    if (partial > cap) partial = cap;
+    bytes += (partial + 255) / 256 * 256;
+    if (!trans_b) bytes += (N * K + 255) / 256 * 256;
+    return bytes;
+}
+
+int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                    const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
+                    int32_t trans_b, float alpha, float beta, const tg_tensor* workspace,
+                    const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(a, "a", 2)) || (rc = check_tensor(b, "b", 2)) || (rc = check_tensor(c, "c", 2))) return rc;
+    if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN)
+        return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7), got %d and %d", a->dtype, b->dtype);
+    const int out_type = out_type_of(c->dtype);
+    if (out_type < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16 or f32, got dtype code %d", c->dtype);
+    const int64_t M = trans_a ? a->shape[1] : a->shape[0], K = trans_a ? a->shape[0] : a->shape[1];
+    const int64_t N = trans_b ? b->shape[0] : b->shape[1], Kb = trans_b ? b->shape[1] : b->shape[0];
+    if (K != Kb) return fail(TG_ERR_INVALID, "incompatible matrices: K of a is %lld, K of b is %lld", (long long)K, (long long)Kb);
+    if (c->shape[0] != M || c->shape[1] != N)
+        return fail(TG_ERR_INVALID, "c must be (%lld, %lld), got (%lld, %lld)", (long long)M, (long long)N, (long long)c->shape[0], (long long)c->shape[1]);
+    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return fail(TG_ERR_INVALID, "extent exceeds int32");
+    const int64_t kblocks = cdiv(K, 128), nblocks = cdiv(N, 128);
+
+    // ---- scales
+    enum Kind { NONE, TENSOR, BLOCK };
+    auto kind_of = [&](const tg_tensor* s, const char* name, int64_t rows, int32_t* err) -> Kind {
+        *err = TG_OK;
+        if (!s) return NONE;
+        if ((*err = check_tensor(s, name, -1))) return NONE;
+        if (s->dtype != TG_F32) { *err = fail(TG_ERR_DTYPE, "%s must be f32", name); return NONE; }
+        if (numel(s) == 1) return TENSOR;
+        if (s->ndim == 2 && s->shape[0] == rows && s->shape[1] == kblocks) return BLOCK;
+        *err = fail(TG_ERR_INVALID, "%s: expected 1 element or shape (%lld, %lld)", name, (long long)rows, (long long)kblocks);
+        return NONE;
+    };
+    const Kind ka = kind_of(scale_a, "scale_a", M, &rc);
+    if (rc) return rc;
+    const Kind kb = kind_of(scale_b, "scale_b", nblocks, &rc);
+    if (rc) return rc;
+    const bool block_scaled = (ka == BLOCK || kb == BLOCK);
+    if (block_scaled && (ka == TENSOR || kb == TENSOR) && !(M == 1 && kblocks == 1) && !(nblocks == 1 && kblocks == 1))
+        return fail(TG_ERR_INVALID, "scale_a and scale_b must both be per-tensor or both be block scales");
+    if (block_scaled && (trans_a || !trans_b))
+        return fail(TG_ERR_INVALID, "block scales require a (M,K) and b (N,K) (trans_a=0, trans_b=1)");
+    if (workspace) {
+        if ((rc = check_tensor(workspace, "workspace", -1))) return rc;
+        if (!aligned16(workspace->ptr)) return fail(TG_ERR_INVALID, "workspace must be 16-byte aligned");
+    }
+    if (M == 0 || N == 0) return TG_OK;
+
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+
+    // ---- workspace carving: [counters][partials ...][optional K-contiguous copy of B]
+    const int64_t ws_bytes = workspace ? numel(workspace) * elem_size(workspace->dtype) : 0;
+    uint8_t* ws = workspace ? reinterpret_cast<uint8_t*>(workspace->ptr) : nullptr;
+    int64_t ws_free = ws_bytes > kCounterBytes ? ws_bytes - kCounterBytes : 0;
+    uint8_t* ws_cursor = ws ? ws + kCounterBytes : nullptr;
+
+    const uint8_t* Bnt = reinterpret_cast<const uint8_t*>(b->ptr);
+    bool b_is_nk = trans_b != 0;
+    const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
+    if (!b_is_nk && !trans_a && want_kernel != 0 && K > 0) {
+        // (K,N) weights: make a K-contiguous copy at the tail of the workspace when it fits
+        const int64_t need = (N * K + 255) / 256 * 256;
+        if (ws_free >= need) {
+            uint8_t* bt = ws + ws_bytes - need;
+            bt = reinterpret_cast<uint8_t*>(reinterpret_cast<uintptr_t>(bt) & ~(uintptr_t)15);
+            if (bt >= ws_cursor) {
+                if (tg::run_transpose_u8(Bnt, bt, (int)K, (int)N, stream) != hipSuccess)
+                    return fail(TG_ERR_LAUNCH, "transpose launch failed");
+                Bnt = bt;
+                b_is_nk = true;
+                ws_free = bt - ws_cursor;
+            }
+        }
+    }
+
+    const bool fast_layout = !trans_a && b_is_nk && (K % 16) == 0 && aligned16(a->ptr) &&
+                             aligned16(reinterpret_cast<uint64_t>(Bnt)) && N * K < kOffsetLimit;
+    Schedule s = choose_dense(M, N, K, block_scaled, fast_layout, cfg, ncfg, ws_free);
+
+    tg::GemmParams p{};
+    p.A = reinterpret_cast<const uint8_t*>(a->ptr);
+    p.B = Bnt;
+    p.C = reinterpret_cast<void*>(c->ptr);
+    p.As = scale_a ? reinterpret_cast<const float*>(scale_a->ptr) : nullptr;
+    p.Bs = scale_b ? reinterpret_cast<const float*>(scale_b->ptr) : nullptr;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    p.kblocks = (int)kblocks; p.nblocks = (int)nblocks;
+    p.alpha = alpha; p.beta = beta;
+    p.out_type = out_type;
+    p.vec_store = ((N % 4) == 0 && aligned16(c->ptr)) ? 1 : 0;
+    p.split_k = 1;
+    p.ksteps_per_split = (int)kblocks;
+    p.E = 1; p.top_k = 1;
+
+    if (s.kernel == 0) {
+        tg::GenericParams q{};
+        q.g = p;
+        q.a_sm = trans_a ? 1 : K; q.a_sk = trans_a ? M : 1;
+        const bool nk = trans_b != 0;  // the fallback reads the caller's own B
+        q.g.B = reinterpret_cast<const uint8_t*>(b->ptr);
+        q.b_sn = nk ? K : 1; q.b_sk = nk ? 1 : N;
+        q.b_se = 0;
+        q.group = tg::GROUP_DENSE;
+        q.block_scaled = block_scaled ? 1 : 0;
+        q.rows = (int)M;
+        remember(s);
+        if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");
+        return TG_OK;
+    }
+
+    if (s.split_k > 1) {
+        p.split_k = s.split_k;
+        p.ksteps_per_split = (int)cdiv(kblocks, s.split_k);
+        p.counters = reinterpret_cast<int*>(ws);
+        p.partials = reinterpret_cast<float*>(ws_cursor);
+    }
+    remember(s);
+
+    if (s.kernel == 2) {
+        const int gx = (int)cdiv(N, 16 * s.row_groups);
+        hipError_t e = tg::run_skinny(s.mt, s.row_groups, block_scaled, p, gx, s.split_k, stream);
+        if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "skinny kernel launch failed: %s", hipGetErrorString(e));
+        return TG_OK;
+    }
+
+    // tiled kernel; rows are chunked so that 32-bit byte offsets into A suffice
+    const int64_t max_rows = K > 0 ? ((kOffsetLimit - 1) / K) / s.bm * s.bm : M;
+    if (max_rows <= 0) return fail(TG_ERR_INVALID, "K too large");
+    for (int64_t r0 = 0; r0 < M; r0 += max_rows) {
+        const int64_t rows = (M - r0) < max_rows ? (M - r0) : max_rows;
+        tg::GemmParams pc = p;
+        pc.A = p.A + r0 * K;
+        pc.C = reinterpret_cast<uint8_t*>(p.C) + r0 * N * elem_size(c->dtype);
+        if (block_scaled && p.As) pc.As = p.As + r0 * kblocks;
+        pc.M = (int)rows;
+        if (rows != M && s.split_k > 1) { pc.split_k = 1; pc.ksteps_per_split = (int)kblocks; }
+        const int gx = (int)(cdiv(rows, s.bm) * cdiv(N, s.bn));
+        const bool split = pc.split_k > 1;
+        hipError_t e = block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
+                                    : tg::run_tile_per_tensor(s.bm, s.bn, split, pc, gx, pc.split_k, stream);
+        if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "tiled kernel launch failed: %s", hipGetErrorString(e));
+    }
+    return TG_OK;
+}
+
+// Shared validation of the two grouped entry points.
+static int32_t grouped_common(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                              const tg_tensor* a_scale, const tg_tensor* b_scale, int64_t* rows_a,
+                              int64_t* E, int64_t* N, int64_t* K, int* out_type) {
+    int32_t rc;
+    if ((rc = check_tensor(a, "a", 2)) || (rc = check_tensor(b, "b", 3)) || (rc = check_tensor(c, "c", 2))) return rc;
+    if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN)
+        return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7)");
+    *out_type = out_type_of(c->dtype);
+    if (*out_type < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16 or f32");
+    *rows_a = a->shape[0];
+    *K = a->shape[1];
+    *E = b->shape[0];
+    *N = b->shape[1];
+    if (b->shape[2] != *K) return fail(TG_ERR_INVALID, "K dimensions must match: %lld != %lld", (long long)*K, (long long)b->shape[2]);
+    if (c->shape[1] != *N) return fail(TG_ERR_INVALID, "c must have %lld columns", (long long)*N);
+    if (*rows_a > INT32_MAX || *N > INT32_MAX || *K > INT32_MAX || *E > INT32_MAX) return fail(TG_ERR_INVALID, "extent exceeds int32");
+    const int64_t kblocks = cdiv(*K, 128), nblocks = cdiv(*N, 128);
+    if (a_scale) {
+        if ((rc = check_tensor(a_scale, "a_scale", 2))) return rc;
+        if (a_scale->dtype != TG_F32) return fail(TG_ERR_DTYPE, "a_scale must be f32");
+        if (a_scale->shape[0] != *rows_a || a_scale->shape[1] != kblocks)
+            return fail(TG_ERR_INVALID, "a_scale must be (%lld, %lld)", (long long)*rows_a, (long long)kblocks);
+    }
+    if (b_scale) {
+        if ((rc = check_tensor(b_scale, "b_scale", 3))) return rc;
+        if (b_scale->dtype != TG_F32) return fail(TG_ERR_DTYPE, "b_scale must be f32");
+        if (b_scale->shape[0] != *E || b_scale->shape[1] != nblocks || b_scale->shape[2] != kblocks)
+            return fail(TG_ERR_INVALID, "b_scale must be (%lld, %lld, %lld)", (long long)*E, (long long)nblocks, (long long)kblocks);
+    }
+    return TG_OK;
+}
+
+static void fill_grouped(tg::GemmParams& p, const tg_tensor* c, const tg_tensor* a,
+                         const tg_tensor* b, const tg_tensor* a_scale, const tg_tensor* b_scale,
+                         int64_t rows_c, int64_t E, int64_t N, int64_t K, int out_type) {
+    p.A = reinterpret_cast<const uint8_t*>(a->ptr);
+    p.B = reinterpret_cast<const uint8_t*>(b->ptr);
+    p.C = reinterpret_cast<void*>(c->ptr);
+    p.As = a_scale ? reinterpret_cast<const float*>(a_scale->ptr) : nullptr;
+    p.Bs = b_scale ? reinterpret_cast<const float*>(b_scale->ptr) : nullptr;
+    p.M = (int)rows_c; p.N = (int)N; p.K = (int)K;
+    p.kblocks = (int)cdiv(K, 128); p.nblocks = (int)cdiv(N, 128);
+    p.alpha = 1.0f; p.beta = 0.0f;
+    p.out_type = out_type;
+    p.vec_store = ((N % 4) == 0 && aligned16(c->ptr)) ? 1 : 0;
+    p.split_k = 1;
+    p.ksteps_per_split = p.kblocks;
+    p.E = (int)E;
+    p.top_k = 1;
+}
+
+int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                           const tg_tensor* a_scale, const tg_tensor* b_scale,
+                           const tg_tensor* m_indptr, const int32_t* cfg, int32_t ncfg,
+                           int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int64_t total_m, E, N, K;
+    int out_type;
+    int32_t rc = grouped_common(c, a, b, a_scale, b_scale, &total_m, &E, &N, &K, &out_type);
+    if (rc) return rc;
+    if (c->shape[0] != total_m) return fail(TG_ERR_INVALID, "c must have %lld rows", (long long)total_m);
+    if ((rc = check_tensor(m_indptr, "m_indptr", 1))) return rc;
+    if (m_indptr->dtype != TG_I32) return fail(TG_ERR_DTYPE, "m_indptr must be int32");
+    if (m_indptr->shape[0] != E + 1) return fail(TG_ERR_INVALID, "m_indptr must have Q+1 = %lld elements", (long long)(E + 1));
+    if (total_m == 0 || N == 0 || E == 0) return TG_OK;
+
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+
+    tg::GemmParams p{};
+    fill_grouped(p, c, a, b, a_scale, b_scale, total_m, E, N, K, out_type);
+    p.m_indptr = reinterpret_cast<const int*>(m_indptr->ptr);
+
+    const bool fast = (K % 128) == 0 && K > 0 && aligned16(a->ptr) && aligned16(b->ptr) &&
+                      total_m * K < kOffsetLimit && N * K < kOffsetLimit &&
+                      cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
+    Schedule s{0, -1, -1, 1, -1, -1};
+    if (!fast) {
+        tg::GenericParams q{};
+        q.g = p;
+        q.a_sm = K; q.a_sk = 1; q.b_sn = K; q.b_sk = 1; q.b_se = N * K;
+        q.group = tg::GROUP_RAGGED;
+        q.block_scaled = 1;
+        q.rows = (int)total_m;
+        remember(s);
+        if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");
+        return TG_OK;
+    }
+    int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
+    if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, true))) {
+        bm = (total_m / E >= 96) ? 128 : 64;
+        bn = (bm == 128 && N >= 2048) ? 256 : 128;
+    }
+    s.kernel = 1; s.bm = bm; s.bn = bn;
+    remember(s);
+    // upper bound on the number of row tiles: every expert adds at most one partial tile
+    const int64_t row_tiles = total_m / bm + E;
+    const int64_t gx = row_tiles * cdiv(N, bn);
+    if (gx > INT32_MAX) return fail(TG_ERR_INVALID, "too many tiles");
+    hipError_t e = tg::run_tile_block_grouped(bm, bn, tg::GROUP_RAGGED, p, (int)gx, stream);
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "grouped kernel launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
+int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                        const tg_tensor* a_scale, const tg_tensor* b_scale,
+                        const tg_tensor* topk_weights, const tg_tensor* sorted_token_ids,
+                        const tg_tensor* expert_ids, const tg_tensor* num_tokens_post_padded,
+                        int32_t mul_routed_weight, int32_t top_k, int32_t block_m,
+                        const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int64_t T, E, N, K;
+    int out_type;
+    int32_t rc = grouped_common(c, a, b, a_scale, b_scale, &T, &E, &N, &K, &out_type);
+    if (rc) return rc;
+    if (top_k <= 0) return fail(TG_ERR_INVALID, "top_k must be positive");
+    if (block_m <= 0 || block_m % 16) return fail(TG_ERR_INVALID, "block_m must be a positive multiple of 16");
+    const int64_t num_valid = c->shape[0];
+    if (num_valid > T * top_k) return fail(TG_ERR_INVALID, "c has %lld rows but a provides only %lld slots", (long long)num_valid, (long long)(T * top_k));
+    if ((rc = check_tensor(sorted_token_ids, "sorted_token_ids", 1)) || (rc = check_tensor(expert_ids, "expert_ids", 1)) ||
+        (rc = check_tensor(num_tokens_post_padded, "num_tokens_post_padded", -1)))
+        return rc;
+    if (sorted_token_ids->dtype != TG_I32 || expert_ids->dtype != TG_I32 || num_tokens_post_padded->dtype != TG_I32)
+        return fail(TG_ERR_DTYPE, "sorted_token_ids, expert_ids and num_tokens_post_padded must be int32");
+    if (numel(num_tokens_post_padded) < 1) return fail(TG_ERR_INVALID, "num_tokens_post_padded must hold one element");
+    const int64_t EM = sorted_token_ids->shape[0];
+    if (expert_ids->shape[0] * block_m < EM)
+        return fail(TG_ERR_INVALID, "expert_ids too short: %lld blocks of %d for %lld slots", (long long)expert_ids->shape[0], block_m, (long long)EM);
+    if (mul_routed_weight) {
+        if (!topk_weights) return fail(TG_ERR_NULL, "topk_weights required when mul_routed_weight is set");
+        if ((rc = check_tensor(topk_weights, "topk_weights", -1))) return rc;
+        if (topk_weights->dtype != TG_F32) return fail(TG_ERR_DTYPE, "topk_weights must be f32");
+        if (numel(topk_weights) < num_valid) return fail(TG_ERR_INVALID, "topk_weights too short");
+    }
+    if (num_valid == 0 || N == 0 || EM == 0) return TG_OK;
+
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+
+    tg::GemmParams p{};
+    fill_grouped(p, c, a, b, a_scale, b_scale, num_valid, E, N, K, out_type);
+    p.sorted_ids = reinterpret_cast<const int*>(sorted_token_ids->ptr);
+    p.expert_ids = reinterpret_cast<const int*>(expert_ids->ptr);
+    p.num_post_pad = reinterpret_cast<const int*>(num_tokens_post_padded->ptr);
+    p.row_weight = mul_routed_weight ? reinterpret_cast<const float*>(topk_weights->ptr) : nullptr;
+    p.top_k = top_k;
+    p.num_valid = (int)num_valid;
+    p.block_m = block_m;
+    p.em_capacity = (int)EM;
+
+    int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
+    if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, true) && block_m % bm == 0)) {
+        bm = (block_m % 128 == 0) ? 128 : (block_m % 64 == 0) ? 64 : 0;
+        bn = (bm == 128 && N >= 2048) ? 256 : 128;
+    }
+    const bool fast = bm > 0 && (K % 128) == 0 && K > 0 && aligned16(a->ptr) && aligned16(b->ptr) &&
+                      T * K < kOffsetLimit && N * K < kOffsetLimit && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
+    Schedule s{0, -1, -1, 1, -1, -1};
+    if (!fast) {
+        tg::GenericParams q{};
+        q.g = p;
+        q.a_sm = K; q.a_sk = 1; q.b_sn = K; q.b_sk = 1; q.b_se = N * K;
+        q.group = tg::GROUP_GATHER;
+        q.block_scaled = 1;
+        q.rows = (int)EM;
+        remember(s);
+        if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");
+        return TG_OK;
+    }
+    s.kernel = 1; s.bm = bm; s.bn = bn;
+    remember(s);
+    const int64_t gx = cdiv(EM, bm) * cdiv(N, bn);
+    if (gx > INT32_MAX) return fail(TG_ERR_INVALID, "too many tiles");
+    hipError_t e = tg::run_tile_block_grouped(bm, bn, tg::GROUP_GATHER, p, (int)gx, stream);
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "grouped kernel launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,185 @@
+""" "hip" implementations of the dense and grouped FP8 GEMM ops.  Each one validates like the
+reference implementation it replaces, allocates the output with torch on the inputs' device,
+and enqueues the HIP kernels on torch's current stream through the C ABI."""
+
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence
+
+import torch
+
+from ... import _lib
+from ...backend import register_impl
+
+FP8 = torch.float8_e4m3fn
+_OUT_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+
+
+def _require_fp8(*tensors):
+    for t in tensors:
+        if t.dtype != FP8:
+            raise NotImplementedError(
+                f"the hip backend implements float8_e4m3fn GEMM only (got {t.dtype})")
+
+
+def _split_scale(scale, alpha: float):
+    """float scales fold into alpha; tensors are passed to the kernel (read on the device)."""
+    if scale is None:
+        return None, alpha
+    if isinstance(scale, (int, float)):
+        return None, alpha * float(scale)
+    if not isinstance(scale, torch.Tensor):
+        raise TypeError("scale must be a float or a tensor")
+    s = scale
+    if s.dtype != torch.float32:
+        s = s.float()
+    return s.contiguous(), alpha
+
+
+@register_impl("matmul", backend="hip")
+def matmul(a, b, trans_a=None, trans_b=None, static_persistent=None, use_tma=None, **kwargs):
+    trans_a = bool(trans_a) if trans_a is not None else False
+    trans_b = bool(trans_b) if trans_b is not None else False
+    _require_fp8(a, b)
+    if a.dim() != 2 or b.dim() != 2:
+        raise ValueError("matmul expects 2-D operands")
+    if trans_a:
+        K, M = a.shape
+    else:
+        M, K = a.shape
+    if trans_b:
+        N, KB = b.shape
+    else:
+        KB, N = b.shape
+    assert K == KB, f"Incompatible matrices: K dimension of A is {K}, K dimension of B is {KB}"
+    assert a.is_contiguous() and b.is_contiguous(), "operands must be contiguous"
+
+    out_dtype = kwargs.get("out_dtype")
+    cast_back = None
+    if out_dtype is None:
+        # reference behaviour: result in a.dtype (src/tilegym/ops/cutile/matmul.py:446)
+        cast_back = a.dtype
+        out_dtype = torch.float32
+    if out_dtype not in _OUT_DTYPES:
+        raise NotImplementedError(f"out_dtype {out_dtype} not supported")
+    sa, alpha = _split_scale(kwargs.get("scale_a"), float(kwargs.get("alpha", 1.0)))
+    sb, alpha = _split_scale(kwargs.get("scale_b"), alpha)
+    c = torch.empty((M, N), device=a.device, dtype=out_dtype)
+    _lib.fp8_gemm(c, a, b, sa, sb, trans_a, trans_b, alpha, 0.0, kwargs.get("kernel_configs"))
+    return c.to(cast_back) if cast_back is not None else c
+
+
+@register_impl("flashinfer.gemm.gemm_alpha_beta", backend="hip")
+def gemm_alpha_beta(a, b, c, trans_a=False, trans_b=True, alpha=1.0, beta=0.0, num_sms=None, **kwargs):
+    """C <- alpha * A @ B(^T) + beta * C, in place
+    (src/tilegym/suites/flashinfer/cutile/gemm/gemm_alpha_beta.py:336-504).  ``num_sms`` throttles
+    the reference's persistent grid and has no meaning here; it is ignored."""
+    _require_fp8(a, b)
+    if trans_a:
+        K, M = a.shape
+    else:
+        M, K = a.shape
+    if trans_b:
+        N, KB = b.shape
+    else:
+        KB, N = b.shape
+    assert K == KB, "incompatible dimensions"
+    assert c.shape == (M, N), "C must have shape [M, N]"
+    assert a.is_contiguous(), "A matrix must be contiguous"
+    assert b.is_contiguous(), "B matrix must be contiguous"
+    assert c.is_contiguous(), "C matrix must be contiguous"
+    if c.dtype not in _OUT_DTYPES:
+        raise NotImplementedError(f"C dtype {c.dtype} not supported")
+    _lib.fp8_gemm(c, a, b, None, None, bool(trans_a), bool(trans_b), float(alpha), float(beta),
+                  kwargs.get("kernel_configs"))
+    return c
+
+
+@register_impl("unsloth.w8a8_block_fp8_matmul", backend="hip")
+def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: Optional[Sequence[int]] = None,
+                          output_dtype: torch.dtype = torch.float32, **kwargs):
+    """Block-scaled FP8 GEMM (src/tilegym/suites/unsloth/cutile/fp8.py:388-446)."""
+    if block_size is None:
+        block_n, block_k = 128, 128
+    else:
+        assert len(block_size) == 2
+        block_n, block_k = block_size[0], block_size[1]
+    if (block_n, block_k) != (128, 128):
+        raise NotImplementedError("the hip backend implements 128x128 quantization blocks only")
+    _require_fp8(A, B)
+    N, K = B.shape
+    assert A.shape[-1] == B.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1] and A.is_contiguous()
+    assert math.ceil(A.shape[-1] / block_k) == As.shape[-1]
+    assert B.ndim == 2 and B.is_contiguous() and Bs.ndim == 2
+    assert math.ceil(N / block_n) == Bs.shape[0]
+    assert math.ceil(K / block_k) == Bs.shape[1]
+    if output_dtype not in _OUT_DTYPES:
+        raise NotImplementedError(f"output_dtype {output_dtype} not supported")
+    M = A.numel() // A.shape[-1]
+    C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
+    if M == 0:
+        return C
+    As2 = As.reshape(M, -1).float().contiguous()
+    Bs2 = Bs.float().contiguous()
+    _lib.fp8_gemm(C.view(M, N), A.view(M, K), B, As2, Bs2, False, True, 1.0, 0.0,
+                  kwargs.get("kernel_configs"))
+    return C
+
+
+@register_impl("flashinfer.gemm.ragged_block_scaled_bmm", backend="hip")
+def ragged_block_scaled_bmm(a, b, a_scale, b_scale, m_indptr, max_m, max_m_device=None,
+                            transpose_a=False, transpose_b=True, out_dtype=None, **kwargs):
+    """Grouped block-scaled FP8 GEMM over expert segments
+    (src/tilegym/suites/flashinfer/cutile/gemm/ragged_block_scaled_bmm.py:497-616).
+    ``max_m`` / ``max_m_device`` bound the reference's uniform tile walk; the expert-offset
+    launch here reads the segment sizes on the device, so both are accepted and unused."""
+    assert transpose_a == False and transpose_b == True, "Only NT layout is supported"  # noqa: E712
+    assert a.is_contiguous(), "A matrix must be contiguous"
+    assert b.is_contiguous(), "B matrix must be contiguous"
+    assert a_scale is None or a_scale.is_contiguous(), "A scale matrix must be contiguous"
+    assert b_scale.is_contiguous(), "B scale matrix must be contiguous"
+    assert m_indptr.is_contiguous(), "m_indptr must be contiguous"
+    _require_fp8(a, b)
+    total_m, K_A = a.shape
+    Q, N, K_B = b.shape
+    assert K_A == K_B, f"K dimensions must match: {K_A} != {K_B}"
+    assert m_indptr.shape[0] == Q + 1, "m_indptr must have Q+1 elements"
+    Q_SB, rnb, rkb = b_scale.shape
+    if K_B // rkb != 128 or math.ceil(N / 128) != rnb:
+        raise NotImplementedError("the hip backend implements 128x128 quantization blocks only")
+    if a_scale is not None:
+        assert a_scale.shape[0] == total_m, "a_scale total_m dimension mismatch"
+    assert Q_SB == Q, "b_scale Q dimension mismatch"
+    if out_dtype is None:
+        out_dtype = torch.bfloat16
+    if out_dtype not in _OUT_DTYPES:
+        raise NotImplementedError(f"out_dtype {out_dtype} not supported")
+    # rows past m_indptr[-1] belong to no segment and are left untouched by the kernel
+    c = torch.zeros((total_m, N), device=a.device, dtype=out_dtype) if kwargs.get("zero_init") \
+        else torch.empty((total_m, N), device=a.device, dtype=out_dtype)
+    ptr = m_indptr if m_indptr.dtype == torch.int32 else m_indptr.to(torch.int32)
+    a_s = None if a_scale is None else a_scale.float()
+    _lib.fp8_ragged_gemm(c, a, b, a_s, b_scale.float(), ptr, kwargs.get("kernel_configs"))
+    return c
+
+
+@register_impl("group_gemm", backend="hip")
+def group_gemm(group_A, group_B, static_persistent=True, use_tma=True, transpose_b=False, **kwargs):
+    """List of GEMMs (src/tilegym/ops/cutile/group_gemm.py:170-197): one launch per group, all
+    on the current stream; outputs in ``A.dtype`` unless ``out_dtype`` is given."""
+    if not group_A or not group_B:
+        raise ValueError("group_A and group_B must not be empty")
+    if len(group_A) != len(group_B):
+        raise ValueError(f"group_A and group_B must have same length, got {len(group_A)} and {len(group_B)}")
+    scales_a: Optional[List] = kwargs.get("scales_a")
+    scales_b: Optional[List] = kwargs.get("scales_b")
+    outs = []
+    for i, (A, B) in enumerate(zip(group_A, group_B)):
+        outs.append(matmul(A, B, False, bool(transpose_b),
+                           scale_a=None if scales_a is None else scales_a[i],
+                           scale_b=None if scales_b is None else scales_b[i],
+                           out_dtype=kwargs.get("out_dtype"),
+                           kernel_configs=kwargs.get("kernel_configs")))
+    return outs

@@ -1,0 +1,74 @@
+""" "hip" implementations of the MoE entry points."""
+
+from __future__ import annotations
+
+import torch
+
+from ... import _lib
+from ...backend import register_impl
+
+FP8 = torch.float8_e4m3fn
+
+
+@register_impl("invoke_fused_moe_kernel", backend="hip")
+def invoke_fused_moe_kernel(A, B, C, A_scale, B_scale, topk_weights, topk_ids, sorted_token_ids,
+                            expert_ids, num_tokens_post_padded, mul_routed_weight, top_k, config,
+                            compute_type=None, use_fp8_w8a8=True, use_int8_w8a16=False,
+                            block_shape=None, **kwargs) -> None:
+    """Token-gather block-scaled FP8 GEMM (src/tilegym/ops/tilecpp/moe.py:241-310): row r of the
+    sorted slot list reads A[id // top_k], multiplies with B[expert_ids[r // BLOCK_SIZE_M]] and
+    writes C[id] (id = sorted_token_ids[r]); padding slots (id >= numel(topk_ids)) are skipped."""
+    if use_int8_w8a16:
+        raise NotImplementedError("int8 weights are not implemented by the hip backend")
+    if not use_fp8_w8a8 or A.dtype != FP8 or B.dtype != FP8:
+        raise NotImplementedError("the hip backend implements the use_fp8_w8a8 path only "
+                                  "(float8_e4m3fn activations and weights)")
+    if block_shape is not None and tuple(block_shape) != (128, 128):
+        raise NotImplementedError("the hip backend implements 128x128 quantization blocks only")
+    assert topk_weights is None or topk_weights.stride(1) == 1
+    assert sorted_token_ids.stride(0) == 1
+    assert A.is_contiguous() and B.is_contiguous() and C.is_contiguous()
+    block_m = int(config.get("BLOCK_SIZE_M", config.get("TILE_SIZE_M", 128)))
+    num_valid = topk_ids.numel()
+    N = B.shape[1]
+    c2 = C.view(-1, N)
+    assert c2.shape[0] == num_valid, "C must provide one row per (token, k) slot"
+    w = None
+    if mul_routed_weight:
+        w = topk_weights.reshape(-1).float().contiguous()
+    a_s = None if A_scale is None else A_scale.float().contiguous()
+    b_s = None if B_scale is None else B_scale.float().contiguous()
+    _lib.fp8_moe_gemm(c2, A, B, a_s, b_s, w, sorted_token_ids.to(torch.int32),
+                      expert_ids.to(torch.int32), num_tokens_post_padded.reshape(-1).to(torch.int32),
+                      bool(mul_routed_weight), int(top_k), block_m, kwargs.get("kernel_configs"))
+    return None
+
+
+@register_impl("moe_align_block_size", backend="hip")
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int):
+    """Device-side token alignment in torch ops, no host synchronisation; same outputs and buffer
+    sizes as src/tilegym/ops/cutile/moe_align_block.py:205-268: (sorted_ids[numel + E*(bs-1)]
+    pre-filled with the sentinel numel, expert_ids[ceil(that/bs)], num_tokens_post_pad[1],
+    cumsum[E+1] of padded counts, max_expert_cnt[1]).  Stable within an expert."""
+    dev = topk_ids.device
+    flat = topk_ids.reshape(-1).to(torch.int64)
+    numel = flat.numel()
+    cap = numel + num_experts * (block_size - 1)
+    nblk = -(-cap // block_size)
+    counts = torch.bincount(flat, minlength=num_experts)[:num_experts]
+    padded = (counts + block_size - 1) // block_size * block_size
+    cumsum = torch.zeros(num_experts + 1, dtype=torch.int64, device=dev)
+    cumsum[1:] = torch.cumsum(padded, 0)
+    starts_unpadded = torch.cumsum(counts, 0) - counts
+    order = torch.argsort(flat, stable=True)
+    sorted_experts = flat[order]
+    rank_in_expert = torch.arange(numel, device=dev) - starts_unpadded[sorted_experts]
+    dest = cumsum[sorted_experts] + rank_in_expert
+    sorted_ids = torch.full((cap,), numel, dtype=torch.int32, device=dev)
+    sorted_ids[dest] = order.to(torch.int32)
+    blk_start = torch.arange(nblk, device=dev, dtype=torch.int64) * block_size
+    expert_ids = torch.searchsorted(cumsum[1:].contiguous(), blk_start, right=True)
+    expert_ids = torch.where(blk_start < cumsum[-1], expert_ids, torch.zeros_like(expert_ids)).to(torch.int32)
+    post = cumsum[-1:].to(torch.int32)
+    mx = counts.max().reshape(1).to(torch.int32) if numel else torch.zeros(1, dtype=torch.int32, device=dev)
+    return sorted_ids, expert_ids, post, cumsum.to(torch.int32), mx
