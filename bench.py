@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 GEMM path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|decode|block|moe|all]
+
+A "step" is one pass over the workload's GEMMs with inputs already resident in HBM.  The headline
+line (one JSON object on stdout) reports the prefill workload -- the four Llama-3.1-8B projection
+GEMMs at M=8192, FP8 per-tensor scales, bf16 out -- as whole-step TFLOP/s (sum of 2*M*N*K over the
+time of K steps), with:
+  roofline      the dominant kernel (the 256x256 LDS-tiled MFMA kernel on the gate+up shape):
+                algorithmic FLOPs per launch / its average launch duration, against 5.0 PFLOP/s
+  decode        the same for the decode workload (M in {1,8,16,64}; weight streaming), in GB/s of
+                algorithmic bytes against 8 TB/s, per shape and aggregated, cold cache (operands
+                are rotated through > 512 MB so that launches do not hit the 256 MB memory-side cache)
+  cpu_baseline  the torch CPU oracle (dequantize -> fp32 matmul -> bf16) timed on this host's cores
+                on a bounded sample of the same workload
+Kernel durations are measured with HIP events on the stream the kernels are launched on.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense FP8 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+ROTATE_BYTES = 640 << 20   # operand footprint to rotate through (> 2x the 256 MB memory-side cache)
+
+
+def _events_ms(fn, iters, stream):
+    """Time `iters` calls of fn() with HIP events on `stream`; returns total milliseconds."""
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record(stream)
+    for i in range(iters):
+        fn(i)
+    end.record(stream)
+    torch.cuda.synchronize()
+    return start.elapsed_time(end)
+
+
+def _graph_ms(fn, launches, replays, stream):
+    """Capture `launches` calls of fn(i) into one HIP graph, replay it `replays` times between two
+    events.  Removes host launch overhead from the timed region (needed for microsecond kernels).
+    Returns total ms, or None if capture is not possible."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        with torch.cuda.stream(side):
+            for i in range(min(launches, 2)):
+                fn(i)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(launches):
+                fn(i)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(replays):
+            graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end)
+    except Exception as exc:  # capture unsupported: report, fall back to plain launches
+        print(f"[bench] graph timing unavailable ({type(exc).__name__}: {exc}); using plain launches", file=sys.stderr)
+        torch.cuda.synchronize()
+        return None
+
+
+class DenseRunner:
+    """One dense problem with its operands replicated `copies` times for cache-cold rotation."""
+
+    def __init__(self, case, device, copies):
+        from tilegym_amd import _lib
+        self._lib = _lib
+        self.case = case
+        self.copies = max(1, copies)
+        d = case.to(device)
+        self.a = [d.a] + [d.a.clone() for _ in range(self.copies - 1)]
+        self.b = [d.b] + [d.b.clone() for _ in range(self.copies - 1)]
+        self.sa, self.sb = d.scale_a, d.scale_b
+        self.c = [torch.empty(case.M, case.N, dtype=torch.bfloat16, device=device) for _ in range(min(self.copies, 4))]
+
+    def __call__(self, i):
+        j = i % self.copies
+        self._lib.fp8_gemm(self.c[i % len(self.c)], self.a[j], self.b[j], self.sa, self.sb, False, True, 1.0, 0.0)
+
+
+class RaggedRunner:
+    def __init__(self, case, device, copies):
+        from tilegym_amd import _lib
+        self._lib = _lib
+        self.case = case
+        self.copies = max(1, copies)
+        d = case.to(device)
+        self.a = [d.a] + [d.a.clone() for _ in range(self.copies - 1)]
+        self.b = [d.b] + [d.b.clone() for _ in range(self.copies - 1)]
+        self.d = d
+        self.c = torch.empty(d.a.shape[0], d.b.shape[1], dtype=torch.bfloat16, device=device)
+
+    def __call__(self, i):
+        j = i % self.copies
+        self._lib.fp8_ragged_gemm(self.c, self.a[j], self.b[j], self.d.a_scale, self.d.b_scale, self.d.m_indptr)
+
+
+def _copies_for(nbytes):
+    return max(2, min(64, -(-ROTATE_BYTES // max(1, int(nbytes)))))
+
+
+def measure_shape(runner, steps, warmup, stream, use_graph):
+    from tilegym_amd import _lib
+    for i in range(max(1, warmup)):
+        runner(i)
+    torch.cuda.synchronize()
+    cfg = _lib.last_config()
+    ms = None
+    launches = steps
+    if use_graph:
+        per_graph = max(runner.copies, 8)
+        replays = max(1, steps // per_graph)
+        ms = _graph_ms(runner, per_graph, replays, stream)
+        launches = per_graph * replays
+    if ms is None:
+        launches = steps
+        ms = _events_ms(runner, launches, stream)
+    us = ms * 1e3 / launches
+    case = runner.case
+    flops, nbytes = case.flops(), case.algorithmic_bytes()
+    return {
+        "name": case.name,
+        "kernel": cfg["KERNEL_NAME"], "block_m": cfg["BLOCK_M"], "block_n": cfg["BLOCK_N"],
+        "split_k": cfg["SPLIT_K"], "row_groups": cfg["ROW_GROUPS"],
+        "us": round(us, 3), "launches": launches,
+        "tflops": round(flops / us * 1e-6, 2), "gbs": round(nbytes / us * 1e-3, 1),
+        "flops": flops, "bytes": nbytes,
+        "frac_mfma": round(flops / us * 1e-6 / PEAK_FP8_TFLOPS, 4),
+        "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
+    }
+
+
+def cpu_baseline(sample_rows=1024):
+    """Time the torch CPU oracle on a bounded sample: `sample_rows` activation rows of the prefill
+    O-projection (N=K=4096), dequantization included."""
+    from oracle import reference as R
+    from tilegym_amd import workloads as W
+
+    case = W.llama_prefill_case("o", M=sample_rows)
+    threads = torch.get_num_threads()
+    R.ref_gemm_per_tensor(case.a[:64], case.b, case.scale_a, case.scale_b, trans_b=True)  # warm-up
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        R.ref_gemm_per_tensor(case.a, case.b, case.scale_a, case.scale_b, trans_b=True)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[1]
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {
+        "value": round(case.flops() / t * 1e-12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"torch CPU oracle (dequantize -> fp32 matmul -> bf16), prefill O-projection, {sample_rows} of 8192 rows "
+                  f"x N=4096 x K=4096, median of 3, {t:.3f} s; os.cpu_count()={os.cpu_count()}, cpu='{cpu_model}'",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="all", choices=["prefill", "decode", "block", "moe", "all"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time microsecond kernels with plain launches")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(1)
+
+    from tilegym_amd import _lib, workloads as W
+
+    _lib.load()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    stream = torch.cuda.current_stream()
+    props = torch.cuda.get_device_properties(device)
+    out = {}
+    detail = {}
+
+    # ------------------------------------------------------------------ prefill (headline)
+    if args.workload in ("prefill", "all"):
+        runners = [DenseRunner(W.llama_prefill_case(p), device, copies=2) for p in W.LLAMA_SHAPES]
+        for w in range(max(1, args.warmup)):
+            for r in runners:
+                r(w)
+        torch.cuda.synchronize()
+
+        def step(i):
+            for r in runners:
+                r(i)
+
+        ms = _events_ms(step, args.steps, stream)
+        total_flops = sum(r.case.flops() for r in runners)
+        ms_per_step = ms / args.steps
+        shapes = [measure_shape(r, args.steps, 1, stream, use_graph=False) for r in runners]
+        dom = max(shapes, key=lambda s: s["us"])
+        out.update({
+            "value": round(total_flops / (ms_per_step * 1e-3) * 1e-12, 2),
+            "ms_per_step": round(ms_per_step, 4),
+            "roofline": {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                         "frac": dom["frac_mfma"], "traffic": None, "kernel": f"fp8_gemm_tile_kernel<{dom['block_m']},{dom['block_n']}> per-tensor",
+                         "shape": dom["name"], "us_per_launch": dom["us"]},
+        })
+        detail["prefill"] = shapes
+        del runners
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ decode
+    if args.workload in ("decode", "all"):
+        shapes = []
+        for proj in W.LLAMA_SHAPES:
+            big = W.llama_decode_case(64, proj)
+            for M in W.DECODE_M:
+                case = W.DenseCase(f"c2_decode_{proj}_M{M}", big.a[:M].contiguous(), big.b, big.scale_a, big.scale_b, True, False)
+                r = DenseRunner(case, device, copies=_copies_for(case.algorithmic_bytes()))
+                shapes.append(measure_shape(r, max(args.steps, 64), args.warmup, stream, use_graph=not args.no_graph))
+                del r
+            torch.cuda.empty_cache()
+        tot_b = sum(s["bytes"] for s in shapes)
+        tot_us = sum(s["us"] for s in shapes)
+        small = [s for s in shapes if int(s["name"].rsplit("M", 1)[1]) <= 16]
+        dom = max(small, key=lambda s: s["us"])
+        dec = {
+            "metric": "FP8 GEMM decode GB/s (algorithmic bytes, cold cache)", "value": round(tot_b / tot_us * 1e-3, 1), "unit": "GB/s",
+            "us_per_step": round(tot_us, 2),
+            "frac_hbm_M_le_16": round(sum(s["bytes"] for s in small) / sum(s["us"] for s in small) * 1e-3 / PEAK_HBM_GBS, 4),
+            "roofline": {"bound": "hbm", "achieved": dom["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
+                         "traffic": None, "kernel": "fp8_gemm_skinny_kernel per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
+        }
+        detail["decode"] = shapes
+        if "value" in out:
+            out["decode"] = dec
+        else:
+            out.update({"value": dec["value"], "ms_per_step": round(tot_us * 1e-3, 5), "roofline": dec["roofline"]})
+            out["_metric"], out["_unit"] = dec["metric"], "GB/s"
+
+    # ------------------------------------------------------------------ block scaled / MoE (extra)
+    if args.workload in ("block", "all"):
+        shapes = []
+        for (N, K) in W.BLOCK_SCALED_SHAPES:
+            big = W.block_scaled_case(4096, N, K)
+            for M in W.BLOCK_SCALED_M:
+                case = W.DenseCase(f"c4_block_M{M}_{N}x{K}", big.a[:M].contiguous(), big.b, big.scale_a[:M].contiguous(), big.scale_b, True, True)
+                r = DenseRunner(case, device, copies=_copies_for(case.algorithmic_bytes()) if M <= 64 else 2)
+                shapes.append(measure_shape(r, args.steps if M > 64 else max(args.steps, 64), args.warmup, stream,
+                                            use_graph=(M <= 64 and not args.no_graph)))
+                del r
+            torch.cuda.empty_cache()
+        detail["block_scaled"] = shapes
+    if args.workload in ("moe", "all"):
+        shapes = []
+        for which in ("gate_up", "down"):
+            r = RaggedRunner(W.moe_grouped_case(which), device, copies=2)
+            shapes.append(measure_shape(r, args.steps, args.warmup, stream, use_graph=False))
+            del r
+            torch.cuda.empty_cache()
+        detail["moe_grouped"] = shapes
+
+    if "value" not in out:  # block / moe only
+        first = next(iter(detail.values()))
+        dom = max(first, key=lambda s: s["us"])
+        out.update({"value": dom["tflops"], "ms_per_step": round(dom["us"] * 1e-3, 5),
+                    "roofline": {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": dom["frac_mfma"], "traffic": None, "shape": dom["name"]}})
+
+    line = {
+        "metric": out.pop("_metric", "FP8 GEMM TFLOP/s (prefill: Llama-3.1-8B projections, M=8192, e4m3 per-tensor scales, bf16 out)"),
+        "value": out.pop("value"),
+        "unit": out.pop("_unit", "TFLOP/s"),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": out.pop("ms_per_step"),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f8e4m3 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": {"prefill": "config 3: Llama-3.1-8B prefill projections, M=8192, (N,K) in qkv/o/gate_up/down",
+                                "decode": "config 2: Llama-3.1-8B decode projections, M in {1,8,16,64}",
+                                "block": "config 4: block-scaled 12288x5120 / 5120x12288, M in {16,4096}",
+                                "moe": "config 5: DeepSeek-V2-Lite MoE grouped GEMMs",
+                                "all": "config 3 (headline) + configs 2, 4, 5"}[args.workload],
+                   "device": props.name, "compute_units": props.multi_processor_count},
+    }
+    line.update(out)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    line["shapes"] = {k: [{kk: vv for kk, vv in s.items() if kk not in ("flops", "bytes")} for s in v] for k, v in detail.items()}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

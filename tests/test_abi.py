@@ -1,0 +1,129 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol the header declares,
+and validates arguments before touching a device (no compute calls here)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from tilegym_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FP8 = torch.float8_e4m3fn
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "tilegym_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    L = _lib.load()
+    names = _declared_symbols()
+    assert {"tg_fp8_gemm", "tg_fp8_ragged_gemm", "tg_fp8_moe_gemm", "tg_fp8_gemm_workspace_bytes",
+            "tg_rc_message", "tg_abi_version", "tg_last_config", "tg_last_error"} <= set(names)
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/tilegym_hip.h but not exported"
+    assert L.tg_abi_version() == 1
+
+
+def test_rc_messages():
+    L = _lib.load()
+    want = {0: b"ok", -2: b"unsupported dtype", -3: b"kernel launch failed", -4: b"device init failed",
+            -5: b"null tensor pointer", -6: b"invalid arguments", -99: b"unknown error"}
+    for rc, msg in want.items():
+        assert L.tg_rc_message(rc) == msg
+
+
+def test_tensor_desc_layout_matches_header():
+    # ptr u64, ndim i32 (+pad), shape i64[5], strides i64[5], dtype i32 (+pad)
+    assert ctypes.sizeof(_lib.TgTensor) == 8 + 8 + 40 + 40 + 8
+    t = torch.zeros(3, 5, dtype=torch.bfloat16)[:, ::2]
+    d = _lib.make_tensor_desc(t)
+    assert d.ndim == 2 and list(d.shape[:2]) == [3, 3] and list(d.strides[:2]) == [5, 2]
+    assert d.dtype == 2 and d.ptr == t.data_ptr()
+    assert _lib.make_tensor_desc(torch.zeros(1).to(FP8)).dtype == 7
+    assert _lib.make_tensor_desc(None) is None
+
+
+def _call_gemm(c, a, b, sa=None, sb=None, ta=0, tb=1, ws=None):
+    L = _lib.load()
+    ds = [_lib.make_tensor_desc(t) for t in (c, a, b, sa, sb)]
+    dws = _lib.make_tensor_desc(ws)
+    cfg, n = _lib.make_cfg(None)
+    refs = [None if d is None else ctypes.byref(d) for d in ds]
+    rc = L.tg_fp8_gemm(*refs, ta, tb, 1.0, 0.0, None if dws is None else ctypes.byref(dws), cfg, n, 0, 0)
+    return rc, L.tg_last_error().decode()
+
+
+def test_gemm_argument_validation_runs_without_a_device():
+    a = torch.zeros(4, 128).to(FP8)
+    b = torch.zeros(8, 128).to(FP8)
+    c = torch.zeros(4, 8, dtype=torch.bfloat16)
+    L = _lib.load()
+    cfg, n = _lib.make_cfg(None)
+    dc, da = _lib.make_tensor_desc(c), _lib.make_tensor_desc(a)
+    assert L.tg_fp8_gemm(ctypes.byref(dc), ctypes.byref(da), None, None, None, 0, 1, 1.0, 0.0, None, cfg, n, 0, 0) == -5
+    assert _call_gemm(c, a.float(), b)[0] == -2                              # A not fp8
+    assert _call_gemm(c.to(torch.int32), a, b)[0] == -2                      # C dtype
+    rc, msg = _call_gemm(c, a, torch.zeros(8, 64).to(FP8))
+    assert rc == -6 and "K of a is 128" in msg                               # mismatched K
+    assert _call_gemm(torch.zeros(4, 9, dtype=torch.bfloat16), a, b)[0] == -6  # C shape
+    assert _call_gemm(c, a, b, sa=torch.ones(3))[0] == -6                    # bad scale shape
+    assert _call_gemm(c, a, b, sa=torch.ones(1, dtype=torch.float16))[0] == -2
+    assert _call_gemm(c, a, b, sa=torch.ones(4, 1), sb=torch.ones(1, 1), tb=0)[0] == -6  # block + NN
+    nc = torch.zeros(8, 8, dtype=torch.bfloat16)[::2]
+    assert _call_gemm(nc, a, b)[0] == -6                                     # non-contiguous
+    # empty problem is a no-op that needs no device
+    assert _call_gemm(torch.zeros(0, 8, dtype=torch.bfloat16), torch.zeros(0, 128).to(FP8), b)[0] == 0
+    if not torch.cuda.is_available():
+        rc, msg = _call_gemm(c, a, b)
+        assert rc == -4 and "device" in msg                                  # valid args, no GPU
+
+
+def test_grouped_argument_validation():
+    L = _lib.load()
+    cfg, n = _lib.make_cfg(None)
+    a = torch.zeros(10, 128).to(FP8)
+    b = torch.zeros(2, 16, 128).to(FP8)
+    c = torch.zeros(10, 16, dtype=torch.bfloat16)
+    ptr = torch.tensor([0, 4, 10], dtype=torch.int32)
+
+    def ragged(c, a, b, a_s, b_s, ptr):
+        ds = [_lib.make_tensor_desc(t) for t in (c, a, b, a_s, b_s, ptr)]
+        return L.tg_fp8_ragged_gemm(*[None if d is None else ctypes.byref(d) for d in ds], cfg, n, 0, 0)
+
+    assert ragged(c, a, b, None, None, ptr[:2]) == -6             # m_indptr length
+    assert ragged(c, a, b, None, None, ptr.long()) == -2          # m_indptr dtype
+    assert ragged(c, a, b, torch.ones(10, 2), None, ptr) == -6    # a_scale shape
+    assert ragged(c, a, b, None, torch.ones(2, 1, 2), ptr) == -6  # b_scale shape
+    assert ragged(c, a, torch.zeros(2, 16, 64).to(FP8), None, None, ptr) == -6
+    assert ragged(c, a, b, None, None, None) == -5
+
+    def moe(block_m=16, top_k=2, w=None, mul=0, sorted_ids=None, expert_ids=None):
+        sorted_ids = torch.zeros(32, dtype=torch.int32) if sorted_ids is None else sorted_ids
+        expert_ids = torch.zeros(2, dtype=torch.int32) if expert_ids is None else expert_ids
+        post = torch.tensor([32], dtype=torch.int32)
+        a5 = torch.zeros(5, 128).to(FP8)
+        ds = [_lib.make_tensor_desc(t) for t in (c, a5, b, None, None, w, sorted_ids, expert_ids, post)]
+        return L.tg_fp8_moe_gemm(*[None if d is None else ctypes.byref(d) for d in ds], mul, top_k, block_m, cfg, n, 0, 0)
+
+    assert moe(block_m=24) == -6                                   # block_m % 16
+    assert moe(top_k=0) == -6
+    assert moe(top_k=1) == -6                                      # 10 output rows > 5 tokens * 1
+    assert moe(mul=1) == -5                                        # weights required
+    assert moe(expert_ids=torch.zeros(1, dtype=torch.int32)) == -6
+
+
+def test_workspace_bytes_and_cfg():
+    L = _lib.load()
+    cfg, n = _lib.make_cfg(None)
+    assert L.tg_fp8_gemm_workspace_bytes(0, 10, 10, 1, cfg, n) == 0
+    nt = L.tg_fp8_gemm_workspace_bytes(16, 4096, 4096, 1, cfg, n)
+    nn = L.tg_fp8_gemm_workspace_bytes(16, 4096, 4096, 0, cfg, n)
+    assert nt >= 65536 + 16 * 4096 * 4 and nn >= nt + 4096 * 4096
+    cfg2, _ = _lib.make_cfg({"KERNEL": "skinny", "SPLIT_K": 4, "block_m": 128, "num_ctas": 2})
+    assert list(cfg2)[:5] == [2, 128, -1, 4, -1]

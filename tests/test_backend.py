@@ -1,0 +1,119 @@
+"""Host-layer semantics that need no GPU: registry/dispatch behaviour and the op signatures."""
+
+import inspect
+
+import pytest
+import torch
+
+import tilegym_amd
+from tilegym_amd import backend
+from tilegym_amd.ops import hip as hip_impls  # noqa: F401
+
+FP8 = torch.float8_e4m3fn
+
+
+def test_registry_holds_the_hot_path_ops():
+    info = tilegym_amd.get_registry_info()
+    for name in ("matmul", "group_gemm", "unsloth.w8a8_block_fp8_matmul", "flashinfer.gemm.gemm_alpha_beta",
+                 "flashinfer.gemm.ragged_block_scaled_bmm", "invoke_fused_moe_kernel", "moe_align_block_size"):
+        assert "hip" in info[name] and "default" in info[name]
+
+
+def test_backend_selection():
+    assert tilegym_amd.get_current_backend() == "hip"
+    assert tilegym_amd.is_backend_available("hip")
+    assert not tilegym_amd.is_backend_available("cutile")
+    with pytest.raises(ValueError):
+        tilegym_amd.set_backend("cutile")
+    tilegym_amd.set_backend("hip")
+
+
+def test_dispatch_semantics():
+    calls = []
+
+    @backend.dispatch("unit.test_op")
+    def op(x, y=1, **kwargs):
+        raise NotImplementedError("stub")
+
+    with pytest.raises(NotImplementedError):
+        op(1)
+
+    @backend.register_impl("unit.test_op", backend="hip")
+    def impl(x, y=1, **kwargs):
+        calls.append((x, y, kwargs))
+        return x + y
+
+    assert op(2, y=3, extra=5) == 5 and calls[-1] == (2, 3, {"extra": 5})
+    assert op(2, backend="hip") == 3            # explicit backend kwarg is consumed
+    assert "backend" not in calls[-1][2]
+    with pytest.raises(NotImplementedError):
+        op(2, backend="triton")
+    assert op._tilegym_op_name == "unit.test_op"
+    assert backend.get_available_backends_for_op("unit.test_op") == ["hip"]
+
+
+def test_signatures_match_the_reference_stubs():
+    from tilegym_amd.ops import group_gemm, matmul
+    from tilegym_amd.ops.moe_interface import invoke_fused_moe_kernel
+    from tilegym_amd.suites.flashinfer.ops import gemm_alpha_beta, ragged_block_scaled_bmm
+    from tilegym_amd.suites.unsloth.ops import w8a8_block_fp8_matmul
+
+    def names(f):
+        return list(inspect.signature(f).parameters)
+
+    assert names(matmul) == ["a", "b", "trans_a", "trans_b", "static_persistent", "use_tma", "kwargs"]
+    assert names(group_gemm) == ["group_A", "group_B", "static_persistent", "use_tma", "kwargs"]
+    assert names(w8a8_block_fp8_matmul) == ["A", "B", "As", "Bs", "block_size", "output_dtype"]
+    assert inspect.signature(w8a8_block_fp8_matmul).parameters["output_dtype"].default == torch.float32
+    assert names(gemm_alpha_beta) == ["a", "b", "c", "trans_a", "trans_b", "alpha", "beta", "num_sms"]
+    assert names(ragged_block_scaled_bmm) == ["a", "b", "a_scale", "b_scale", "m_indptr", "max_m",
+                                              "max_m_device", "transpose_a", "transpose_b", "out_dtype"]
+    assert names(invoke_fused_moe_kernel)[:12] == ["A", "B", "C", "A_scale", "B_scale", "topk_weights", "topk_ids",
+                                                   "sorted_token_ids", "expert_ids", "num_tokens_post_padded",
+                                                   "mul_routed_weight", "top_k"]
+
+
+def test_install_as_tilegym_aliases_import_paths():
+    tilegym_amd.install_as_tilegym()
+    import tilegym
+    from tilegym.suites import flashinfer, unsloth  # noqa: F401
+    from tilegym.ops.moe_interface import invoke_fused_moe_kernel  # noqa: F401
+
+    assert tilegym.ops.matmul is tilegym_amd.ops.matmul
+    assert unsloth.ops.w8a8_block_fp8_matmul is tilegym_amd.suites.unsloth.ops.w8a8_block_fp8_matmul
+    assert hasattr(flashinfer.ops, "ragged_block_scaled_bmm")
+
+
+def test_host_side_errors_mirror_the_reference():
+    from tilegym_amd.ops import group_gemm, matmul
+    from tilegym_amd.suites.flashinfer.ops import ragged_block_scaled_bmm
+    from tilegym_amd.suites.unsloth.ops import w8a8_block_fp8_matmul
+
+    a = torch.zeros(4, 128).to(FP8)
+    b = torch.zeros(8, 64).to(FP8)
+    with pytest.raises(AssertionError):
+        matmul(a, b, trans_b=True)                      # K mismatch asserts, as in the reference
+    with pytest.raises(NotImplementedError):
+        matmul(a.float(), a.float())                    # only e4m3 here
+    with pytest.raises(ValueError):
+        group_gemm([], [])
+    with pytest.raises(ValueError):
+        group_gemm([a], [a, a])
+    with pytest.raises(AssertionError):
+        w8a8_block_fp8_matmul(a, torch.zeros(8, 128).to(FP8), torch.ones(4, 2), torch.ones(1, 1))
+    with pytest.raises(AssertionError):
+        ragged_block_scaled_bmm(a, torch.zeros(2, 128, 128).to(FP8), None, torch.ones(2, 1, 1),
+                                torch.zeros(3, dtype=torch.int32), 4, transpose_b=False)
+    # a CPU tensor never silently computes: there is no CPU path
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        matmul(a, torch.zeros(8, 128).to(FP8), trans_b=True, out_dtype=torch.bfloat16)
+
+
+def test_moe_align_host_logic_matches_known_answer():
+    from tilegym_amd.ops import moe_align_block_size
+
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]]) - 1
+    s, e, post, cum, mx = moe_align_block_size(ids, 4, 4)
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert s.numel() == 24 and e.numel() == 6 and e[:4].tolist() == [0, 1, 2, 3]
+    assert int(post) == 16 and cum.tolist() == [0, 4, 8, 12, 16] and int(mx) == 3

@@ -1,0 +1,502 @@
+"""Parity of the HIP FP8 GEMM path (through the C ABI) with the CPU oracle.
+
+Tolerance (stated by the task): |out - ref| <= 2e-2 * sigma_ref + 2e-2 * |ref| with
+sigma_ref = std of the oracle output ("relative to output scale").  Kernel and oracle consume
+the same quantized bytes, so the real error is fp32 re-association plus one output rounding;
+TIGHT below is the much smaller bound we additionally expect (and flag when exceeded).
+"""
+
+import math
+
+import pytest
+import torch
+
+import tilegym_amd
+from oracle import reference as R
+from tilegym_amd import _lib, workloads as W
+from tilegym_amd.ops import group_gemm, matmul, moe_align_block_size
+from tilegym_amd.ops.moe_interface import invoke_fused_moe_kernel
+from tilegym_amd.suites.flashinfer.ops import gemm_alpha_beta, ragged_block_scaled_bmm
+from tilegym_amd.suites.unsloth.ops import w8a8_block_fp8_matmul
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+RTOL = ATOL = 2e-2
+TIGHT = 6e-3  # bf16 output rounding is 2^-9 relative
+
+
+def _g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def check(out, ref, tight=TIGHT, what=""):
+    ok, rep = R.compare_to_oracle(out, ref, RTOL, ATOL)
+    assert ok, f"{what}: outside tolerance: {rep}"
+    ok2, rep2 = R.compare_to_oracle(out, ref, tight, tight)
+    assert ok2, f"{what}: inside the stated tolerance but worse than expected: {rep2}"
+
+
+def fp8_randn(shape, g, std=1.0):
+    return (torch.randn(shape, generator=g) * std).clamp(-448, 448).to(FP8)
+
+
+def used(kernel_name):
+    cfg = _lib.last_config()
+    assert cfg["KERNEL_NAME"] == kernel_name, f"expected the {kernel_name} kernel, library chose {cfg}"
+    return cfg
+
+
+# ----------------------------------------------------------------------------- per-tensor, tiled
+@pytest.mark.parametrize("bm,bn", [(256, 256), (128, 128), (128, 256), (64, 128)])
+@pytest.mark.parametrize("M,N,K", [(256, 512, 1024), (200, 328, 384), (77, 130, 128), (513, 1000, 256)])
+def test_per_tensor_tiled_configs(device, bm, bn, M, N, K):
+    g = _g(M + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
+    sa, sb = torch.tensor([0.37]), torch.tensor([1.9])
+    ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "tiled", "BLOCK_M": bm, "BLOCK_N": bn, "SPLIT_K": 1})
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (bm, bn)
+    assert out.dtype == torch.bfloat16 and out.shape == (M, N)
+    check(out, ref, what=f"tiled {bm}x{bn} {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("split", [2, 3, 8])
+def test_per_tensor_tiled_split_k(device, split):
+    g = _g(split)
+    M, N, K = 200, 264, 2048
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g)
+    ref = R.ref_gemm_per_tensor(a, b, 0.01, 0.5, trans_b=True)
+    kc = {"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128, "SPLIT_K": split}
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.5, out_dtype=torch.bfloat16, kernel_configs=kc)
+    assert used("tiled")["SPLIT_K"] > 1
+    check(out, ref, what=f"split-K {split}")
+    # the reduction order is fixed: reruns are bit-identical, and the counters were left at zero
+    for _ in range(3):
+        again = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.5, out_dtype=torch.bfloat16, kernel_configs=kc)
+        assert torch.equal(again, out)
+
+
+# ----------------------------------------------------------------------------- skinny
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K,rg,split", [(1000, 512, 1, 1), (4096, 1024, 2, 2), (520, 2064, 4, 4), (256, 128, 1, 1)])
+def test_per_tensor_skinny(device, M, N, K, rg, split):
+    g = _g(M * 7 + N)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
+    ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "skinny", "ROW_GROUPS": rg, "SPLIT_K": split})
+    used("skinny")
+    check(out, ref, what=f"skinny M={M} N={N} K={K} rg={rg} split={split}")
+
+
+def test_skinny_auto_schedule_and_determinism(device):
+    case = W.llama_decode_case(16, "o")
+    ref = R.ref_gemm_per_tensor(case.a, case.b, case.scale_a, case.scale_b, trans_b=True)
+    d = case.to(device)
+    outs = [matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a, scale_b=d.scale_b, out_dtype=torch.bfloat16) for _ in range(4)]
+    cfg = used("skinny")
+    assert cfg["SPLIT_K"] > 1, "decode O-proj should use split-K to fill the chip"
+    check(outs[0], ref, what="decode o M=16")
+    assert all(torch.equal(outs[0], o) for o in outs[1:])
+
+
+# ----------------------------------------------------------------------------- layouts / fallbacks / dtypes
+def test_all_four_layouts_agree_with_the_oracle(device):
+    g = _g(21)
+    M, N, K = 96, 136, 256
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g)
+    at = a.view(torch.uint8).t().contiguous().view(FP8)
+    bt = b.view(torch.uint8).t().contiguous().view(FP8)
+    ref = R.ref_gemm_per_tensor(a, b, trans_b=True)
+    for (x, y, ta, tb) in [(a, b, False, True), (a, bt, False, False), (at, bt, True, False), (at, b, True, True)]:
+        out = matmul(x.to(device), y.to(device), trans_a=ta, trans_b=tb, out_dtype=torch.bfloat16)
+        check(out, ref, what=f"layout ta={ta} tb={tb}")
+    # (K,N) weights go through a K-contiguous copy in the workspace and then the MFMA kernels
+    matmul(a.to(device), bt.to(device), out_dtype=torch.bfloat16)
+    assert _lib.last_config()["KERNEL_NAME"] in ("tiled", "skinny")
+    matmul(at.to(device), b.to(device), trans_a=True, trans_b=True, out_dtype=torch.bfloat16)
+    used("fallback")
+
+
+@pytest.mark.parametrize("M,N,K", [(32, 64, 1023), (130, 70, 200), (5, 33, 17)])
+def test_odd_k_uses_the_fallback_and_is_correct(device, M, N, K):
+    """K=1023 is the case the reference skips (tests/ops/test_matmul.py:130-131)."""
+    g = _g(K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g)
+    ref = R.ref_gemm_per_tensor(a, b, 0.5, 2.0, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.5, scale_b=2.0, out_dtype=torch.bfloat16)
+    used("fallback")
+    check(out, ref, what=f"fallback K={K}")
+
+
+def test_k_tail_multiple_of_16_skinny(device):
+    g = _g(33)
+    M, N, K = 8, 256, 1040
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g)
+    ref = R.ref_gemm_per_tensor(a, b, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, out_dtype=torch.bfloat16)
+    used("skinny")
+    check(out, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_output_dtypes(device, dtype):
+    g = _g(4)
+    a, b = fp8_randn((150, 256), g, 0.1), fp8_randn((264, 256), g, 0.1)
+    for kernel in ("tiled", "fallback"):
+        out = matmul(a.to(device), b.to(device), trans_b=True, out_dtype=dtype, kernel_configs={"KERNEL": kernel})
+        assert out.dtype == dtype
+        ref = R.ref_gemm_per_tensor(a, b, trans_b=True, out_dtype=dtype)
+        check(out, ref, what=f"{kernel} {dtype}")
+    out = matmul(a[:9].contiguous().to(device), b.to(device), trans_b=True, out_dtype=dtype)
+    used("skinny")
+    check(out, R.ref_gemm_per_tensor(a[:9], b, trans_b=True, out_dtype=dtype))
+
+
+def test_reference_default_returns_input_dtype(device):
+    """Without keywords the op returns a.dtype like the reference (src/tilegym/ops/cutile/matmul.py:446);
+    oracle as in tests/ops/test_matmul.py:231-236 (matmul then cast to fp8), tolerance 1 there."""
+    g = _g(5)
+    a = (torch.randn(128, 256, generator=g) * 0.3).to(FP8)
+    b = (torch.randn(256, 192, generator=g) * 0.3).to(FP8)
+    out = matmul(a.to(device), b.to(device))
+    assert out.dtype == FP8 and out.shape == (128, 192)
+    ref = R.ref_gemm_per_tensor(a, b, out_dtype=torch.float32).to(FP8)
+    assert torch.allclose(out.float().cpu(), ref.float(), atol=1.0, rtol=1.0)
+    ok, rep = R.compare_to_oracle(out.float(), ref.float(), 0.13, 0.02)  # one e4m3 ulp
+    assert ok, rep
+
+
+def test_power_of_two_scales_are_exact(device):
+    g = _g(6)
+    a, b = fp8_randn((64, 512), g), fp8_randn((256, 512), g)
+    base = matmul(a.to(device), b.to(device), trans_b=True, out_dtype=torch.bfloat16)
+    scaled = matmul(a.to(device), b.to(device), trans_b=True, scale_a=4.0, scale_b=torch.tensor([0.125], device=device), out_dtype=torch.bfloat16)
+    assert torch.equal(scaled.float(), base.float() * 0.5)
+
+
+# ----------------------------------------------------------------------------- alpha / beta
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.5, 2.0)])
+@pytest.mark.parametrize("M,N,K,kernel", [(512, 512, 512, None), (16, 520, 256, None), (100, 72, 136, "fallback")])
+def test_gemm_alpha_beta(device, alpha, beta, M, N, K, kernel):
+    """Data recipe of tests/suites/flashinfer/test_flashinfer_gemm_alpha_beta.py:24-43 (rand in [0,1))."""
+    g = _g(7)
+    a = torch.rand(M, K, generator=g).to(torch.float16).to(FP8)
+    b = torch.rand(N, K, generator=g).to(torch.float16).to(FP8)
+    c0 = torch.rand(M, N, generator=g).to(torch.bfloat16)
+    ref = R.ref_gemm_alpha_beta(a, b, c0.clone(), False, True, alpha, beta)
+    c = c0.clone().to(device)
+    kw = {"kernel_configs": {"KERNEL": kernel}} if kernel else {}
+    out = tilegym_amd.backend._REGISTRY["flashinfer.gemm.gemm_alpha_beta"]["hip"](a.to(device), b.to(device), c, False, True, alpha, beta, **kw)
+    assert out.data_ptr() == c.data_ptr()
+    check(c, ref, what=f"alpha={alpha} beta={beta}")
+    c2 = c0.clone().to(device)
+    gemm_alpha_beta(a.to(device), b.to(device), c2, False, True, alpha, beta)
+    if kernel is None:
+        assert torch.equal(c2, c)
+
+
+# ----------------------------------------------------------------------------- block scaled
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 256, 256), (512, 1024, 512), (1024, 2048, 1024)])
+def test_block_scaled_reference_test_shapes(device, M, N, K):
+    """Shapes, data recipe and tolerance of Test_Unsloth_W8A8_FP8_Matmul (tests/suites/unsloth/test_fp8.py:193-231)."""
+    g = _g(42)
+    A = (torch.randn(M, K, generator=g) * 0.1).to(FP8)
+    B = (torch.randn(N, K, generator=g) * 0.1).to(FP8)
+    As = torch.rand(M, K // 128, generator=g) + 0.1
+    Bs = torch.rand(N // 128, K // 128, generator=g) + 0.1
+    ref = R.ref_w8a8_block_fp8_matmul(A, B, As, Bs, [128, 128])
+    out = w8a8_block_fp8_matmul(A.to(device), B.to(device), As.to(device), Bs.to(device), [128, 128])
+    used("tiled")
+    assert out.dtype == torch.float32
+    assert torch.allclose(out.cpu(), ref, rtol=5e-2, atol=5e-2)
+    check(out, ref, tight=1e-4, what="block-scaled f32")
+
+
+@pytest.mark.parametrize("bm,bn", [(128, 128), (128, 256), (64, 128)])
+@pytest.mark.parametrize("M,N,K", [(300, 640, 384), (129, 136, 256)])
+def test_block_scaled_tiled_configs_and_edges(device, bm, bn, M, N, K):
+    case = W.block_scaled_case(M, N, K, seed=M)
+    ref = R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, output_dtype=torch.bfloat16)
+    d = case.to(device)
+    out = tilegym_amd.backend._REGISTRY["unsloth.w8a8_block_fp8_matmul"]["hip"](
+        d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs={"KERNEL": "tiled", "BLOCK_M": bm, "BLOCK_N": bn})
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (bm, bn)
+    check(out, ref, what=f"block-scaled {bm}x{bn}")
+
+
+@pytest.mark.parametrize("M", [1, 16, 40, 64])
+@pytest.mark.parametrize("split", [1, 4])
+def test_block_scaled_skinny(device, M, split):
+    case = W.block_scaled_case(M, 640, 1024, seed=M)
+    ref = R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, output_dtype=torch.bfloat16)
+    d = case.to(device)
+    out = tilegym_amd.backend._REGISTRY["unsloth.w8a8_block_fp8_matmul"]["hip"](
+        d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs={"KERNEL": "skinny", "SPLIT_K": split})
+    used("skinny")
+    check(out, ref, what=f"block-scaled skinny M={M}")
+
+
+def test_block_scaled_batched_leading_dims_and_invariants(device):
+    g = _g(9)
+    A = fp8_randn((2, 3, 256), g)
+    B = fp8_randn((128, 256), g)
+    As = torch.rand(2, 3, 2, generator=g) + 0.5
+    Bs = torch.rand(1, 2, generator=g) + 0.5
+    out = w8a8_block_fp8_matmul(A.to(device), B.to(device), As.to(device), Bs.to(device), None, torch.bfloat16)
+    assert out.shape == (2, 3, 128)
+    check(out, R.ref_w8a8_block_fp8_matmul(A, B, As, Bs, None, torch.bfloat16))
+    # all-equal block scales == per-tensor scales (bit-exact)
+    A2, B2 = fp8_randn((200, 512), g), fp8_randn((256, 512), g)
+    blk = w8a8_block_fp8_matmul(A2.to(device), B2.to(device), torch.full((200, 4), 0.25, device=device),
+                                torch.full((2, 4), 2.0, device=device), None, torch.float32)
+    pt = matmul(A2.to(device), B2.to(device), trans_b=True, scale_a=0.25, scale_b=2.0, out_dtype=torch.float32,
+                kernel_configs={"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128})
+    check(blk, pt.cpu(), tight=1e-5)
+    # doubling every activation scale doubles the result exactly
+    case = W.block_scaled_case(130, 256, 512, seed=3).to(device)
+    o1 = w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16)
+    o2 = w8a8_block_fp8_matmul(case.a, case.b, case.scale_a * 2, case.scale_b, None, torch.bfloat16)
+    assert torch.equal(o2.float(), o1.float() * 2)
+
+
+# ----------------------------------------------------------------------------- grouped (ragged)
+def _ragged_inputs(sizes, N, K, seed, total_extra=0):
+    g = _g(seed)
+    Q = len(sizes)
+    total = sum(sizes) + total_extra
+    ptr = torch.zeros(Q + 1, dtype=torch.int32)
+    ptr[1:] = torch.cumsum(torch.tensor(sizes), 0)
+    a = fp8_randn((total, K), g)
+    b = fp8_randn((Q, N, K), g, 0.5)
+    a_s = torch.rand(total, K // 128, generator=g) * 1e-2 + 1e-3
+    b_s = torch.rand(Q, -(-N // 128), K // 128, generator=g) * 1e-2 + 1e-3
+    return a, b, a_s, b_s, ptr
+
+
+@pytest.mark.parametrize("groups,m", [(4, 128), (16, 128), (4, 512)])
+@pytest.mark.parametrize("n,k", [(2048, 2048)])
+def test_ragged_reference_test_shapes(device, groups, m, n, k):
+    """Group counts / segment sizes of Test_FlashInfer_RaggedBlockScaledBMM
+    (tests/suites/flashinfer/test_flashinfer_ragged_block_scaled_bmm.py:216-223); that test allows atol=rtol=1."""
+    a, b, a_s, b_s, ptr = _ragged_inputs([m] * groups, n, k, groups + m)
+    ref = R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr)
+    out = ragged_block_scaled_bmm(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), m)
+    used("tiled")
+    assert out.dtype == torch.bfloat16
+    assert torch.allclose(out.float().cpu(), ref.float(), atol=1.0, rtol=1.0)
+    check(out, ref, what="ragged aligned")
+
+
+@pytest.mark.parametrize("bm,bn", [(128, 128), (128, 256), (64, 128)])
+def test_ragged_unaligned_empty_and_single_experts(device, bm, bn):
+    sizes = [5, 0, 131, 64, 0, 0, 257, 1, 77]
+    a, b, a_s, b_s, ptr = _ragged_inputs(sizes, 392, 256, 17, total_extra=6)
+    ref = R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr)
+    impl = tilegym_amd.backend._REGISTRY["flashinfer.gemm.ragged_block_scaled_bmm"]["hip"]
+    out = impl(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), max(sizes),
+               kernel_configs={"BLOCK_M": bm, "BLOCK_N": bn}, zero_init=True)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (bm, bn)
+    check(out, ref, what=f"ragged unaligned {bm}x{bn}")
+    assert torch.equal(out[sum(sizes):].cpu().float(), torch.zeros(6, 392))  # rows of no segment untouched
+    # single expert == dense
+    a1, b1, as1, bs1, p1 = _ragged_inputs([150], 256, 384, 3)
+    o1 = impl(a1.to(device), b1.to(device), as1.to(device), bs1.to(device), p1.to(device), 150, kernel_configs={"BLOCK_M": bm, "BLOCK_N": bn})
+    dense = w8a8_block_fp8_matmul(a1.to(device), b1[0].to(device), as1.to(device), bs1[0].to(device), None, torch.bfloat16)
+    check(o1, dense.cpu(), tight=1e-5)
+    # no activation scales
+    o2 = impl(a.to(device), b.to(device), None, b_s.to(device), ptr.to(device), max(sizes), zero_init=True)
+    check(o2, R.ref_ragged_block_scaled_bmm(a, b, None, b_s, ptr))
+
+
+def test_ragged_many_experts_and_permutation(device):
+    g = _g(31)
+    sizes = torch.randint(0, 40, (150,), generator=g).tolist()  # > 64 experts: multi-pass expert search
+    a, b, a_s, b_s, ptr = _ragged_inputs(sizes, 128, 128, 5)
+    ref = R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr)
+    out = ragged_block_scaled_bmm(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), max(sizes))
+    check(out, ref, what="150 experts")
+    again = ragged_block_scaled_bmm(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), max(sizes))
+    assert torch.equal(out, again)
+
+
+def test_ragged_fallback_for_odd_k(device):
+    g = _g(8)
+    sizes = [3, 0, 9]
+    Q, N, K = 3, 40, 200
+    ptr = torch.tensor([0, 3, 3, 12], dtype=torch.int32)
+    a, b = fp8_randn((12, K), g), fp8_randn((Q, N, K), g)
+    a_s = torch.rand(12, 2, generator=g) + 0.1
+    b_s = torch.rand(Q, 1, 2, generator=g) + 0.1
+    ref = R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr)
+    L = _lib
+    c = torch.empty(12, N, dtype=torch.bfloat16, device=device)
+    L.fp8_ragged_gemm(c, a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device))
+    used("fallback")
+    check(c, ref)
+
+
+# ----------------------------------------------------------------------------- MoE token gather
+@pytest.mark.parametrize("block_m", [64, 128, 16])
+@pytest.mark.parametrize("mul_w", [False, True])
+def test_moe_gather_gemm(device, block_m, mul_w):
+    g = _g(block_m)
+    T, E, N, K, top_k = 70, 8, 264, 256, 2
+    A = fp8_randn((T, K), g)
+    B = fp8_randn((E, N, K), g, 0.5)
+    a_s = torch.rand(T, K // 128, generator=g) + 0.1
+    b_s = torch.rand(E, -(-N // 128), K // 128, generator=g) + 0.1
+    w, ids = W.moe_routing(T, E, top_k, seed=1)
+    ids[ids == 3] = 2  # an expert without tokens
+    ref = R.ref_fused_moe_gemm(A, B, a_s, b_s, w, ids, mul_w, top_k)
+    sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids.to(device), block_m, E)
+    rs, re_, rpost, _, _ = R.moe_align_block_size_ref(ids, block_m, E)
+    assert torch.equal(sorted_ids.cpu(), rs) and int(post) == int(rpost)
+    assert torch.equal(expert_ids.cpu()[: int(rpost) // block_m], re_[: int(rpost) // block_m])
+    C = torch.zeros(T, top_k, N, dtype=torch.bfloat16, device=device)
+    ret = invoke_fused_moe_kernel(A.to(device), B.to(device), C, a_s.to(device), b_s.to(device), w.to(device), ids.to(device),
+                                  sorted_ids, expert_ids, post, mul_w, top_k, {"BLOCK_SIZE_M": block_m},
+                                  use_fp8_w8a8=True, block_shape=[128, 128])
+    assert ret is None
+    used("tiled" if block_m % 64 == 0 else "fallback")
+    check(C, ref, what=f"moe gather block_m={block_m} mul={mul_w}")
+
+
+def test_moe_fc2_shape_top_k_1(device):
+    """Second MoE GEMM: activations already expanded per slot (top_k = 1), routed weight applied
+    (src/tilegym/ops/moe_interface.py:290-307)."""
+    g = _g(77)
+    T, E, N, K, top_k = 40, 4, 128, 384, 2
+    w, ids = W.moe_routing(T, E, top_k, seed=2)
+    A = fp8_randn((T * top_k, K), g)
+    B = fp8_randn((E, N, K), g, 0.5)
+    a_s = torch.rand(T * top_k, 3, generator=g) + 0.1
+    b_s = torch.rand(E, 1, 3, generator=g) + 0.1
+    ref = R.ref_fused_moe_gemm(A, B, a_s, b_s, w, ids, True, 1)
+    sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids.to(device), 64, E)
+    C = torch.zeros(T, top_k, N, dtype=torch.bfloat16, device=device)
+    invoke_fused_moe_kernel(A.to(device), B.to(device), C, a_s.to(device), b_s.to(device), w.to(device), ids.to(device),
+                            sorted_ids, expert_ids, post, True, 1, {"BLOCK_SIZE_M": 64})
+    check(C, ref, what="moe fc2")
+
+
+# ----------------------------------------------------------------------------- group_gemm (list form)
+def test_group_gemm_list_form(device):
+    g = _g(12)
+    shapes = [(64, 128, 256), (130, 72, 128), (8, 264, 512)]
+    As = [fp8_randn((m, k), g) for m, n, k in shapes]
+    Bs = [fp8_randn((k, n), g) for m, n, k in shapes]
+    outs = group_gemm([x.to(device) for x in As], [x.to(device) for x in Bs], out_dtype=torch.bfloat16)
+    refs = R.ref_group_gemm(As, Bs, out_dtype=torch.bfloat16)
+    for o, r in zip(outs, refs):
+        check(o, r)
+    Bt = [b.view(torch.uint8).t().contiguous().view(FP8) for b in Bs]
+    outs_t = group_gemm([x.to(device) for x in As], [x.to(device) for x in Bt], transpose_b=True, out_dtype=torch.bfloat16,
+                        scales_a=[0.5] * 3, scales_b=[torch.tensor([2.0], device=device)] * 3)
+    for o, r in zip(outs_t, refs):
+        check(o, r)
+    default = group_gemm([As[0].to(device)], [Bs[0].to(device)])
+    assert default[0].dtype == FP8
+
+
+# ----------------------------------------------------------------------------- BASELINE configs at full size
+def _rows_subset(M, count, seed=0):
+    if M <= count:
+        return torch.arange(M)
+    idx = torch.randperm(M, generator=_g(seed))[:count].sort().values
+    idx[0], idx[-1] = 0, M - 1
+    return idx
+
+
+def test_config1_full(device):
+    for trans_b in (True, False):
+        case = W.config1(trans_b=trans_b)
+        ref = R.ref_gemm_per_tensor(case.a, case.b, case.scale_a, case.scale_b, trans_b=trans_b)
+        d = case.to(device)
+        out = matmul(d.a, d.b, trans_b=trans_b, scale_a=d.scale_a, scale_b=d.scale_b, out_dtype=torch.bfloat16)
+        assert _lib.last_config()["KERNEL_NAME"] == "tiled"
+        check(out, ref, what=f"config 1 trans_b={trans_b}")
+
+
+@pytest.mark.parametrize("proj", list(W.LLAMA_SHAPES))
+def test_config2_llama_decode_full(device, proj):
+    N, K = W.LLAMA_SHAPES[proj]
+    big = W.llama_decode_case(64, proj)
+    bd = big.b.to(device)
+    bref = R.fp8_to_f32(big.b) * big.scale_b
+    for M in W.DECODE_M:
+        a = big.a[:M].contiguous()
+        ref = ((R.fp8_to_f32(a) * big.scale_a) @ bref.t()).to(torch.bfloat16)
+        out = matmul(a.to(device), bd, trans_b=True, scale_a=big.scale_a.to(device), scale_b=big.scale_b.to(device), out_dtype=torch.bfloat16)
+        used("skinny")
+        check(out, ref, what=f"config 2 {proj} M={M}")
+
+
+@pytest.mark.parametrize("proj", list(W.LLAMA_SHAPES))
+def test_config3_llama_prefill_sampled_rows(device, proj):
+    """Full-size launch; the oracle is evaluated on 96 sampled activation rows (each output row
+    depends on its own activation row only) and on linearity across the whole output."""
+    case = W.llama_prefill_case(proj)
+    d = case.to(device)
+    out = matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a, scale_b=d.scale_b, out_dtype=torch.bfloat16)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (256, 256)
+    rows = _rows_subset(case.M, 96)
+    ref = R.ref_gemm_per_tensor(case.a[rows], case.b, case.scale_a, case.scale_b, trans_b=True)
+    check(out[rows.to(device)], ref, what=f"config 3 {proj}")
+    assert torch.isfinite(out.float()).all()
+    # doubling a scale doubles every element exactly (bf16, power of two)
+    out2 = matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a * 2, scale_b=d.scale_b, out_dtype=torch.bfloat16)
+    assert torch.equal(out2.float(), out.float() * 2)
+
+
+@pytest.mark.parametrize("N,K", W.BLOCK_SCALED_SHAPES)
+def test_config4_block_scaled_full(device, N, K):
+    big = W.block_scaled_case(4096, N, K)
+    d = big.to(device)
+    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16)
+    used("tiled")
+    rows = _rows_subset(4096, 64)
+    ref = R.ref_w8a8_block_fp8_matmul(big.a[rows], big.b, big.scale_a[rows], big.scale_b, None, torch.bfloat16)
+    check(out[rows.to(device)], ref, what=f"config 4 M=4096 {N}x{K}")
+    out16 = w8a8_block_fp8_matmul(d.a[:16].contiguous(), d.b, d.scale_a[:16].contiguous(), d.scale_b, None, torch.bfloat16)
+    used("skinny")
+    ref16 = R.ref_w8a8_block_fp8_matmul(big.a[:16], big.b, big.scale_a[:16], big.scale_b, None, torch.bfloat16)
+    check(out16, ref16, what=f"config 4 M=16 {N}x{K}")
+
+
+@pytest.mark.parametrize("which", ["gate_up", "down"])
+def test_config5_moe_grouped_full(device, which):
+    case = W.moe_grouped_case(which)
+    d = case.to(device)
+    sizes = (case.m_indptr[1:] - case.m_indptr[:-1])
+    assert int(case.m_indptr[-1]) == 4096 * 6 and sizes.min() != sizes.max()  # uneven experts
+    out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, int(sizes.max()))
+    used("tiled")
+    # per-expert reference GEMMs on a subset of experts (smallest, largest, first, last + 4 others)
+    experts = sorted({0, 63, int(sizes.argmin()), int(sizes.argmax()), 7, 21, 38, 50})
+    for e in experts:
+        lo, hi = int(case.m_indptr[e]), int(case.m_indptr[e + 1])
+        ref = R.ref_w8a8_block_fp8_matmul(case.a[lo:hi], case.b[e], case.a_scale[lo:hi], case.b_scale[e], None, torch.bfloat16)
+        check(out[lo:hi], ref, what=f"config 5 {which} expert {e}")
+    assert torch.isfinite(out.float()).all()
+    # the token-gather form of the same GEMM gives the same numbers slot by slot
+    if which == "gate_up":
+        ids, order, k = case.extra["topk_ids"], case.extra["order"], case.extra["top_k"]
+        T = ids.shape[0]
+        x_rows = torch.empty(T, case.a.shape[1], dtype=torch.uint8)
+        x_rows[order // k] = case.a.view(torch.uint8)
+        xs = torch.empty(T, case.a_scale.shape[1])
+        xs[order // k] = case.a_scale
+        sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids.to(device), 128, 64)
+        C = torch.zeros(T, k, case.b.shape[1], dtype=torch.bfloat16, device=device)
+        invoke_fused_moe_kernel(x_rows.view(FP8).to(device), d.b, C, xs.to(device), d.b_scale, None, ids.to(device),
+                                sorted_ids, expert_ids, post, False, k, {"BLOCK_SIZE_M": 128})
+        used("tiled")
+        gathered = C.view(T * k, -1)[order.to(device)]
+        assert torch.equal(gathered, out)

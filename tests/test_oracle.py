@@ -1,0 +1,273 @@
+"""Pins of the CPU oracle (oracle/reference.py, oracle/fp8_oracle.c): closed forms, exact integer
+cases, brute force on tiny inputs, invariants, and the reference's one known-answer vector."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as C
+from oracle import reference as R
+
+FP8 = torch.float8_e4m3fn
+
+
+def _g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ---------------------------------------------------------------- codec
+def test_decode_table_matches_torch_view_and_closed_form():
+    torch_tab = torch.arange(256, dtype=torch.uint8).view(FP8).float().numpy()
+    for tab in (R.e4m3fn_decode_table(), C.decode_table()):
+        assert np.array_equal(np.isnan(tab), np.isnan(torch_tab))
+        ok = ~np.isnan(tab)
+        assert np.array_equal(tab[ok], torch_tab[ok])
+    tab = R.e4m3fn_decode_table()
+    assert tab[0x7E] == 448.0 and tab[0xFE] == -448.0          # max finite
+    assert tab[0x01] == 2.0 ** -9 and tab[0x08] == 2.0 ** -6   # min subnormal, min normal
+    assert np.isnan(tab[0x7F]) and np.isnan(tab[0xFF])
+    assert tab[0x38] == 1.0 and tab[0x40] == 2.0 and tab[0x3C] == 1.5
+
+
+def test_encode_rne_matches_torch_cast_dense_grid():
+    x = torch.cat([torch.linspace(-448, 448, 100001), torch.linspace(-0.05, 0.05, 20001),
+                   torch.tensor([0.0, -0.0, 2.0 ** -10, 3 * 2.0 ** -10, 2.0 ** -9, 447.9, 448.0])])
+    want = x.to(FP8).view(torch.uint8).numpy()
+    got = R.e4m3fn_encode_rne(x.numpy())
+    assert np.array_equal(got, want)
+    L = C.lib()
+    sub = x[::53]
+    got_c = np.array([L.orc_e4m3_encode(float(v)) for v in sub.tolist()], dtype=np.uint8)
+    assert np.array_equal(got_c, sub.to(FP8).view(torch.uint8).numpy())
+
+
+def test_bf16_rounding_matches_torch():
+    x = torch.randn(5000, generator=_g(3)) * 100
+    want = x.to(torch.bfloat16).view(torch.int16).numpy().astype(np.uint16)
+    L = C.lib()
+    got = np.array([L.orc_bf16_bits(float(v)) for v in x.tolist()], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- quantizers
+def test_quantizers_scale_rule_and_zero_blocks():
+    x = torch.randn(7, 256, generator=_g(0))
+    x[2, :128] = 0
+    q, s = R.quantize_act_1x128(x)                 # unsloth rule
+    assert s.shape == (7, 2) and s[2, 0] == 1.0
+    assert torch.equal(s[0, 0], x[0, :128].abs().max() / 448.0)
+    assert R.fp8_to_f32(q).abs().max() == 448.0    # every non-zero block hits +-448
+    q2, s2 = R.quantize_act_1x128(x, eps=1e-10)    # flashinfer rule
+    assert s2[2, 0] == pytest.approx(1e-10 / 448.0)
+    deq = R.fp8_to_f32(q) * s.repeat_interleave(128, 1)
+    assert (deq - x).abs().max() <= x.abs().max() * 2 ** -4   # e4m3 has 3 mantissa bits
+    w = torch.randn(200, 300, generator=_g(1)) * 0.02
+    qw, sw = R.quantize_weight_128x128(w)
+    assert sw.shape == (2, 3)
+    assert torch.equal(sw[1, 2], w[128:, 256:].abs().max() / 448.0)
+    back = R.weight_dequant(qw, sw, 128, torch.float32)
+    assert (back - w).abs().max() <= w.abs().max() * 2 ** -4
+    qt, st = R.quantize_per_tensor(w)
+    assert st.shape == (1,) and torch.equal(st[0], w.abs().max() / 448.0)
+
+
+# ---------------------------------------------------------------- GEMMs
+def _int_fp8(shape, g, lo=-8, hi=9):
+    return torch.randint(lo, hi, shape, generator=g).float().to(FP8)
+
+
+def test_per_tensor_gemm_exact_integers_and_layouts():
+    g = _g(5)
+    M, N, K = 5, 7, 96
+    a, b = _int_fp8((M, K), g), _int_fp8((N, K), g)
+    want = a.float().long() @ b.float().long().t()          # exact int64
+    got = R.ref_gemm_per_tensor(a, b, trans_b=True, out_dtype=torch.float32)
+    assert torch.equal(got.long(), want)
+    # the same product through the other three layouts
+    bt = b.view(torch.uint8).t().contiguous().view(FP8)      # (K,N)
+    at = a.view(torch.uint8).t().contiguous().view(FP8)      # (K,M)
+    assert torch.equal(R.ref_gemm_per_tensor(a, bt, out_dtype=torch.float32).long(), want)
+    assert torch.equal(R.ref_gemm_per_tensor(at, bt, trans_a=True, out_dtype=torch.float32).long(), want)
+    assert torch.equal(R.ref_gemm_per_tensor(at, b, trans_a=True, trans_b=True, out_dtype=torch.float32).long(), want)
+    # power-of-two scales are exact
+    got2 = R.ref_gemm_per_tensor(a, b, 0.5, torch.tensor([4.0]), trans_b=True, out_dtype=torch.float32)
+    assert torch.equal(got2, got * 2.0)
+    # C restatement
+    c = C.gemm_per_tensor(R.fp8_bytes(a), R.fp8_bytes(b), 0.5, 4.0)
+    assert np.array_equal(c, got2.numpy())
+
+
+def test_alpha_beta_is_linear_in_the_per_tensor_oracle():
+    g = _g(6)
+    a, b = _int_fp8((4, 64), g), _int_fp8((6, 64), g)
+    c0 = torch.randn(4, 6, generator=g).to(torch.bfloat16)
+    base = R.ref_gemm_per_tensor(a, b, trans_b=True, out_dtype=torch.float32)
+    got = R.ref_gemm_alpha_beta(a, b, c0.clone(), False, True, 1.5, 2.0)
+    assert got.dtype == torch.bfloat16
+    assert torch.equal(got, (1.5 * base + 2.0 * c0.float()).to(torch.bfloat16))
+    assert torch.equal(R.ref_gemm_alpha_beta(a, b, c0.clone(), False, True, 1.0, 0.0), base.to(torch.bfloat16))
+
+
+def _loop_block_gemm(A, B, As, Bs, bn, bk):
+    """The reference test's own formulation: per-element loops (tests/suites/unsloth/test_fp8.py:159-191)."""
+    Af, Bf = R.fp8_to_f32(A), R.fp8_to_f32(B)
+    M, K = Af.shape
+    N = Bf.shape[0]
+    A_deq = torch.zeros(M, K)
+    for m in range(M):
+        for k0 in range(0, K, bk):
+            A_deq[m, k0:k0 + bk] = Af[m, k0:k0 + bk] * As[m, k0 // bk]
+    B_deq = torch.zeros(N, K)
+    for n0 in range(0, N, bn):
+        for k0 in range(0, K, bk):
+            B_deq[n0:n0 + bn, k0:k0 + bk] = Bf[n0:n0 + bn, k0:k0 + bk] * Bs[n0 // bn, k0 // bk]
+    return A_deq @ B_deq.t()
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 130, 256), (5, 256, 384), (2, 100, 200)])
+def test_block_scaled_oracle_against_loops_and_c(M, N, K):
+    g = _g(7)
+    A = (torch.randn(M, K, generator=g) * 0.1).to(FP8)
+    B = (torch.randn(N, K, generator=g) * 0.1).to(FP8)
+    As = torch.rand(M, -(-K // 128), generator=g) + 0.1
+    Bs = torch.rand(-(-N // 128), -(-K // 128), generator=g) + 0.1
+    want = _loop_block_gemm(A, B, As, Bs, 128, 128)
+    got = R.ref_w8a8_block_fp8_matmul(A, B, As, Bs)
+    assert torch.allclose(got, want, rtol=1e-6, atol=1e-6)
+    c = C.gemm_block_scaled(R.fp8_bytes(A), R.fp8_bytes(B), As.numpy(), Bs.numpy())
+    assert np.allclose(c, want.numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_block_scaled_invariants():
+    g = _g(8)
+    M, N, K = 4, 256, 256
+    A, B = _int_fp8((M, K), g, -4, 5), _int_fp8((N, K), g, -4, 5)
+    ones_a, ones_b = torch.ones(M, 2), torch.ones(2, 2)
+    exact = (A.float().long() @ B.float().long().t()).float()
+    # all-ones scales == unscaled GEMM (exact for small integers)
+    assert torch.equal(R.ref_w8a8_block_fp8_matmul(A, B, ones_a, ones_b), exact)
+    # all blocks equal == per-tensor
+    assert torch.equal(R.ref_w8a8_block_fp8_matmul(A, B, ones_a * 0.25, ones_b * 2.0),
+                       R.ref_gemm_per_tensor(A, B, 0.25, 2.0, trans_b=True, out_dtype=torch.float32))
+    # scaling one K block of As by 2^k scales only that block's contribution
+    As = ones_a.clone(); As[:, 1] = 4.0
+    part1 = (A[:, 128:].float().long() @ B[:, 128:].float().long().t()).float()
+    assert torch.equal(R.ref_w8a8_block_fp8_matmul(A, B, As, ones_b), exact + 3.0 * part1)
+    # one N block of Bs
+    Bs = ones_b.clone(); Bs[1, :] = 0.5
+    got = R.ref_w8a8_block_fp8_matmul(A, B, ones_a, Bs)
+    assert torch.equal(got[:, :128], exact[:, :128]) and torch.equal(got[:, 128:], 0.5 * exact[:, 128:])
+
+
+def test_ragged_oracle_properties():
+    g = _g(9)
+    Q, N, K = 4, 128, 256
+    sizes = [5, 0, 9, 3]
+    ptr = torch.tensor([0, 5, 5, 14, 17], dtype=torch.int32)
+    total = 20  # three rows belong to no segment
+    a = (torch.randn(total, K, generator=g) * 0.5).to(FP8)
+    b = (torch.randn(Q, N, K, generator=g) * 0.5).to(FP8)
+    a_s = torch.rand(total, 2, generator=g) + 0.1
+    b_s = torch.rand(Q, 1, 2, generator=g) + 0.1
+    out = R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr, out_dtype=torch.float32)
+    assert torch.equal(out[17:], torch.zeros(3, N))
+    for q in range(Q):
+        lo, hi = int(ptr[q]), int(ptr[q + 1])
+        if hi > lo:
+            dense = R.ref_w8a8_block_fp8_matmul(a[lo:hi], b[q], a_s[lo:hi], b_s[q])
+            assert torch.equal(out[lo:hi], dense)
+    # permuting experts permutes the output segments
+    perm = [2, 0, 3, 1]
+    segs = [(int(ptr[q]), int(ptr[q + 1])) for q in perm]
+    a_p = torch.cat([a[lo:hi] for lo, hi in segs] + [a[17:]])
+    as_p = torch.cat([a_s[lo:hi] for lo, hi in segs] + [a_s[17:]])
+    ptr_p = torch.tensor([0] + list(np.cumsum([sizes[q] for q in perm])), dtype=torch.int32)
+    out_p = R.ref_ragged_block_scaled_bmm(a_p, b[perm], as_p, b_s[perm], ptr_p, out_dtype=torch.float32)
+    assert torch.equal(out_p[:17], torch.cat([out[lo:hi] for lo, hi in segs]))
+    # C restatement
+    c = C.gemm_ragged(R.fp8_bytes(a), R.fp8_bytes(b), a_s.numpy(), b_s.numpy(), ptr.numpy())
+    assert np.allclose(c, out.numpy(), rtol=1e-5, atol=1e-5)
+    # a_scale=None means ones
+    o1 = R.ref_ragged_block_scaled_bmm(a, b, None, b_s, ptr, out_dtype=torch.float32)
+    o2 = R.ref_ragged_block_scaled_bmm(a, b, torch.ones(total, 2), b_s, ptr, out_dtype=torch.float32)
+    assert torch.equal(o1, o2)
+
+
+def test_group_gemm_oracle_is_a_list_of_gemms():
+    g = _g(10)
+    As = [_int_fp8((3, 32), g), _int_fp8((5, 64), g)]
+    Bs = [_int_fp8((32, 4), g), _int_fp8((64, 6), g)]
+    outs = R.ref_group_gemm(As, Bs, out_dtype=torch.float32)
+    for A, B, o in zip(As, Bs, outs):
+        assert torch.equal(o.long(), A.float().long() @ B.float().long())
+    Bt = [b.view(torch.uint8).t().contiguous().view(FP8) for b in Bs]
+    outs_t = R.ref_group_gemm(As, Bt, transpose_b=True, out_dtype=torch.float32)
+    assert all(torch.equal(x, y) for x, y in zip(outs, outs_t))
+
+
+# ---------------------------------------------------------------- MoE
+def test_moe_align_known_answer_vector():
+    """Worked example of src/tilegym/ops/cutile/moe_align_block.py:234-250 (expert labels 1..4 there;
+    0-based here)."""
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]]) - 1
+    want_sorted = [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    s, e, post, cum, mx = R.moe_align_block_size_ref(ids, 4, 4)
+    assert s[:16].tolist() == want_sorted and s[16:].tolist() == [12] * 8
+    assert s.numel() == 12 + 4 * 3 and e.numel() == 6
+    assert e[:4].tolist() == [0, 1, 2, 3]
+    assert int(post) == 16 and cum.tolist() == [0, 4, 8, 12, 16] and int(mx) == 3
+    cs, ce, cpost, ccum, cmx = C.moe_align(ids.numpy(), 4, 4)
+    assert cs[:16].tolist() == want_sorted and cpost == 16 and ccum.tolist() == [0, 4, 8, 12, 16] and cmx == 3
+    assert ce[:4].tolist() == [0, 1, 2, 3]
+
+
+def test_moe_align_random_properties():
+    g = _g(11)
+    E, bs = 8, 16
+    ids = torch.randint(0, E, (50, 3), generator=g)
+    ids[ids == 5] = 4  # expert 5 gets no tokens
+    s, e, post, cum, mx = R.moe_align_block_size_ref(ids, bs, E)
+    flat = ids.reshape(-1)
+    post = int(post)
+    assert post % bs == 0 and cum[-1] == post
+    valid = s[:post][s[:post] < flat.numel()]
+    assert sorted(valid.tolist()) == list(range(flat.numel()))          # a permutation of all slots
+    for blk in range(post // bs):
+        rows = s[blk * bs:(blk + 1) * bs]
+        rows = rows[rows < flat.numel()]
+        assert (flat[rows.long()] == e[blk]).all()                      # one expert per block
+        assert rows.tolist() == sorted(rows.tolist())                   # stable
+    assert int(mx) == int(torch.bincount(flat, minlength=E).max())
+    cs, ce, cpost, ccum, cmx = C.moe_align(ids.numpy(), bs, E)
+    assert np.array_equal(cs, s.numpy()) and cpost == post and np.array_equal(ccum, cum.numpy())
+    assert np.array_equal(ce[:post // bs], e[:post // bs].numpy())
+
+
+def test_fused_moe_gemm_oracle_against_token_loops():
+    g = _g(12)
+    T, E, N, K, topk = 6, 4, 128, 256, 2
+    A = (torch.randn(T, K, generator=g) * 0.3).to(FP8)
+    B = (torch.randn(E, N, K, generator=g) * 0.3).to(FP8)
+    a_s = torch.rand(T, 2, generator=g) + 0.1
+    b_s = torch.rand(E, 1, 2, generator=g) + 0.1
+    ids = torch.randint(0, E, (T, topk), generator=g)
+    w = torch.rand(T, topk, generator=g)
+    got = R.ref_fused_moe_gemm(A, B, a_s, b_s, w, ids, True, topk, out_dtype=torch.float32)
+    for t in range(T):
+        for j in range(topk):
+            e = int(ids[t, j])
+            a_deq = R.fp8_to_f32(A[t]) * a_s[t].repeat_interleave(128)
+            b_deq = R.fp8_to_f32(B[e]) * b_s[e].repeat_interleave(128, 0).repeat_interleave(128, 1)
+            want = (b_deq @ a_deq) * w[t, j]
+            assert torch.allclose(got[t, j], want, rtol=1e-5, atol=1e-5)
+
+
+def test_compare_to_oracle_flags_errors():
+    ref = torch.randn(64, 64, generator=_g(13))
+    ok, _ = R.compare_to_oracle(ref.to(torch.bfloat16), ref)
+    assert ok
+    bad = ref.clone(); bad[3, 4] += 1.0
+    ok, rep = R.compare_to_oracle(bad, ref)
+    assert not ok and rep["matched"] < 1.0
+    nan = ref.clone(); nan[0, 0] = float("nan")
+    assert not R.compare_to_oracle(nan, ref)[0]
