@@ -22,7 +22,7 @@ from tilegym_amd.suites.unsloth.ops import w8a8_block_fp8_matmul
 pytestmark = pytest.mark.gpu
 FP8 = torch.float8_e4m3fn
 RTOL = ATOL = 2e-2
-TIGHT = 6e-3  # bf16 output rounding is 2^-9 relative
+TIGHT = 8.5e-3  # one bf16 ulp is at most 2^-7 = 7.8e-3 relative (a rounding tie may flip one ulp)
 
 
 def _g(seed):
