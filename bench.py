@@ -142,7 +142,7 @@ def measure_shape(runner, steps, warmup, stream, use_graph):
     return {
         "name": case.name,
         "kernel": cfg["KERNEL_NAME"], "block_m": cfg["BLOCK_M"], "block_n": cfg["BLOCK_N"],
-        "split_k": cfg["SPLIT_K"], "row_groups": cfg["ROW_GROUPS"],
+        "split_k": cfg["SPLIT_K"], "row_groups": cfg["ROW_GROUPS"], "waves": cfg["WAVES"],
         "us": round(us, 3), "launches": launches,
         "tflops": round(flops / us * 1e-6, 2), "gbs": round(nbytes / us * 1e-3, 1),
         "flops": flops, "bytes": nbytes,

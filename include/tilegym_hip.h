@@ -64,6 +64,7 @@ enum {
     TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (128/256)               */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
     TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4)         */
+    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16)       */
     TG_CFG_COUNT = 8
 };
 
@@ -83,11 +84,11 @@ enum {
  *     scale_a (M, ceil(K/128)) and scale_b (ceil(N/128), ceil(K/128)) -> block scaled:
  *        C[m,n] = sum_kb scale_a[m,kb] * scale_b[n/128,kb] * sum_{k in kb} A[m,k] * B[n,k]
  *     (both must be of the same kind; block form requires the NT layout.)
- * workspace: NULL, or a u8/any-dtype 1-D buffer of at least tg_fp8_gemm_workspace_bytes()
- *     bytes that was ZERO-FILLED when allocated; the library leaves its counter region
- *     zeroed on return, so one buffer can serve every later call on the same stream.
- *     Calls that share a workspace must not overlap in time.  Without a workspace the
- *     split-K schedules are not used.
+ * workspace: NULL, or a 16-byte-aligned scratch buffer (any dtype, contents irrelevant) of at
+ *     least tg_fp8_gemm_workspace_bytes() bytes.  It holds split-K partial sums and, for
+ *     (K,N) weights, a K-contiguous copy of b.  Calls that share a workspace must not overlap
+ *     in time (calls on one stream never do).  Without a workspace the split-K schedules and
+ *     the (K,N) fast path are not used.
  */
 int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
                     const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
@@ -139,7 +140,7 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
                         const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream);
 
 /* The schedule the most recent GEMM call on this host thread chose: fills out[0..n) with the
- * TG_CFG_* slots (kernel, BLOCK_M, BLOCK_N, SPLIT_K, ROW_GROUPS).  Returns slots written. */
+ * TG_CFG_* slots (kernel, BLOCK_M, BLOCK_N, SPLIT_K, ROW_GROUPS, WAVES).  Returns slots written. */
 int32_t tg_last_config(int32_t* out, int32_t n);
 
 /* Static message for a return code (src/tilegym/ops/cutile_rs/ffi_util.rs:125-135). */

@@ -80,16 +80,17 @@ def test_per_tensor_tiled_split_k(device, split):
 
 # ----------------------------------------------------------------------------- skinny
 @pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
-@pytest.mark.parametrize("N,K,rg,split", [(1000, 512, 1, 1), (4096, 1024, 2, 2), (520, 2064, 4, 4), (256, 128, 1, 1)])
-def test_per_tensor_skinny(device, M, N, K, rg, split):
+@pytest.mark.parametrize("N,K,rg,split,waves", [(1000, 512, 1, 1, 4), (4096, 1024, 2, 2, 8), (520, 2064, 4, 4, 16), (256, 128, 1, 1, 16)])
+def test_per_tensor_skinny(device, M, N, K, rg, split, waves):
     g = _g(M * 7 + N)
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
     sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
     ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
     out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
-                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "skinny", "ROW_GROUPS": rg, "SPLIT_K": split})
-    used("skinny")
-    check(out, ref, what=f"skinny M={M} N={N} K={K} rg={rg} split={split}")
+                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "skinny", "ROW_GROUPS": rg, "SPLIT_K": split, "WAVES": waves})
+    cfg = used("skinny")
+    assert cfg["WAVES"] == waves
+    check(out, ref, what=f"skinny M={M} N={N} K={K} rg={rg} split={split} waves={waves}")
 
 
 def test_skinny_auto_schedule_and_determinism(device):
@@ -98,7 +99,7 @@ def test_skinny_auto_schedule_and_determinism(device):
     d = case.to(device)
     outs = [matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a, scale_b=d.scale_b, out_dtype=torch.bfloat16) for _ in range(4)]
     cfg = used("skinny")
-    assert cfg["SPLIT_K"] > 1, "decode O-proj should use split-K to fill the chip"
+    assert cfg["WAVES"] == 16, "decode O-proj should split K over 16 waves per workgroup to fill the chip"
     check(outs[0], ref, what="decode o M=16")
     assert all(torch.equal(outs[0], o) for o in outs[1:])
 

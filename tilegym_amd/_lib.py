@@ -21,7 +21,7 @@ DEFAULT_LIB_PATH = os.path.join(_HERE, "libtilegym_hip.so")
 
 TG_MAX_DIMS = 5
 TG_CFG_COUNT = 8
-CFG_SLOTS = {"KERNEL": 0, "BLOCK_M": 1, "BLOCK_N": 2, "SPLIT_K": 3, "ROW_GROUPS": 4}
+CFG_SLOTS = {"KERNEL": 0, "BLOCK_M": 1, "BLOCK_N": 2, "SPLIT_K": 3, "ROW_GROUPS": 4, "WAVES": 5}
 KERNEL_NAMES = {0: "fallback", 1: "tiled", 2: "skinny"}
 
 # dtype codes of the ABI (include/tilegym_hip.h)
@@ -165,15 +165,15 @@ _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
 def workspace_for(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
-    """Zero-initialised scratch buffer for the current stream of ``device`` (grown on demand).
-    One buffer per (device, stream): calls on one stream are ordered, so they can share it."""
+    """Scratch buffer for the current stream of ``device`` (grown on demand).  One buffer per
+    (device, stream): calls on one stream are ordered, so they can share it."""
     if nbytes <= 0:
         return None
     stream = torch.cuda.current_stream(device)
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(int(nbytes), dtype=torch.uint8, device=device)
+        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 

@@ -89,6 +89,38 @@ __global__ void __launch_bounds__(256) transpose_u8_kernel(const uint8_t* __rest
     }
 }
 
+// Second pass of the split-K schedules: one thread adds the split_k partial sums of four
+// consecutive outputs in z order, then scales, applies beta and casts.
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmParams p, int block_scaled) {
+    const int64_t quads_per_row = (p.N + 3) / 4;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= quads_per_row * p.M) return;
+    const int m = (int)(idx / quads_per_row), col = (int)(idx % quads_per_row) * 4;
+    const int64_t MN = (int64_t)p.M * p.N, at = (int64_t)m * p.N + col;
+    const bool vec_ok = p.vec_store != 0;
+    v4f sum = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < p.split_k; ++z) {
+        const float* src = p.partials + z * MN + at;
+        if (vec_ok && col + 3 < p.N) sum += *reinterpret_cast<const v4f*>(src);
+        else
+            for (int q = 0; q < 4 && col + q < p.N; ++q) sum[q] += src[q];
+    }
+    float scale = p.alpha;
+    if (!block_scaled) {
+        if (p.As) scale *= p.As[0];
+        if (p.Bs) scale *= p.Bs[0];
+    }
+    store4(p.C, p.out_type, m, col, p.N, sum * scale, p.beta, vec_ok);
+}
+
+hipError_t run_splitk_reduce(const GemmParams& p, bool block_scaled, hipStream_t s) {
+    const int64_t work = (int64_t)((p.N + 3) / 4) * p.M;
+    if (work <= 0) return hipSuccess;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, p,
+                       block_scaled ? 1 : 0);
+    return hipGetLastError();
+}
+
 hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s) {
     if (rows <= 0 || cols <= 0) return hipSuccess;
     dim3 grid((cols + 63) / 64, (rows + 63) / 64, 1);

@@ -160,7 +160,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     __shared__ __align__(1024) uint8_t sB1[BN * kKBlock];
     __shared__ int s_src[GROUP == GROUP_DENSE ? 1 : BM];
     __shared__ int s_dst[GROUP == GROUP_DENSE ? 1 : BM];
-    __shared__ int s_flag;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -437,29 +436,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
         }
     }
 
-    if constexpr (SPLIT) {
-        if (!splitk_arrive(p.counters, tile_m * tiles_n + tile_n, p.split_k, &s_flag)) return;
-        // last workgroup for this tile: add the partial tiles in a fixed order
-        for (int idx = tid; idx < BM * (BN / 8); idx += NT) {
-            const int r = idx / (BN / 8), col = n0 + (idx % (BN / 8)) * 8;
-            if (r >= rows_valid || col >= p.N) continue;
-            const int64_t at = (int64_t)(m0 + r) * p.N + col;
-            v4f lo = v4f{0.f, 0.f, 0.f, 0.f}, hi = lo;
-            for (int z = 0; z < p.split_k; ++z) {
-                const float* src = p.partials + z * MN + at;
-                if (vec_ok && col + 7 < p.N) {
-                    lo += reinterpret_cast<const v4f*>(src)[0];
-                    hi += reinterpret_cast<const v4f*>(src)[1];
-                } else {
-                    for (int q = 0; q < 8 && col + q < p.N; ++q) {
-                        if (q < 4) lo[q & 3] += src[q];
-                        else hi[q & 3] += src[q];
-                    }
-                }
-            }
-            store8(p.C, p.out_type, m0 + r, col, p.N, lo * scale, hi * scale, p.beta, vec_ok);
-        }
-    }
 #endif
 }
 

@@ -13,7 +13,6 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 namespace tg {
 
 constexpr int kKBlock = 128;    // bytes of K consumed by one 16x16x128 MFMA = the quant block
-constexpr int kCounterSlots = 16384;  // ints at the start of a workspace (split-K arrival counters)
 
 enum OutType { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2 };  // same numbering as the ABI dtype codes
 
@@ -31,11 +30,11 @@ struct GemmParams {
     float alpha, beta;
     int out_type;
     int vec_store;      // 1 when N % 4 == 0 and C is 16-byte aligned: 4-wide stores allowed
-    // split-K
+    // split-K: grid.y partitions of the K steps; each writes raw fp32 sums to partials[z][M][N]
+    // and a separate reduction kernel adds them in z order and applies the epilogue
     int split_k;        // >= 1
     int ksteps_per_split;
-    float* partials;    // [split_k][M][N] fp32
-    int* counters;      // one per output tile, zero on entry, zero on exit
+    float* partials;
     // grouped forms
     const int* m_indptr;   // ragged: (E+1)
     int E;
@@ -116,26 +115,6 @@ __device__ __forceinline__ void store4(void* C, int out_type, int64_t row, int c
             *p = (_Float16)x;
         }
     }
-}
-
-// Split-K arrival: every workgroup that worked on `tile` calls this after writing its partial
-// sums.  Returns true in exactly one workgroup -- the last to arrive -- which then owns the
-// reduction.  The counter is returned to zero by that workgroup.
-__device__ __forceinline__ bool splitk_arrive(int* counters, int tile, int split_k, int* s_flag) {
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int old = __hip_atomic_fetch_add(&counters[tile], 1, __ATOMIC_ACQ_REL,
-                                         __HIP_MEMORY_SCOPE_AGENT);
-        int last = (old == split_k - 1);
-        if (last)
-            __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *s_flag = last;
-    }
-    __syncthreads();
-    bool last = (*s_flag != 0);
-    if (last) __threadfence();
-    return last;
 }
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Re-number them so that each

@@ -71,9 +71,8 @@ inline int cfg_get(const int32_t* cfg, int32_t ncfg, int slot) {
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
-constexpr int64_t kCounterBytes = (int64_t)tg::kCounterSlots * 4;
 constexpr int64_t kOffsetLimit = (int64_t)1 << 31;  // kernels index operands with 32-bit byte offsets
-constexpr int kTargetWorkgroups = 1024;             // 4 per CU on 256 CUs
+constexpr int kTargetWaves = 4096;                  // 16 waves on each of 256 CUs
 
 // Switches to the caller's device for the lifetime of a call.
 struct DeviceGuard {
@@ -97,7 +96,7 @@ struct DeviceGuard {
 
 struct Schedule {
     int kernel;  // 0 fallback, 1 tiled, 2 skinny
-    int bm, bn, split_k, row_groups, mt;
+    int bm, bn, split_k, row_groups, mt, waves;
 };
 
 void remember(const Schedule& s) {
@@ -107,6 +106,7 @@ void remember(const Schedule& s) {
     g_last_cfg[TG_CFG_BLOCK_N] = s.bn;
     g_last_cfg[TG_CFG_SPLIT_K] = s.split_k;
     g_last_cfg[TG_CFG_ROW_GROUPS] = s.row_groups;
+    g_last_cfg[TG_CFG_WAVES] = s.waves;
 }
 
 bool tile_exists(int bm, int bn, bool block_scaled) {
@@ -117,12 +117,12 @@ bool tile_exists(int bm, int bn, bool block_scaled) {
     return false;
 }
 
-// Split-K factor: enough workgroups to fill the chip, at least `min_steps` K steps per split,
-// partial sums must fit the workspace.
-int pick_split(int64_t workgroups, int64_t kblocks, int min_steps, int64_t M, int64_t N,
-               int64_t partial_bytes_avail, int want) {
-    int64_t split = want > 0 ? want : cdiv(kTargetWorkgroups, workgroups > 0 ? workgroups : 1);
-    if (want <= 0) split = split > 16 ? 16 : split;
+// Split-K factor: `want` if given, else enough to reach `target_units` units of parallel work;
+// at least `min_steps` K steps per split, and the partial sums must fit the workspace.
+int pick_split(int64_t units, int64_t target_units, int64_t kblocks, int min_steps, int64_t M,
+               int64_t N, int64_t partial_bytes_avail, int want) {
+    int64_t split = want > 0 ? want : cdiv(target_units, units > 0 ? units : 1);
+    if (want <= 0 && split > 16) split = 16;
     const int64_t by_k = kblocks / min_steps > 0 ? kblocks / min_steps : 1;
     if (split > by_k) split = by_k;
     const int64_t per = M * N * 4;
@@ -130,13 +130,12 @@ int pick_split(int64_t workgroups, int64_t kblocks, int min_steps, int64_t M, in
     if (split < 1) split = 1;
     // every split must own at least one K step
     const int64_t kps = cdiv(kblocks, split);
-    split = cdiv(kblocks, kps);
-    return (int)split;
+    return (int)cdiv(kblocks, kps);
 }
 
 Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
                       const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
-    Schedule s{0, -1, -1, 1, -1, -1};
+    Schedule s{0, -1, -1, 1, -1, -1, -1};
     const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
     const int64_t kblocks = cdiv(K, 128);
     if (!fast_layout || want_kernel == 0 || K == 0) return s;
@@ -150,14 +149,19 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         s.kernel = 2;
         s.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
         int rg = cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS);
-        if (rg != 1 && rg != 2 && rg != 4) {
-            rg = 1;
-            if (cdiv(N, 32) >= 768) rg = 2;
-            if (cdiv(N, 64) >= 1024 && s.mt <= 2) rg = 4;
-        }
+        if (!(rg == 1 || rg == 2 || (rg == 4 && s.mt == 1))) rg = (N >= 16384 && s.mt <= 2) ? 2 : 1;
         s.row_groups = rg;
         const int64_t wgs = cdiv(N, 16 * rg);
-        s.split_k = wgs > tg::kCounterSlots ? 1 : pick_split(wgs, kblocks, 8, M, N, partial_bytes_avail, want_split);
+        // waves per workgroup: they split K inside the workgroup, no traffic between workgroups
+        int nw = cfg_get(cfg, ncfg, TG_CFG_WAVES);
+        if (nw != 4 && nw != 8 && nw != 16) {
+            nw = wgs * 4 >= kTargetWaves ? 4 : wgs * 8 >= kTargetWaves ? 8 : 16;
+            while (nw > 4 && kblocks < nw) nw /= 2;
+        }
+        s.waves = nw;
+        s.split_k = 1;
+        if (want_split > 1 || (want_split < 0 && wgs * nw * 2 <= kTargetWaves))
+            s.split_k = pick_split(wgs * nw, kTargetWaves, kblocks, 2 * nw, M, N, partial_bytes_avail, want_split);
         return s;
     }
     s.kernel = 1;
@@ -173,8 +177,8 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     s.bn = bn;
     const int64_t wgs = cdiv(M, bm) * cdiv(N, bn);
     s.split_k = 1;
-    if (wgs <= tg::kCounterSlots && (want_split > 1 || (want_split < 0 && wgs < 192)))
-        s.split_k = pick_split(wgs * 4, kblocks, 8, M, N, partial_bytes_avail, want_split);
+    if (want_split > 1 || (want_split < 0 && wgs <= 128))
+        s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
     return s;
 }
 
@@ -217,7 +221,7 @@ int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t tra
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     int64_t split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
     if (split <= 0) split = 16;
-    int64_t bytes = kCounterBytes;
+    int64_t bytes = 0;
     // partial sums are only used while they stay a modest part of the traffic
     int64_t partial = split * M * N * 4;
     const int64_t cap = (int64_t)256 << 20;
@@ -277,11 +281,11 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
     if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
 
-    // ---- workspace carving: [counters][partials ...][optional K-contiguous copy of B]
+    // ---- workspace carving: [split-K partial sums ...][optional K-contiguous copy of B]
     const int64_t ws_bytes = workspace ? numel(workspace) * elem_size(workspace->dtype) : 0;
     uint8_t* ws = workspace ? reinterpret_cast<uint8_t*>(workspace->ptr) : nullptr;
-    int64_t ws_free = ws_bytes > kCounterBytes ? ws_bytes - kCounterBytes : 0;
-    uint8_t* ws_cursor = ws ? ws + kCounterBytes : nullptr;
+    int64_t ws_free = ws_bytes;
+    uint8_t* ws_cursor = ws;
 
     const uint8_t* Bnt = reinterpret_cast<const uint8_t*>(b->ptr);
     bool b_is_nk = trans_b != 0;
@@ -340,15 +344,16 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
     if (s.split_k > 1) {
         p.split_k = s.split_k;
         p.ksteps_per_split = (int)cdiv(kblocks, s.split_k);
-        p.counters = reinterpret_cast<int*>(ws);
         p.partials = reinterpret_cast<float*>(ws_cursor);
     }
     remember(s);
 
     if (s.kernel == 2) {
         const int gx = (int)cdiv(N, 16 * s.row_groups);
-        hipError_t e = tg::run_skinny(s.mt, s.row_groups, block_scaled, p, gx, s.split_k, stream);
+        hipError_t e = tg::run_skinny(s.mt, s.row_groups, s.waves, block_scaled, p, gx, s.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "skinny kernel launch failed: %s", hipGetErrorString(e));
+        if (s.split_k > 1 && tg::run_splitk_reduce(p, block_scaled, stream) != hipSuccess)
+            return fail(TG_ERR_LAUNCH, "split-K reduction launch failed");
         return TG_OK;
     }
 
@@ -368,6 +373,8 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
         hipError_t e = block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
                                     : tg::run_tile_per_tensor(s.bm, s.bn, split, pc, gx, pc.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "tiled kernel launch failed: %s", hipGetErrorString(e));
+        if (split && tg::run_splitk_reduce(pc, block_scaled, stream) != hipSuccess)
+            return fail(TG_ERR_LAUNCH, "split-K reduction launch failed");
     }
     return TG_OK;
 }
@@ -450,7 +457,7 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
     const bool fast = (K % 128) == 0 && K > 0 && aligned16(a->ptr) && aligned16(b->ptr) &&
                       total_m * K < kOffsetLimit && N * K < kOffsetLimit &&
                       cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
-    Schedule s{0, -1, -1, 1, -1, -1};
+    Schedule s{0, -1, -1, 1, -1, -1, -1};
     if (!fast) {
         tg::GenericParams q{};
         q.g = p;
@@ -532,7 +539,7 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
     }
     const bool fast = bm > 0 && (K % 128) == 0 && K > 0 && aligned16(a->ptr) && aligned16(b->ptr) &&
                       T * K < kOffsetLimit && N * K < kOffsetLimit && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
-    Schedule s{0, -1, -1, 1, -1, -1};
+    Schedule s{0, -1, -1, 1, -1, -1, -1};
     if (!fast) {
         tg::GenericParams q{};
         q.g = p;
