@@ -28,14 +28,34 @@
 
 namespace tg {
 
-#if defined(__HIP_DEVICE_COMPILE__)
 // Raw buffer descriptor over [base, base + 2 GiB): byte offsets, no format conversion.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), (short)0, 0x7FFFFFFF, 0x00020000);
+__device__ __forceinline__ v4i make_rsrc(const void* base) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(base);
+    return v4i{(int)(uint32_t)a, (int)((uint32_t)(a >> 32) & 0xFFFFu), 0x7FFFFFFF, 0x00020000};
 }
-#endif
 
-__device__ __forceinline__ int swz16(int r) { return ((r & 7) + ((r >> 3) & 1)) & 7; }
+// One direct global->LDS load: every lane fetches 16 bytes at rsrc.base + voffset + soffset and
+// the wave's 64 x 16 bytes land at LDS address lds_addr + 16 * lane.  Written as inline assembly
+// on purpose: the compiler's wait-count insertion treats a builtin direct load that is still in
+// flight as possibly aliasing every later LDS read and drains the whole memory pipeline
+// (vmcnt(0)) in front of it, which would undo the multi-step prefetch.  Completion is tracked by
+// hand with the vmcnt waits in the kernel; the "memory" clobber keeps LDS reads from being
+// cached across it.
+__device__ __forceinline__ void direct_load_b128(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory");
+}
+
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+// Chunk swizzle of a 128-byte slab row: 16-byte chunk j of row r sits at chunk position j ^ (r % 8).
+// Measured on gfx950 (256 B/clk LDS): ds_read_b128 of 16 consecutive rows at one logical chunk is
+// conflict free with this XOR (4.0 clk per wave-read); additive variants are 2-way conflicted.
+__device__ __forceinline__ int swz16(int r) { return r & 7; }
 
 // Number of BM-row tiles over all experts (every lane returns the same value).
 __device__ __forceinline__ int ragged_count_tiles(const int* indptr, int E, int BM, int lane) {
@@ -132,14 +152,39 @@ __device__ __forceinline__ void store8(void* C, int out_type, int64_t row, int c
     }
 }
 
+// Instruction-order hint for one K step of a wave: the LDS fragment reads and the direct
+// global->LDS loads of the next stage are spread between the MFMAs instead of being issued in
+// bursts (all waves of a workgroup run in phase, so a burst of memory instructions leaves the
+// matrix pipe idle).  Order requested from the scheduler: the reads of the first two column
+// tiles, then per column tile: TM MFMAs, a share of the direct loads, the two reads of the column
+// tile after next.
+#define TG_SGB_MFMA 0x008
+#define TG_SGB_VMEM_READ 0x020
+#define TG_SGB_DS_READ 0x100
+template <int TM, int TN, int LOADS>
+__device__ __forceinline__ void pipeline_hint() {
+    constexpr int PER = (LOADS + TN - 1) / TN;  // direct loads issued per column tile
+    __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 4, 0);  // wf[0], wf[1]
+#define TG_GROUP(i)                                                                         \
+    if constexpr (TN > (i)) {                                                                \
+        __builtin_amdgcn_sched_group_barrier(TG_SGB_MFMA, TM, 0);                            \
+        if constexpr ((i) * PER < LOADS)                                                     \
+            __builtin_amdgcn_sched_group_barrier(TG_SGB_VMEM_READ, PER, 0);                  \
+        if constexpr ((i) + 2 < TN) __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 2, 0); \
+    }
+    TG_GROUP(0) TG_GROUP(1) TG_GROUP(2) TG_GROUP(3) TG_GROUP(4) TG_GROUP(5) TG_GROUP(6) TG_GROUP(7)
+#undef TG_GROUP
+}
+
 template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>
 __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_gemm_tile_kernel(const GemmParams p) {
-#if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only types; the host pass only needs the stub
+#if defined(__HIP_DEVICE_COMPILE__)  // the body is device-only assembly; the host pass only needs the stub
     constexpr int NT = 64 * WGM * WGN;
     constexpr int NW = WGM * WGN;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 16, TN = WTN / 16;
-    constexpr int RPP = 8 * NW;  // slab rows filled per pass of the whole workgroup
+    constexpr int NL = NW == 8 ? 4 : NW;  // waves that issue the direct global->LDS loads
+    constexpr int RPP = 8 * NL;           // slab rows filled per pass of the loader waves
     constexpr int A_IT = BM / RPP, B_IT = BN / RPP;
     // epilogue slices: PCOLS columns of the wave tile at a time, fp32, through one LDS object
     constexpr int OBJ = (BM < BN ? BM : BN) * kKBlock;  // bytes of the smaller stage object
@@ -237,15 +282,18 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     }
 
     // ---------------------------------------------------------------- loader set-up
-    // Pass i of wave w fills the 8-row group g = i*NW + w: lane l lands at row 8g + l/8, chunk
-    // position l%8, and therefore fetches logical chunk (l%8) ^ swz16(row%16).  NW is even, so
-    // row%16 = 8*(w&1) + l/8 for every pass.
+    // The first NL waves of the workgroup issue every direct load (one loader per SIMD when there
+    // are two waves per SIMD: while a loader waits for room in the memory pipeline, the other
+    // wave of its SIMD keeps the matrix pipe fed).  Pass i of loader w fills the 8-row group
+    // g = i*NL + w: lane l lands at row 8g + l/8, chunk position l%8, and therefore fetches
+    // logical chunk (l%8) ^ swz16(row) = (l%8) ^ (l/8).
     const int lrow = lane >> 3;
-    const int lj = (lane & 7) ^ swz16(((wave & 1) << 3) + lrow);
+    const int lj = (lane & 7) ^ swz16(lrow);
+    const bool loader = wave < NL;
     uint32_t a_off[A_IT], b_off[B_IT];
 #pragma unroll
     for (int i = 0; i < A_IT; ++i) {
-        const int r = (i * NW + wave) * 8 + lrow;
+        const int r = (i * NL + (wave % NL)) * 8 + lrow;
         int src;
         if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
         else src = s_src[r];
@@ -253,7 +301,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     }
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
-        const int n = min(n0 + (i * NW + wave) * 8 + lrow, p.N - 1);
+        const int n = min(n0 + (i * NL + (wave % NL)) * 8 + lrow, p.N - 1);
         b_off[i] = (uint32_t)n * (uint32_t)K + lj * 16;
     }
 
@@ -290,24 +338,23 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
 
     float sc_next[TM];
 
-    // Direct global->LDS load of one K step into (dA, dB), as buffer loads: 32-bit per-lane
-    // offset + scalar K offset, no 64-bit address arithmetic in the loop.  K is a multiple of
-    // 128 here (the host sends other K to the fallback kernel), so every lane's 16 bytes are
-    // in range.
-    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(Bbase);
-    auto issue_loads = [&](int kstep, uint8_t* dA, uint8_t* dB) {
+    // Direct global->LDS loads of one K step, as buffer loads: 32-bit per-lane offset + scalar
+    // K offset, no 64-bit address arithmetic in the loop.  K is a multiple of 128 here (the host
+    // sends other K to the fallback kernel), so every lane's 16 bytes are in range.
+    const v4i rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(Bbase);
+    auto issue_a = [&](int kstep, uint8_t* dA) {
+        if (!loader) return;
         const int k0 = kstep * kKBlock;
+        const uint32_t dst = lds_address(dA) + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < A_IT; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                rsrc_a, (__attribute__((address_space(3))) void*)(dA + (i * NW + wave) * 1024), 16,
-                a_off[i], k0, 0, 0);
+        for (int i = 0; i < A_IT; ++i) direct_load_b128(rsrc_a, dst + i * NL * 1024, a_off[i], k0);
+    };
+    auto issue_b = [&](int kstep, uint8_t* dB) {
+        if (!loader) return;
+        const int k0 = kstep * kKBlock;
+        const uint32_t dst = lds_address(dB) + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < B_IT; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                rsrc_b, (__attribute__((address_space(3))) void*)(dB + (i * NW + wave) * 1024), 16,
-                b_off[i], k0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int i = 0; i < B_IT; ++i) direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
     };
     auto load_scales = [&](int kstep) {
         if constexpr (BLOCKSCALE) {
@@ -319,14 +366,16 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
             }
         }
     };
-    auto compute = [&](const uint8_t* cA, const uint8_t* cB, const float* sc) {
-        v8i af[TM];
+    v8i af[TM];
+    auto read_a = [&](const uint8_t* cA) {
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
             const uint8_t* base = cA + a_frag_base + tm * 16 * kKBlock;
             af[tm] = join(*reinterpret_cast<const v4i*>(base + frag0),
                           *reinterpret_cast<const v4i*>(base + frag1));
         }
+    };
+    auto mma = [&](const uint8_t* cB, const float* sc) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
             const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
@@ -343,47 +392,61 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
             }
         }
     };
-    // All of this wave's direct loads have landed in LDS; then every wave's have.
-    auto stage_ready = [&]() {
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
-        __syncthreads();
+    // vmcnt(n): this wave's direct loads, except the n most recent, have landed in LDS.
+    constexpr int kWaitAllButA = 0x0F70 | (A_IT & 15) | ((A_IT >> 4) << 14);
+    constexpr int kWaitAll = 0x0F70;
+    constexpr int kWaitLds = 0xC07F;  // lgkmcnt(0) only
+    // Workgroup barrier without the memory fence of __syncthreads(): that fence would also wait
+    // for every direct load in flight (vmcnt(0)), which is exactly what the deeper prefetch must
+    // not do.  LDS reads are ordered with lgkmcnt, direct loads with the vmcnt waits below.
+    auto lds_barrier = [&]() {
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        __builtin_amdgcn_s_barrier();
     };
 
     // ---------------------------------------------------------------- main loop
-    // Two K steps per trip (stage 0 then stage 1); an odd last step is peeled.
+    // Stage buffers (sA0,sB0) and (sA1,sB1); step k computes from stage k%2.  The B slab of a stage
+    // is read throughout the step, the A slab only at its start (the A fragments stay in
+    // registers), so A is prefetched two steps ahead and B one:
+    //   top of step k : issue B(k+1) -> other stage;  read A fragments of stage k%2;  barrier
+    //                   (every wave holds its A fragments: that A slab is free)
+    //   then          : issue A(k+2) -> this stage's A slab;  MFMAs with B fragments streamed from LDS
+    //   end of step k : wait for all direct loads except A(k+2);  barrier
+    // Steps past the end are clamped to the last step: they re-fetch it into an idle slab, which
+    // keeps the loop body free of branches.
     float sc_cur[TM];
-    const int nsteps = ks_end - ks;
-    issue_loads(ks, sA0, sB0);
+    const int nsteps = ks_end - ks, last = ks_end - 1;
+    issue_a(ks, sA0);
+    issue_b(ks, sB0);
+    issue_a(min(ks + 1, last), sA1);
     load_scales(ks);
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = BLOCKSCALE ? sc_next[tm] : 1.0f;
-    stage_ready();
+    if (loader) __builtin_amdgcn_s_waitcnt(kWaitAllButA);
+    lds_barrier();
+    auto step = [&](int k, uint8_t* cA, uint8_t* cB, uint8_t* oB) {
+        issue_b(min(k + 1, last), oB);
+        load_scales(min(k + 1, last));
+        read_a(cA);
+        lds_barrier();
+        issue_a(min(k + 2, last), cA);
+        mma(cB, sc_cur);
+        if constexpr (!BLOCKSCALE) pipeline_hint<TM, TN, A_IT>();
+        if constexpr (BLOCKSCALE) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = sc_next[tm];
+        }
+        if (loader) __builtin_amdgcn_s_waitcnt(kWaitAllButA);
+        lds_barrier();
+    };
     int i = 0;
     for (; i + 1 < nsteps; i += 2) {
-        issue_loads(ks + i + 1, sA1, sB1);
-        load_scales(ks + i + 1);
-        compute(sA0, sB0, sc_cur);
-        if constexpr (BLOCKSCALE) {
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = sc_next[tm];
-        }
-        stage_ready();
-        if (i + 2 < nsteps) {
-            issue_loads(ks + i + 2, sA0, sB0);
-            load_scales(ks + i + 2);
-        }
-        compute(sA1, sB1, sc_cur);
-        if constexpr (BLOCKSCALE) {
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = sc_next[tm];
-        }
-        stage_ready();
+        step(ks + i, sA0, sB0, sB1);
+        step(ks + i + 1, sA1, sB1, sB0);
     }
-    if (i < nsteps) {
-        compute(sA0, sB0, sc_cur);
-        __syncthreads();
-    }
+    if (i < nsteps) step(ks + i, sA0, sB0, sB1);
+    __builtin_amdgcn_s_waitcnt(kWaitAll);
+    __syncthreads();
 
     // ---------------------------------------------------------------- epilogue
     // Every wave is past the last barrier, so the stage buffers are free: wave w stages through
