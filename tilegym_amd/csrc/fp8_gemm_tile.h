@@ -28,10 +28,15 @@
 
 namespace tg {
 
+constexpr int kMaxKBlocks = 512;  // K <= 65536 for the block-scaled tiled kernels (host checks)
+
 // Raw buffer descriptor over [base, base + 2 GiB): byte offsets, no format conversion.
 __device__ __forceinline__ v4i make_rsrc(const void* base) {
+    // the base is the same in every lane; say so, so that the descriptor lives in scalar registers
     const uintptr_t a = reinterpret_cast<uintptr_t>(base);
-    return v4i{(int)(uint32_t)a, (int)((uint32_t)(a >> 32) & 0xFFFFu), 0x7FFFFFFF, 0x00020000};
+    const int lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    const int hi = __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xFFFFu));
+    return v4i{lo, hi, 0x7FFFFFFF, 0x00020000};
 }
 
 // One direct global->LDS load: every lane fetches 16 bytes at rsrc.base + voffset + soffset and
@@ -43,6 +48,14 @@ __device__ __forceinline__ v4i make_rsrc(const void* base) {
 // cached across it.
 __device__ __forceinline__ void direct_load_b128(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory");
+}
+
+// Same for 4 bytes per lane (the wave's 64 x 4 bytes land at lds_addr + 4 * lane).
+__device__ __forceinline__ void direct_load_b32(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
                  : "memory");
@@ -176,6 +189,23 @@ __device__ __forceinline__ void pipeline_hint() {
 #undef TG_GROUP
 }
 
+// Block-scaled variant: after the MFMAs of a column tile, the 4*TM multiply-adds that fold the
+// previous column tile's products into the accumulators.
+#define TG_SGB_VALU 0x002
+template <int TM, int TN, int LOADS>
+__device__ __forceinline__ void pipeline_hint_scaled() {
+    __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 4, 0);
+#define TG_GROUP(i)                                                                         \
+    if constexpr (TN > (i)) {                                                                \
+        __builtin_amdgcn_sched_group_barrier(TG_SGB_MFMA, TM, 0);                            \
+        if constexpr ((i) > 0) __builtin_amdgcn_sched_group_barrier(TG_SGB_VALU, 4 * TM, 0); \
+        if constexpr ((i) + 2 < TN) __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 2, 0); \
+    }
+    TG_GROUP(0) TG_GROUP(1) TG_GROUP(2) TG_GROUP(3) TG_GROUP(4) TG_GROUP(5) TG_GROUP(6) TG_GROUP(7)
+#undef TG_GROUP
+    __builtin_amdgcn_sched_group_barrier(TG_SGB_VALU, 4 * TM, 0);
+}
+
 template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>
 __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_gemm_tile_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body is device-only assembly; the host pass only needs the stub
@@ -203,6 +233,11 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     __shared__ __align__(1024) uint8_t sA1[BM * kKBlock];
     __shared__ __align__(1024) uint8_t sB0[BN * kKBlock];
     __shared__ __align__(1024) uint8_t sB1[BN * kKBlock];
+    // per-stage activation scales of the slab rows (block-scaled kernels only)
+    __shared__ __align__(256) float sS0[BLOCKSCALE ? BM : 1];
+    __shared__ __align__(256) float sS1[BLOCKSCALE ? BM : 1];
+    // weight block scales of this tile's column blocks for every K step (fetched once)
+    __shared__ float sBs[BLOCKSCALE ? (BN + 127) / 128 : 1][BLOCKSCALE ? kMaxKBlocks : 1];
     __shared__ int s_src[GROUP == GROUP_DENSE ? 1 : BM];
     __shared__ int s_dst[GROUP == GROUP_DENSE ? 1 : BM];
 
@@ -310,18 +345,28 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     const uint32_t frag1 = frag0 ^ 64;
     const uint32_t a_frag_base = wm * WTM * kKBlock, b_frag_base = wn * WTN * kKBlock;
 
-    // block scales: one activation scale per (lane, tm), one weight scale per wave
-    int srow[TM];
-    const float* bs_ptr = nullptr;
+    // block scales: the activation scales of a K step travel with its slabs (one 4-byte direct
+    // load per slab row into sS0/sS1, issued by the first BM/64 loader waves), the weight scale
+    // is one scalar per wave and K step.
+    uint32_t s_off = 0;
+    constexpr int S_WAVES = (BM + 63) / 64;
+    static_assert(!BLOCKSCALE || S_WAVES <= NL, "scale rows are fetched by the loader waves");
     if constexpr (BLOCKSCALE) {
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
-            const int r = wm * WTM + tm * 16 + li;
-            if constexpr (GROUP == GROUP_DENSE) srow[tm] = m0 + min(r, rows_valid - 1);
-            else srow[tm] = s_src[r];
+        constexpr int NBT = (BN + 127) / 128;
+        for (int idx = tid; idx < NBT * p.kblocks; idx += NT) {
+            const int j = idx / p.kblocks, kb = idx % p.kblocks;
+            const int nb = min(n0 / 128 + j, p.nblocks - 1);
+            sBs[j][kb] = Bsbase ? Bsbase[(int64_t)nb * p.kblocks + kb] : 1.0f;
         }
-        const int nb = min((n0 + wn * WTN) / 128, p.nblocks - 1);
-        if (Bsbase) bs_ptr = Bsbase + (int64_t)nb * p.kblocks;
+        const int r = min(wave * 64 + lane, BM - 1);
+        int src;
+        if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
+        else src = s_src[r];
+        s_off = (uint32_t)src * (uint32_t)p.kblocks * 4u;
+        if (!p.As) {  // no activation scales: ones
+            for (int r2 = tid; r2 < BM; r2 += NT) sS0[r2] = sS1[r2] = 1.0f;
+        }
+        __syncthreads();
     }
 
     int ks = 0, ks_end = p.kblocks;
@@ -335,8 +380,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
-
-    float sc_next[TM];
 
     // Direct global->LDS loads of one K step, as buffer loads: 32-bit per-lane offset + scalar
     // K offset, no 64-bit address arithmetic in the loop.  K is a multiple of 128 here (the host
@@ -356,14 +399,19 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
     };
-    auto load_scales = [&](int kstep) {
+    const v4i rsrc_s = make_rsrc(p.As);
+    auto issue_s = [&](int kstep, float* dS) {
         if constexpr (BLOCKSCALE) {
-            const float bs = bs_ptr ? bs_ptr[kstep] : 1.0f;
+            if (p.As && wave < S_WAVES && (BM >= 64 || lane < BM))
+                direct_load_b32(rsrc_s, lds_address(dS) + wave * 256, s_off, kstep * 4);
+        }
+    };
+    float sc[TM];
+    auto read_scales = [&](int kstep, const float* cS) {
+        if constexpr (BLOCKSCALE) {
+            const float bs = sBs[(wn * WTN) / 128][kstep];
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) {
-                const float as = p.As ? p.As[(int64_t)srow[tm] * p.kblocks + kstep] : 1.0f;
-                sc_next[tm] = as * bs;
-            }
+            for (int tm = 0; tm < TM; ++tm) sc[tm] = cS[wm * WTM + tm * 16 + li] * bs;
         }
     };
     v8i af[TM];
@@ -375,20 +423,34 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
                           *reinterpret_cast<const v4i*>(base + frag1));
         }
     };
-    auto mma = [&](const uint8_t* cB, const float* sc) {
+    auto mma = [&](const uint8_t* cB) {
+        if constexpr (BLOCKSCALE) {
+            // The 16x16 products of column tile tn are scaled and added while the MFMAs of
+            // column tile tn+1 run: MFMA and VALU work overlap instead of alternating.
+            v4f part[2][TM];
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
-            const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
-            const v8i wf = join(*reinterpret_cast<const v4i*>(base + frag0),
-                                *reinterpret_cast<const v4i*>(base + frag1));
+            for (int tn = 0; tn < TN; ++tn) {
+                const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
+                const v8i wf = join(*reinterpret_cast<const v4i*>(base + frag0),
+                                    *reinterpret_cast<const v4i*>(base + frag1));
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) {
-                if constexpr (BLOCKSCALE) {
-                    const v4f part = mfma_e4m3(wf, af[tm], v4f{0.f, 0.f, 0.f, 0.f});
-                    acc[tn][tm] += part * sc[tm];
-                } else {
-                    acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
+                for (int tm = 0; tm < TM; ++tm)
+                    part[tn & 1][tm] = mfma_e4m3(wf, af[tm], v4f{0.f, 0.f, 0.f, 0.f});
+                if (tn > 0) {
+#pragma unroll
+                    for (int tm = 0; tm < TM; ++tm) acc[tn - 1][tm] += part[(tn - 1) & 1][tm] * sc[tm];
                 }
+            }
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) acc[TN - 1][tm] += part[(TN - 1) & 1][tm] * sc[tm];
+        } else {
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+                const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
+                const v8i wf = join(*reinterpret_cast<const v4i*>(base + frag0),
+                                    *reinterpret_cast<const v4i*>(base + frag1));
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
             }
         }
     };
@@ -408,43 +470,39 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     // Stage buffers (sA0,sB0) and (sA1,sB1); step k computes from stage k%2.  The B slab of a stage
     // is read throughout the step, the A slab only at its start (the A fragments stay in
     // registers), so A is prefetched two steps ahead and B one:
-    //   top of step k : issue B(k+1) -> other stage;  read A fragments of stage k%2;  barrier
+    //   top of step k : issue B(k+1) (and its activation scales) -> other stage;  read A fragments
+    //                   (and scales) of stage k%2;  barrier
     //                   (every wave holds its A fragments: that A slab is free)
     //   then          : issue A(k+2) -> this stage's A slab;  MFMAs with B fragments streamed from LDS
     //   end of step k : wait for all direct loads except A(k+2);  barrier
     // Steps past the end are clamped to the last step: they re-fetch it into an idle slab, which
     // keeps the loop body free of branches.
-    float sc_cur[TM];
     const int nsteps = ks_end - ks, last = ks_end - 1;
     issue_a(ks, sA0);
     issue_b(ks, sB0);
+    issue_s(ks, sS0);
     issue_a(min(ks + 1, last), sA1);
-    load_scales(ks);
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = BLOCKSCALE ? sc_next[tm] : 1.0f;
     if (loader) __builtin_amdgcn_s_waitcnt(kWaitAllButA);
     lds_barrier();
-    auto step = [&](int k, uint8_t* cA, uint8_t* cB, uint8_t* oB) {
+    auto step = [&](int k, uint8_t* cA, uint8_t* cB, float* cS, uint8_t* oB, float* oS) {
         issue_b(min(k + 1, last), oB);
-        load_scales(min(k + 1, last));
+        issue_s(min(k + 1, last), oS);
         read_a(cA);
+        read_scales(k, cS);
         lds_barrier();
         issue_a(min(k + 2, last), cA);
-        mma(cB, sc_cur);
+        mma(cB);
         if constexpr (!BLOCKSCALE) pipeline_hint<TM, TN, A_IT>();
-        if constexpr (BLOCKSCALE) {
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm) sc_cur[tm] = sc_next[tm];
-        }
+        else pipeline_hint_scaled<TM, TN, A_IT>();
         if (loader) __builtin_amdgcn_s_waitcnt(kWaitAllButA);
         lds_barrier();
     };
     int i = 0;
     for (; i + 1 < nsteps; i += 2) {
-        step(ks + i, sA0, sB0, sB1);
-        step(ks + i + 1, sA1, sB1, sB0);
+        step(ks + i, sA0, sB0, sS0, sB1, sS1);
+        step(ks + i + 1, sA1, sB1, sS1, sB0, sS0);
     }
-    if (i < nsteps) step(ks + i, sA0, sB0, sB1);
+    if (i < nsteps) step(ks + i, sA0, sB0, sS0, sB1, sS1);
     __builtin_amdgcn_s_waitcnt(kWaitAll);
     __syncthreads();
 

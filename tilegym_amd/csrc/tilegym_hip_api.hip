@@ -139,7 +139,8 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
     const int64_t kblocks = cdiv(K, 128);
     if (!fast_layout || want_kernel == 0 || K == 0) return s;
-    const bool tile_ok = (K % 128) == 0;
+    // the block-scaled tiled kernels keep a tile's weight scales for all K steps in LDS (512 steps)
+    const bool tile_ok = (K % 128) == 0 && (!block_scaled || kblocks <= 512);
     bool skinny = M <= 64;
     if (want_kernel == 1 && tile_ok) skinny = false;
     if (want_kernel == 2 && M <= 64) skinny = true;
@@ -454,7 +455,7 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
     fill_grouped(p, c, a, b, a_scale, b_scale, total_m, E, N, K, out_type);
     p.m_indptr = reinterpret_cast<const int*>(m_indptr->ptr);
 
-    const bool fast = (K % 128) == 0 && K > 0 && aligned16(a->ptr) && aligned16(b->ptr) &&
+    const bool fast = (K % 128) == 0 && K > 0 && K <= 65536 && aligned16(a->ptr) && aligned16(b->ptr) &&
                       total_m * K < kOffsetLimit && N * K < kOffsetLimit &&
                       cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
     Schedule s{0, -1, -1, 1, -1, -1, -1};
@@ -537,7 +538,7 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
         bm = (block_m % 128 == 0) ? 128 : (block_m % 64 == 0) ? 64 : 0;
         bn = (bm == 128 && N >= 2048) ? 256 : 128;
     }
-    const bool fast = bm > 0 && (K % 128) == 0 && K > 0 && aligned16(a->ptr) && aligned16(b->ptr) &&
+    const bool fast = bm > 0 && (K % 128) == 0 && K > 0 && K <= 65536 && aligned16(a->ptr) && aligned16(b->ptr) &&
                       T * K < kOffsetLimit && N * K < kOffsetLimit && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
     Schedule s{0, -1, -1, 1, -1, -1, -1};
     if (!fast) {
