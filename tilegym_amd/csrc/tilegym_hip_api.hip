@@ -169,8 +169,10 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
     if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, block_scaled))) {
         auto tiles = [&](int64_t a, int64_t b) { return cdiv(M, a) * cdiv(N, b); };
+        // measured on MI355X: per-tensor prefers the largest tile that still fills the chip;
+        // block-scaled (extra multiply-adds per K step, two workgroups per CU) prefers 128x128
         if (!block_scaled && tiles(256, 256) >= 200) { bm = 256; bn = 256; }
-        else if (tiles(128, 256) >= 200) { bm = 128; bn = 256; }
+        else if (!block_scaled && tiles(128, 256) >= 200) { bm = 128; bn = 256; }
         else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
         else { bm = 64; bn = 128; }
     }
@@ -473,7 +475,7 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
     int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
     if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, true))) {
         bm = (total_m / E >= 96) ? 128 : 64;
-        bn = (bm == 128 && N >= 2048) ? 256 : 128;
+        bn = 128;
     }
     s.kernel = 1; s.bm = bm; s.bn = bn;
     remember(s);
@@ -536,7 +538,7 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
     int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
     if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, true) && block_m % bm == 0)) {
         bm = (block_m % 128 == 0) ? 128 : (block_m % 64 == 0) ? 64 : 0;
-        bn = (bm == 128 && N >= 2048) ? 256 : 128;
+        bn = 128;
     }
     const bool fast = bm > 0 && (K % 128) == 0 && K > 0 && K <= 65536 && aligned16(a->ptr) && aligned16(b->ptr) &&
                       T * K < kOffsetLimit && N * K < kOffsetLimit && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
