@@ -59,7 +59,7 @@ typedef struct tg_tensor {
  * This is the C form of the reference's per-call `kernel_configs={...}` override
  * (src/tilegym/kernel_utils.py:14-36). */
 enum {
-    TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (weight-streaming) kernel */
+    TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (direct weight streaming), 3 stream (weight streaming through LDS) */
     TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (64/128/256)            */
     TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (128/256)               */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */

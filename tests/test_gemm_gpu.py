@@ -93,13 +93,27 @@ def test_per_tensor_skinny(device, M, N, K, rg, split, waves):
     check(out, ref, what=f"skinny M={M} N={N} K={K} rg={rg} split={split} waves={waves}")
 
 
-def test_skinny_auto_schedule_and_determinism(device):
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64])
+@pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 1), (264, 2064, 1), (256, 9216, 1), (128, 16384, 4), (72, 512, 1)])
+def test_per_tensor_stream(device, M, N, K, split):
+    """Weight streaming through LDS: K tails inside a 1 KiB piece, ragged N, single and double buffering, split-K."""
+    g = _g(M * 11 + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
+    ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "stream", "SPLIT_K": split})
+    cfg = used("stream")
+    assert cfg["SPLIT_K"] == split
+    check(out, ref, what=f"stream M={M} N={N} K={K} split={split}")
+
+
+def test_decode_auto_schedule_and_determinism(device):
     case = W.llama_decode_case(16, "o")
     ref = R.ref_gemm_per_tensor(case.a, case.b, case.scale_a, case.scale_b, trans_b=True)
     d = case.to(device)
     outs = [matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a, scale_b=d.scale_b, out_dtype=torch.bfloat16) for _ in range(4)]
-    cfg = used("skinny")
-    assert cfg["WAVES"] == 16, "decode O-proj should split K over 16 waves per workgroup to fill the chip"
+    used("stream")
     check(outs[0], ref, what="decode o M=16")
     assert all(torch.equal(outs[0], o) for o in outs[1:])
 
@@ -139,7 +153,7 @@ def test_k_tail_multiple_of_16_skinny(device):
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g)
     ref = R.ref_gemm_per_tensor(a, b, trans_b=True)
     out = matmul(a.to(device), b.to(device), trans_b=True, out_dtype=torch.bfloat16)
-    used("skinny")
+    used("stream")
     check(out, ref)
 
 
@@ -153,7 +167,7 @@ def test_output_dtypes(device, dtype):
         ref = R.ref_gemm_per_tensor(a, b, trans_b=True, out_dtype=dtype)
         check(out, ref, what=f"{kernel} {dtype}")
     out = matmul(a[:9].contiguous().to(device), b.to(device), trans_b=True, out_dtype=dtype)
-    used("skinny")
+    used("skinny")  # K = 256: too short for 1 KiB pieces
     check(out, R.ref_gemm_per_tensor(a[:9], b, trans_b=True, out_dtype=dtype))
 
 
@@ -232,14 +246,15 @@ def test_block_scaled_tiled_configs_and_edges(device, bm, bn, M, N, K):
 
 @pytest.mark.parametrize("M", [1, 16, 40, 64])
 @pytest.mark.parametrize("split", [1, 4])
-def test_block_scaled_skinny(device, M, split):
-    case = W.block_scaled_case(M, 640, 1024, seed=M)
+@pytest.mark.parametrize("kernel,K", [("skinny", 1024), ("stream", 1024), ("stream", 4224)])
+def test_block_scaled_skinny(device, M, split, kernel, K):
+    case = W.block_scaled_case(M, 640, K, seed=M)
     ref = R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, output_dtype=torch.bfloat16)
     d = case.to(device)
     out = tilegym_amd.backend._REGISTRY["unsloth.w8a8_block_fp8_matmul"]["hip"](
-        d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs={"KERNEL": "skinny", "SPLIT_K": split})
-    used("skinny")
-    check(out, ref, what=f"block-scaled skinny M={M}")
+        d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs={"KERNEL": kernel, "SPLIT_K": split})
+    used(kernel)
+    check(out, ref, what=f"block-scaled {kernel} M={M} K={K}")
 
 
 def test_block_scaled_batched_leading_dims_and_invariants(device):
@@ -434,7 +449,7 @@ def test_config2_llama_decode_full(device, proj):
         a = big.a[:M].contiguous()
         ref = ((R.fp8_to_f32(a) * big.scale_a) @ bref.t()).to(torch.bfloat16)
         out = matmul(a.to(device), bd, trans_b=True, scale_a=big.scale_a.to(device), scale_b=big.scale_b.to(device), out_dtype=torch.bfloat16)
-        used("skinny")
+        used("stream")
         check(out, ref, what=f"config 2 {proj} M={M}")
 
 
@@ -466,7 +481,7 @@ def test_config4_block_scaled_full(device, N, K):
     ref = R.ref_w8a8_block_fp8_matmul(big.a[rows], big.b, big.scale_a[rows], big.scale_b, None, torch.bfloat16)
     check(out[rows.to(device)], ref, what=f"config 4 M=4096 {N}x{K}")
     out16 = w8a8_block_fp8_matmul(d.a[:16].contiguous(), d.b, d.scale_a[:16].contiguous(), d.scale_b, None, torch.bfloat16)
-    used("skinny")
+    used("stream")
     ref16 = R.ref_w8a8_block_fp8_matmul(big.a[:16], big.b, big.scale_a[:16], big.scale_b, None, torch.bfloat16)
     check(out16, ref16, what=f"config 4 M=16 {N}x{K}")
 

@@ -1,0 +1,232 @@
+// Weight-streaming FP8 GEMM for skinny activations (M <= 64), second generation:
+// C[m,n] = sum_k A[m,k] * B[n,k], bound by reading B once from HBM.
+//
+// Measured on MI355X: a wave-wide load whose 64 lanes cover 1 KiB of ONE weight row streams at
+// ~6.5 TB/s, while loads shaped like the MFMA operand (16 rows x 64 bytes per instruction) stay
+// near 4.5 TB/s.  So the weights are fetched with direct global->LDS loads of one row x 1 KiB per
+// instruction and LDS does the transposition into the MFMA operand layout: a wave owns a
+// private 16-row x 1 KiB LDS buffer (or two, double buffered), fills it with 16 such loads,
+// waits for its own loads only (no workgroup barrier in the loop) and runs 8 K steps of
+// 16x16x128 MFMAs from it.  Lane l of the load for row r fetches 16-byte chunk l ^ r of the
+// 1 KiB piece, which makes the later fragment reads (16 rows, same logical chunk) bank-conflict
+// free.  The 4 waves of a workgroup take interleaved 1 KiB pieces of the same 16 rows; their
+// accumulators are added through LDS at the end.  K can additionally be split across
+// workgroups (grid.y) into fp32 partial sums reduced by a second kernel.
+#pragma once
+#include "fp8_gemm_tile.h"
+
+namespace tg {
+
+constexpr int kStreamChunk = 1024;  // bytes of one row fetched by one load instruction
+
+template <int MT, int NBUF, bool BLOCKSCALE>
+__global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int NW = 4;
+    constexpr int BUF = 16 * kStreamChunk;
+    __shared__ __align__(1024) uint8_t sW[NW * NBUF * BUF];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int K = p.K, N = p.N, M = p.M;
+    const int n_base = blockIdx.x * 16;
+    const int nchunks_total = (K + kStreamChunk - 1) / kStreamChunk;
+
+    int c_begin = 0, c_end = nchunks_total;
+    if (p.split_k > 1) {  // ksteps_per_split counts 1 KiB pieces here
+        c_begin = blockIdx.y * p.ksteps_per_split;
+        c_end = min(c_begin + p.ksteps_per_split, nchunks_total);
+    }
+
+    // per-row byte offsets of this lane's 16-byte chunk: row r, logical chunk lane ^ r
+    const v4i rsrc_b = make_rsrc(p.B);
+    uint8_t* my_buf = sW + wave * NBUF * BUF;
+    const uint32_t my_lds = lds_address(my_buf);
+
+    auto issue_chunk = [&](int c, int buf) {
+        const int k0 = c * kStreamChunk;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int n = min(n_base + r, N - 1);
+            const int j = lane ^ r;
+            const uint32_t voff = (uint32_t)n * (uint32_t)K + j * 16;
+            const uint32_t dst = my_lds + buf * BUF + r * kStreamChunk;
+            if (k0 + j * 16 < K) {
+                direct_load_b128(rsrc_b, dst, voff, k0);
+            } else {  // past the end of K: zeros
+                *reinterpret_cast<v4i*>(my_buf + buf * BUF + r * kStreamChunk + lane * 16) = v4i{0, 0, 0, 0};
+            }
+        }
+    };
+
+    const uint8_t* aptr[MT];
+    bool aok[MT];
+    int arow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + li;
+        aok[mt] = m < M;
+        arow[mt] = min(m, M - 1);
+        aptr[mt] = p.A + (int64_t)arow[mt] * K + lg * 16;
+    }
+    const float* bs_ptr = nullptr;
+    if constexpr (BLOCKSCALE) {
+        const int nb = min(n_base / 128, p.nblocks - 1);
+        bs_ptr = p.Bs ? p.Bs + (int64_t)nb * p.kblocks : nullptr;
+    }
+
+    v4f acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    auto load_act = [&](int kstep, v4i* lo, v4i* hi) {
+        const int k0 = kstep * kKBlock;
+        const bool ok0 = (k0 + lg * 16) < K, ok1 = (k0 + 64 + lg * 16) < K;
+        const v4i zero = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            lo[mt] = (aok[mt] && ok0) ? *reinterpret_cast<const v4i*>(aptr[mt] + k0) : zero;
+            hi[mt] = (aok[mt] && ok1) ? *reinterpret_cast<const v4i*>(aptr[mt] + k0 + 64) : zero;
+        }
+    };
+
+    constexpr int SPC = kStreamChunk / kKBlock;  // K steps per 1 KiB piece
+    // M <= 16: the activation fragments of a whole piece are fetched up front (before the piece
+    // after it is requested: loads complete in order, so an activation load issued behind the
+    // next piece's direct loads would have to wait for them).  Larger M: one K step ahead.
+    constexpr bool PRELOAD = MT == 1;
+    v4i pa_lo[PRELOAD ? SPC : 1], pa_hi[PRELOAD ? SPC : 1];
+    auto preload_act = [&](int c) {
+        if constexpr (PRELOAD) {
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) load_act(c * SPC + s, &pa_lo[s], &pa_hi[s]);
+        }
+    };
+    auto mma_step = [&](int ks, v8i wf, const v8i* af) {
+        float sc[MT];
+        if constexpr (BLOCKSCALE) {
+            const float sb = bs_ptr ? bs_ptr[ks] : 1.0f;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                sc[mt] = (p.As ? p.As[(int64_t)arow[mt] * p.kblocks + ks] : 1.0f) * sb;
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if constexpr (BLOCKSCALE) {
+                const v4f part = mfma_e4m3(wf, af[mt], v4f{0.f, 0.f, 0.f, 0.f});
+                acc[mt] += part * sc[mt];
+            } else {
+                acc[mt] = mfma_e4m3(wf, af[mt], acc[mt]);
+            }
+        }
+    };
+    auto compute_chunk = [&](int c, int buf) {
+        const uint8_t* base = my_buf + buf * BUF + li * kStreamChunk;
+        const int ks0 = c * SPC;
+        const int nks = min(SPC, p.kblocks - ks0);
+        if constexpr (PRELOAD) {
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) {
+                if (s < nks) {
+                    const int j0 = s * 8 + lg, j1 = j0 + 4;
+                    const v8i wf = join(*reinterpret_cast<const v4i*>(base + ((j0 ^ li) << 4)),
+                                        *reinterpret_cast<const v4i*>(base + ((j1 ^ li) << 4)));
+                    const v8i af = join(pa_lo[s], pa_hi[s]);
+                    mma_step(ks0 + s, wf, &af);
+                }
+            }
+        } else {
+            v4i a_lo[MT], a_hi[MT];
+            load_act(ks0, a_lo, a_hi);
+            for (int s = 0; s < nks; ++s) {
+                v8i af[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) af[mt] = join(a_lo[mt], a_hi[mt]);
+                if (s + 1 < nks) load_act(ks0 + s + 1, a_lo, a_hi);
+                const int j0 = s * 8 + lg, j1 = j0 + 4;
+                const v8i wf = join(*reinterpret_cast<const v4i*>(base + ((j0 ^ li) << 4)),
+                                    *reinterpret_cast<const v4i*>(base + ((j1 ^ li) << 4)));
+                mma_step(ks0 + s, wf, af);
+            }
+        }
+    };
+
+    // ---- stream this wave's 1 KiB pieces
+    constexpr int kWaitMine = 0x0070;                                   // vmcnt(0) lgkmcnt(0)
+    constexpr int kWaitAllBut16 = 0x0F70 | (16 & 15) | ((16 >> 4) << 14);  // vmcnt(16)
+    constexpr int kWaitLds = 0xC07F;                                    // lgkmcnt(0)
+    int c = c_begin + wave;
+    if constexpr (NBUF == 1) {
+        for (; c < c_end; c += NW) {
+            preload_act(c);
+            issue_chunk(c, 0);
+            __builtin_amdgcn_s_waitcnt(kWaitMine);  // my loads and zero fills have landed
+            compute_chunk(c, 0);
+            __builtin_amdgcn_s_waitcnt(kWaitLds);   // my LDS reads are done before the refill
+        }
+    } else {
+        int buf = 0;
+        if (c < c_end) issue_chunk(c, 0);
+        for (; c < c_end; c += NW) {
+            const int nxt = c + NW;
+            preload_act(c);
+            if (nxt < c_end) {
+                issue_chunk(nxt, buf ^ 1);
+                __builtin_amdgcn_s_waitcnt(kWaitAllBut16);  // everything older than the next piece
+                __builtin_amdgcn_s_waitcnt(kWaitLds);
+            } else {
+                __builtin_amdgcn_s_waitcnt(kWaitMine);
+            }
+            compute_chunk(c, buf);
+            __builtin_amdgcn_s_waitcnt(kWaitLds);
+            buf ^= 1;
+        }
+    }
+
+    // ---- add the four waves' accumulators through LDS (each wave's buffer is its own until here)
+    __syncthreads();
+    v4f* red = reinterpret_cast<v4f*>(sW);
+    if (wave > 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) red[((wave - 1) * MT + mt) * 64 + lane] = acc[mt];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int w = 0; w < NW - 1; ++w) acc[mt] += red[(w * MT + mt) * 64 + lane];
+
+    const bool vec_ok = p.vec_store != 0;
+    const int col = n_base + lg * 4;
+    if (p.split_k > 1) {
+        float* mine = p.partials + (int64_t)blockIdx.y * M * N;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + li;
+            if (m < M && col < N) store4(mine, OUT_F32, m, col, N, acc[mt], 0.f, vec_ok);
+        }
+        return;
+    }
+    float scale = p.alpha;
+    if constexpr (!BLOCKSCALE) {
+        if (p.As) scale *= p.As[0];
+        if (p.Bs) scale *= p.Bs[0];
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + li;
+        if (m < M && col < N) store4(p.C, p.out_type, m, col, N, acc[mt] * scale, p.beta, vec_ok);
+    }
+#endif
+}
+
+template <int MT, int NBUF, bool BLOCKSCALE>
+inline hipError_t launch_stream(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
+    auto kern = fp8_gemm_stream_kernel<MT, NBUF, BLOCKSCALE>;
+    hipLaunchKernelGGL(kern, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace tg

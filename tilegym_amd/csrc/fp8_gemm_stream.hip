@@ -1,0 +1,16 @@
+// Instantiations of the second-generation weight-streaming skinny-M kernel.
+#include "fp8_gemm_stream.h"
+#include "tg_host.h"
+
+namespace tg {
+
+hipError_t run_stream(int mt, int nbuf, bool bs, const GemmParams& p, int gx, int gy, hipStream_t s) {
+#define TG_CASE(MT, NBUF)                                                   \
+    if (mt == MT && nbuf == NBUF)                                           \
+        return bs ? launch_stream<MT, NBUF, true>(p, gx, gy, s) : launch_stream<MT, NBUF, false>(p, gx, gy, s);
+    TG_CASE(1, 1) TG_CASE(1, 2) TG_CASE(2, 1) TG_CASE(2, 2) TG_CASE(4, 1) TG_CASE(4, 2)
+#undef TG_CASE
+    return hipErrorInvalidConfiguration;
+}
+
+}  // namespace tg

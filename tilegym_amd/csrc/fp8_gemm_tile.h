@@ -47,6 +47,8 @@ __device__ __forceinline__ v4i make_rsrc(const void* base) {
 // hand with the vmcnt waits in the kernel; the "memory" clobber keeps LDS reads from being
 // cached across it.
 __device__ __forceinline__ void direct_load_b128(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);  // wave-uniform by construction
+    soffset = __builtin_amdgcn_readfirstlane(soffset);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
@@ -55,6 +57,8 @@ __device__ __forceinline__ void direct_load_b128(v4i rsrc, uint32_t lds_addr, ui
 
 // Same for 4 bytes per lane (the wave's 64 x 4 bytes land at lds_addr + 4 * lane).
 __device__ __forceinline__ void direct_load_b32(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+    soffset = __builtin_amdgcn_readfirstlane(soffset);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)

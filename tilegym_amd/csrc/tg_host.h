@@ -23,6 +23,7 @@ hipError_t run_tile_per_tensor(int bm, int bn, bool split, const GemmParams& p, 
 hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
 hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_skinny(int mt, int rg, int nw, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
+hipError_t run_stream(int mt, int nbuf, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
 // C <- epilogue(sum_z partials[z]) for the split-K schedules (fixed z order: bit-reproducible)
 hipError_t run_splitk_reduce(const GemmParams& p, bool block_scaled, hipStream_t s);
 hipError_t run_generic(const GenericParams& p, hipStream_t s);

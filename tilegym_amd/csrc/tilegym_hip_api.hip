@@ -95,7 +95,7 @@ struct DeviceGuard {
 };
 
 struct Schedule {
-    int kernel;  // 0 fallback, 1 tiled, 2 skinny
+    int kernel;  // 0 fallback, 1 tiled, 2 skinny, 3 stream
     int bm, bn, split_k, row_groups, mt, waves;
 };
 
@@ -143,9 +143,21 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     const bool tile_ok = (K % 128) == 0 && (!block_scaled || kblocks <= 512);
     bool skinny = M <= 64;
     if (want_kernel == 1 && tile_ok) skinny = false;
-    if (want_kernel == 2 && M <= 64) skinny = true;
+    if ((want_kernel == 2 || want_kernel == 3) && M <= 64) skinny = true;
     if (!skinny && !tile_ok) return s;
     const int want_split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
+    if (skinny && want_kernel != 2 && (want_kernel == 3 || K >= 1024)) {
+        // weight streaming through LDS, 1 KiB of a row per load instruction
+        s.kernel = 3;
+        s.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+        s.row_groups = 1;
+        s.waves = 4;
+        const int64_t pieces = cdiv(K, 1024), wgs = cdiv(N, 16);
+        s.split_k = 1;
+        if (want_split > 1 || (want_split < 0 && wgs * 4 * 4 <= kTargetWaves && pieces >= 16))
+            s.split_k = pick_split(wgs * 4, kTargetWaves / 2, pieces, want_split > 1 ? 1 : 8, M, N, partial_bytes_avail, want_split);
+        return s;
+    }
     if (skinny) {
         s.kernel = 2;
         s.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
@@ -351,6 +363,17 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
     }
     remember(s);
 
+    if (s.kernel == 3) {
+        const int64_t pieces = cdiv(K, 1024);
+        if (s.split_k > 1) p.ksteps_per_split = (int)cdiv(pieces, s.split_k);
+        const int64_t per_wave = cdiv(s.split_k > 1 ? p.ksteps_per_split : pieces, 4);
+        const int nbuf = (per_wave >= 2 && s.mt == 1) ? 2 : 1;
+        hipError_t e = tg::run_stream(s.mt, nbuf, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
+        if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "stream kernel launch failed: %s", hipGetErrorString(e));
+        if (s.split_k > 1 && tg::run_splitk_reduce(p, block_scaled, stream) != hipSuccess)
+            return fail(TG_ERR_LAUNCH, "split-K reduction launch failed");
+        return TG_OK;
+    }
     if (s.kernel == 2) {
         const int gx = (int)cdiv(N, 16 * s.row_groups);
         hipError_t e = tg::run_skinny(s.mt, s.row_groups, s.waves, block_scaled, p, gx, s.split_k, stream);
