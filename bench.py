@@ -32,6 +32,8 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense FP8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+KERNEL_SYMBOLS = {"tiled": "fp8_gemm_tile_kernel", "skinny": "fp8_gemm_skinny_kernel", "stream": "fp8_gemm_stream_kernel",
+                  "fallback": "fp8_gemm_generic_kernel"}
 ROTATE_BYTES = 640 << 20   # operand footprint to rotate through (> 2x the 256 MB memory-side cache)
 
 
@@ -190,6 +192,9 @@ def main():
     ap.add_argument("--workload", default="all", choices=["prefill", "decode", "block", "moe", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time microsecond kernels with plain launches")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run a plain elementwise copy of known size (256 MiB read + 256 MiB written, 3 launches): "
+                         "the yardstick that hardware traffic counters are scaled by when this command runs under a profiler")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
@@ -207,6 +212,14 @@ def main():
     props = torch.cuda.get_device_properties(device)
     out = {}
     detail = {}
+    if args.calibrate_copy:
+        src = torch.zeros(64 << 20, dtype=torch.float32, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ prefill (headline)
     if args.workload in ("prefill", "all"):
@@ -256,7 +269,7 @@ def main():
             "us_per_step": round(tot_us, 2),
             "frac_hbm_M_le_16": round(sum(s["bytes"] for s in small) / sum(s["us"] for s in small) * 1e-3 / PEAK_HBM_GBS, 4),
             "roofline": {"bound": "hbm", "achieved": dom["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
-                         "traffic": None, "kernel": "fp8_gemm_skinny_kernel per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
+                         "traffic": None, "kernel": KERNEL_SYMBOLS[dom["kernel"]] + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
         }
         detail["decode"] = shapes
         if "value" in out:

@@ -141,7 +141,9 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     if (!fast_layout || want_kernel == 0 || K == 0) return s;
     // the block-scaled tiled kernels keep a tile's weight scales for all K steps in LDS (512 steps)
     const bool tile_ok = (K % 128) == 0 && (!block_scaled || kblocks <= 512);
-    bool skinny = M <= 64;
+    // above 16 rows the streaming kernels would re-read the activations once per 16 weight rows;
+    // the LDS-tiled kernel with a 64-row tile and split-K shares them across 128 weight rows
+    bool skinny = M <= 16 || (M <= 64 && !tile_ok);
     if (want_kernel == 1 && tile_ok) skinny = false;
     if ((want_kernel == 2 || want_kernel == 3) && M <= 64) skinny = true;
     if (!skinny && !tile_ok) return s;
@@ -183,7 +185,8 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         auto tiles = [&](int64_t a, int64_t b) { return cdiv(M, a) * cdiv(N, b); };
         // measured on MI355X: per-tensor prefers the largest tile that still fills the chip;
         // block-scaled (extra multiply-adds per K step, two workgroups per CU) prefers 128x128
-        if (!block_scaled && tiles(256, 256) >= 200) { bm = 256; bn = 256; }
+        if (M <= 64) { bm = 64; bn = 128; }
+        else if (!block_scaled && tiles(256, 256) >= 200) { bm = 256; bn = 256; }
         else if (!block_scaled && tiles(128, 256) >= 200) { bm = 128; bn = 256; }
         else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
         else { bm = 64; bn = 128; }
@@ -192,8 +195,19 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     s.bn = bn;
     const int64_t wgs = cdiv(M, bm) * cdiv(N, bn);
     s.split_k = 1;
-    if (want_split > 1 || (want_split < 0 && wgs <= 128))
+    if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
+    } else if (want_split < 0 && M <= 64) {
+        // weight-streaming regime: at least 128 workgroups and at most 16 K steps per split
+        int64_t units = 128;
+        if (kblocks / 16 * wgs > units) units = kblocks / 16 * wgs;
+        if (units > 512) units = 512;
+        int want = 1;
+        while (want * wgs < units && want < 16) want *= 2;
+        if (want > 1) s.split_k = pick_split(wgs, units, kblocks, 4, M, N, partial_bytes_avail, want);
+    } else if (want_split < 0 && wgs <= 128) {
+        s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
+    }
     return s;
 }
 
