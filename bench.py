@@ -34,7 +34,29 @@ PEAK_FP8_TFLOPS = 5000.0   # MI355X dense FP8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 KERNEL_SYMBOLS = {"tiled": "fp8_gemm_tile_kernel", "skinny": "fp8_gemm_skinny_kernel", "stream": "fp8_gemm_stream_kernel",
                   "fallback": "fp8_gemm_generic_kernel"}
-ROTATE_BYTES = 640 << 20   # operand footprint to rotate through (> 2x the 256 MB memory-side cache)
+ROTATE_BYTES = 640 << 20
+
+# HBM bytes per launch (reads + writes) from the hardware counters FETCH_SIZE and WRITE_SIZE, collected in
+# two profiler passes of this program and scaled by what the same counters read for --calibrate-copy's
+# elementwise add of known size (reads x2.000, writes x1.000); figures and commands are in
+# profiles/fp8_gemm_tile_kernel_prefill_pmc.txt and profiles/fp8_gemm_stream_kernel_decode_pmc.txt.
+# Decode entries are the average over M = 1, 8, 16 of one projection (same grid).
+KIB = 1024
+MEASURED_TRAFFIC = {
+    "c3_prefill_qkv_M8192": (147620.4 * 2 + 98304.0) * KIB,
+    "c3_prefill_gate_up_M8192": (688551.8 * 2 + 458752.0) * KIB,
+    "c2_decode_qkv": (12497.2 * 2 + 100.0) * KIB,
+    "c2_decode_o": (8370.3 * 2 + 66.7) * KIB,
+    "c2_decode_gate_up": (57712.5 * 2 + 466.7) * KIB,
+    "c2_decode_down": (29204.2 * 2 + 66.7) * KIB,
+}
+
+
+def measured_traffic(shape_name):
+    for key, val in MEASURED_TRAFFIC.items():
+        if shape_name == key or (key.startswith("c2_decode") and shape_name.startswith(key + "_M") and not shape_name.endswith("M64")):
+            return int(val)
+    return None   # operand footprint to rotate through (> 2x the 256 MB memory-side cache)
 
 
 def _events_ms(fn, iters, stream):
@@ -242,7 +264,7 @@ def main():
             "value": round(total_flops / (ms_per_step * 1e-3) * 1e-12, 2),
             "ms_per_step": round(ms_per_step, 4),
             "roofline": {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                         "frac": dom["frac_mfma"], "traffic": None, "kernel": f"fp8_gemm_tile_kernel<{dom['block_m']},{dom['block_n']}> per-tensor",
+                         "frac": dom["frac_mfma"], "traffic": measured_traffic(dom["name"]), "kernel": f"fp8_gemm_tile_kernel<{dom['block_m']},{dom['block_n']}> per-tensor",
                          "shape": dom["name"], "us_per_launch": dom["us"]},
         })
         detail["prefill"] = shapes
@@ -269,7 +291,7 @@ def main():
             "us_per_step": round(tot_us, 2),
             "frac_hbm_M_le_16": round(sum(s["bytes"] for s in small) / sum(s["us"] for s in small) * 1e-3 / PEAK_HBM_GBS, 4),
             "roofline": {"bound": "hbm", "achieved": dom["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
-                         "traffic": None, "kernel": KERNEL_SYMBOLS[dom["kernel"]] + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
+                         "traffic": measured_traffic(dom["name"]), "kernel": KERNEL_SYMBOLS[dom["kernel"]] + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
         }
         detail["decode"] = shapes
         if "value" in out:
