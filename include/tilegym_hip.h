@@ -59,12 +59,12 @@ typedef struct tg_tensor {
  * This is the C form of the reference's per-call `kernel_configs={...}` override
  * (src/tilegym/kernel_utils.py:14-36). */
 enum {
-    TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (direct weight streaming), 3 stream (weight streaming through LDS) */
+    TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (direct weight streaming), 3 stream (weight streaming through LDS), 4 pipe (register-pipelined 256x256 tile; per-tensor scales, beta == 0, bf16/f16 out) */
     TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (64/128/256)            */
     TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (128/256)               */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
     TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4)         */
-    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16)       */
+    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); pipe kernel: loader waves (4/8) */
     TG_CFG_COUNT = 8
 };
 

@@ -78,6 +78,39 @@ def test_per_tensor_tiled_split_k(device, split):
         assert torch.equal(again, out)
 
 
+# ----------------------------------------------------------------------------- per-tensor, register-pipelined 256x256 tile
+@pytest.mark.parametrize("loaders", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 520, 384), (257, 255, 512), (1024, 768, 1280), (40, 1000, 256), (512, 252, 640)])
+def test_per_tensor_pipe(device, M, N, K, loaders):
+    """K = 128 (two half-steps), K with an odd number of 128-byte steps (loop tail), ragged M and N,
+    N not a multiple of 8 (scalar store path), both loader-wave counts."""
+    g = _g(M + 3 * N + K + loaders)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.013]), torch.tensor([0.0004])
+    ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
+    out = torch.full((M + 1, N), 7.0, dtype=torch.bfloat16, device=device)  # one guard row past the end
+    res = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "pipe", "WAVES": loaders})
+    cfg = used("pipe")
+    assert cfg["WAVES"] == loaders
+    check(res, ref, what=f"pipe M={M} N={N} K={K} loaders={loaders}")
+    one = torch.tensor([1.0])  # keep the f16 outputs in the normal range
+    ref16 = R.ref_gemm_per_tensor(a, b, one, one, trans_b=True, out_dtype=torch.float16)
+    res16 = matmul(a.to(device), b.to(device), trans_b=True, scale_a=one.to(device), scale_b=one.to(device),
+                   out_dtype=torch.float16, kernel_configs={"KERNEL": "pipe"})
+    used("pipe")
+    check(res16, ref16, what=f"pipe f16 M={M} N={N} K={K}")
+    del out
+
+
+def test_pipe_falls_back_to_tiled_for_beta_and_f32(device):
+    g = _g(91)
+    a, b = fp8_randn((300, 256), g), fp8_randn((520, 256), g, 0.1)
+    out = matmul(a.to(device), b.to(device), trans_b=True, out_dtype=torch.float32, kernel_configs={"KERNEL": "pipe"})
+    used("tiled")
+    check(out, R.ref_gemm_per_tensor(a, b, trans_b=True, out_dtype=torch.float32))
+
+
 # ----------------------------------------------------------------------------- skinny
 @pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K,rg,split,waves", [(1000, 512, 1, 1, 4), (4096, 1024, 2, 2, 8), (520, 2064, 4, 4, 16), (256, 128, 1, 1, 16)])

@@ -94,8 +94,23 @@ struct DeviceGuard {
     }
 };
 
+// Compute units of a device (queried once per device; 256 on MI355X).
+int compute_units(int dev) {
+    static int cached[64] = {0};
+    if (dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 struct Schedule {
-    int kernel;  // 0 fallback, 1 tiled, 2 skinny, 3 stream
+    int kernel;  // 0 fallback, 1 tiled, 2 skinny, 3 stream, 4 pipe (register-pipelined 256x256 tile)
     int bm, bn, split_k, row_groups, mt, waves;
 };
 
@@ -133,7 +148,7 @@ int pick_split(int64_t units, int64_t target_units, int64_t kblocks, int min_ste
     return (int)cdiv(kblocks, kps);
 }
 
-Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
+Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout, bool pipe_ok,
                       const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
     Schedule s{0, -1, -1, 1, -1, -1, -1};
     const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
@@ -144,7 +159,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     // above 16 rows the streaming kernels would re-read the activations once per 16 weight rows;
     // the LDS-tiled kernel with a 64-row tile and split-K shares them across 128 weight rows
     bool skinny = M <= 16 || (M <= 64 && !tile_ok);
-    if (want_kernel == 1 && tile_ok) skinny = false;
+    if ((want_kernel == 1 || want_kernel == 4) && tile_ok) skinny = false;
     if ((want_kernel == 2 || want_kernel == 3) && M <= 64) skinny = true;
     if (!skinny && !tile_ok) return s;
     const int want_split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
@@ -191,10 +206,16 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
         else { bm = 64; bn = 128; }
     }
+    if (want_kernel == 4 && pipe_ok) { bm = 256; bn = 256; }
     s.bm = bm;
     s.bn = bn;
     const int64_t wgs = cdiv(M, bm) * cdiv(N, bn);
     s.split_k = 1;
+    if (bm == 256 && bn == 256 && pipe_ok && want_split <= 1 && want_kernel == 4) {  // opt-in: slower than the tiled kernel so far
+        s.kernel = 4;
+        s.waves = cfg_get(cfg, ncfg, TG_CFG_WAVES) == 8 ? 8 : 4;  // loader waves (of eight)
+        return s;
+    }
     if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
     } else if (want_split < 0 && M <= 64) {
@@ -337,7 +358,9 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
 
     const bool fast_layout = !trans_a && b_is_nk && (K % 16) == 0 && aligned16(a->ptr) &&
                              aligned16(reinterpret_cast<uint64_t>(Bnt)) && N * K < kOffsetLimit;
-    Schedule s = choose_dense(M, N, K, block_scaled, fast_layout, cfg, ncfg, ws_free);
+    const bool pipe_ok = !block_scaled && beta == 0.0f && (K % 128) == 0 &&
+                         (out_type == tg::OUT_BF16 || out_type == tg::OUT_F16);
+    Schedule s = choose_dense(M, N, K, block_scaled, fast_layout, pipe_ok, cfg, ncfg, ws_free);
 
     tg::GemmParams p{};
     p.A = reinterpret_cast<const uint8_t*>(a->ptr);
@@ -408,9 +431,14 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
         if (block_scaled && p.As) pc.As = p.As + r0 * kblocks;
         pc.M = (int)rows;
         if (rows != M && s.split_k > 1) { pc.split_k = 1; pc.ksteps_per_split = (int)kblocks; }
-        const int gx = (int)(cdiv(rows, s.bm) * cdiv(N, s.bn));
+        int gx = (int)(cdiv(rows, s.bm) * cdiv(N, s.bn));
+        if (s.kernel == 4) {  // persistent: one workgroup per compute unit
+            const int cus = compute_units(device_id);
+            if (gx > cus) gx = cus;
+        }
         const bool split = pc.split_k > 1;
-        hipError_t e = block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
+        hipError_t e = s.kernel == 4 ? tg::run_pipe(8, s.waves, pc, gx, stream)
+                     : block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
                                     : tg::run_tile_per_tensor(s.bm, s.bn, split, pc, gx, pc.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "tiled kernel launch failed: %s", hipGetErrorString(e));
         if (split && tg::run_splitk_reduce(pc, block_scaled, stream) != hipSuccess)
