@@ -139,6 +139,22 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
                         int32_t mul_routed_weight, int32_t top_k, int32_t block_m,
                         const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream);
 
+/*
+ * moe_align_block_size: group the (token, slot) pairs of a top-k routing by expert and pad every
+ * group to a multiple of block_size, in one launch and without host synchronisation.
+ * Replaces src/tilegym/ops/cutile/moe_align_block.py:205-268 (four launches) and
+ * src/tilegym/ops/tilecpp/moe_align_block.py:274-335; arithmetic of src/tilegym/ops/moe_interface.py:30-79.
+ * topk_ids: any shape, i32 or i64, numel pairs, expert labels in [0, num_experts) (others are skipped).
+ * sorted_token_ids (numel + num_experts * (block_size - 1)) i32: pair indices grouped by expert,
+ *   ascending inside an expert; every unused position holds numel.
+ * expert_ids (ceil(that / block_size)) i32; num_tokens_post_padded (1) i32; cumsum (num_experts + 1) i32
+ * (padded prefix sums); max_expert_count (1) i32.  num_experts <= 512 (rc -6 beyond).
+ */
+int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
+                                const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
+                                const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,
+                                const tg_tensor* max_expert_count, int32_t device_id, uint64_t hip_stream);
+
 /* The schedule the most recent GEMM call on this host thread chose: fills out[0..n) with the
  * TG_CFG_* slots (kernel, BLOCK_M, BLOCK_N, SPLIT_K, ROW_GROUPS, WAVES).  Returns slots written. */
 int32_t tg_last_config(int32_t* out, int32_t n);

@@ -118,6 +118,28 @@ def test_grouped_argument_validation():
     assert moe(expert_ids=torch.zeros(1, dtype=torch.int32)) == -6
 
 
+def test_moe_align_argument_validation():
+    L = _lib.load()
+
+    def align(ids, bs, E, sorted_n=None, cum_n=None, dtype=torch.int32):
+        n = ids.numel()
+        cap = n + E * (bs - 1) if bs > 0 else n
+        outs = [torch.zeros(cap if sorted_n is None else sorted_n, dtype=dtype), torch.zeros(max(1, -(-cap // max(bs, 1))), dtype=torch.int32),
+                torch.zeros(1, dtype=torch.int32), torch.zeros(E + 1 if cum_n is None else cum_n, dtype=torch.int32),
+                torch.zeros(1, dtype=torch.int32)]
+        ds = [_lib.make_tensor_desc(t) for t in [ids] + outs]
+        return L.tg_moe_align_block_size(ctypes.byref(ds[0]), bs, E, *[ctypes.byref(d) for d in ds[1:]], 0, 0)
+
+    ids = torch.zeros(4, 3, dtype=torch.int64)
+    assert align(ids, 0, 4) == -6                      # block size
+    assert align(ids, 4, 0) == -6 and align(ids, 4, 513) == -6
+    assert align(ids.float(), 4, 4) == -2              # id dtype
+    assert align(ids, 4, 4, dtype=torch.int64) == -2   # output dtype
+    assert align(ids, 4, 4, sorted_n=10) == -6         # capacity numel + E*(bs-1)
+    assert align(ids, 4, 4, cum_n=4) == -6
+    assert b"sorted_token_ids" in L.tg_last_error() or b"cumsum" in L.tg_last_error()
+
+
 def test_workspace_bytes_and_cfg():
     L = _lib.load()
     cfg, n = _lib.make_cfg(None)

@@ -434,6 +434,31 @@ def test_moe_fc2_shape_top_k_1(device):
     check(C, ref, what="moe fc2")
 
 
+@pytest.mark.parametrize("T,top_k,E,bs,dtype", [(4, 3, 4, 4, torch.int64), (1, 1, 1, 16, torch.int32), (77, 6, 64, 16, torch.int64),
+                                                 (4096, 6, 64, 128, torch.int32), (1000, 2, 512, 64, torch.int64),
+                                                 (333, 8, 8, 1, torch.int32), (50, 4, 600, 32, torch.int64)])
+def test_moe_align_kernel_matches_oracle(device, T, top_k, E, bs, dtype):
+    """All five outputs, bit for bit, against the oracle (stable order inside an expert, sentinel
+    fill, padded prefix sums); empty experts, one expert, block size 1, int32 and int64 ids, and
+    more experts than the one-launch kernel takes (torch device ops then)."""
+    g = _g(T + E)
+    ids = torch.randint(0, E, (T, top_k), generator=g)
+    if E >= 8:
+        ids[ids == 3] = 5  # an expert without tokens
+    want = R.moe_align_block_size_ref(ids, bs, E)
+    got = moe_align_block_size(ids.to(dtype).to(device), bs, E)
+    names = ["sorted_ids", "expert_ids", "num_tokens_post_padded", "cumsum", "max_expert_count"]
+    nblk_used = int(want[2]) // bs
+    for name, w, gt in zip(names, want, got):
+        w, gt = w.reshape(-1).long(), gt.reshape(-1).long().cpu()
+        if name == "expert_ids":  # entries past the padded total are unspecified in the reference
+            w, gt = w[:nblk_used], gt[:nblk_used]
+        assert w.numel() == gt.numel(), name
+        assert torch.equal(w, gt), f"{name} differs"
+    again = moe_align_block_size(ids.to(dtype).to(device), bs, E)
+    assert all(torch.equal(a, b) for a, b in zip(got, again))
+
+
 # ----------------------------------------------------------------------------- group_gemm (list form)
 def test_group_gemm_list_form(device):
     g = _g(12)

@@ -100,6 +100,8 @@ def load():
     L.tg_fp8_moe_gemm.restype = ctypes.c_int32
     L.tg_fp8_moe_gemm.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_int32, ctypes.c_int32,
                                   ctypes.c_int32, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_moe_align_block_size.restype = ctypes.c_int32
+    L.tg_moe_align_block_size.argtypes = [P, ctypes.c_int32, ctypes.c_int32, P, P, P, P, P, ctypes.c_int32, ctypes.c_uint64]
     if L.tg_abi_version() != 1:
         raise RuntimeError(f"libtilegym_hip.so ABI version {L.tg_abi_version()} != 1")
     _lib = L
@@ -232,3 +234,30 @@ def fp8_moe_gemm(c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids, expe
     rc = L.tg_fp8_moe_gemm(*[_ref(d) for d in ds], int(bool(mul_routed_weight)), int(top_k),
                            int(block_m), cfg, ncfg, dev, _stream_handle(a))
     check_rc(rc, "tg_fp8_moe_gemm")
+
+
+MOE_ALIGN_MAX_EXPERTS = 512
+
+
+def moe_align_block_size(topk_ids, block_size: int, num_experts: int):
+    """One-launch device alignment (tg_moe_align_block_size); allocates the five outputs with the
+    worst-case, data-independent sizes of src/tilegym/ops/cutile/moe_align_block.py:252-268."""
+    L = load()
+    ids = topk_ids if topk_ids.dtype in (torch.int32, torch.int64) else topk_ids.to(torch.int64)
+    ids = ids.contiguous()
+    dev = ids.device
+    numel = ids.numel()
+    cap = numel + num_experts * (block_size - 1)
+    nblk = -(-cap // block_size)
+    sorted_ids = torch.empty(cap, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(max(nblk, 1), dtype=torch.int32, device=dev)[:nblk]
+    post = torch.empty(1, dtype=torch.int32, device=dev)
+    cumsum = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+    mx = torch.empty(1, dtype=torch.int32, device=dev)
+    rc = L.tg_moe_align_block_size(_ref(make_tensor_desc(ids)), int(block_size), int(num_experts),
+                                   _ref(make_tensor_desc(sorted_ids)), _ref(make_tensor_desc(expert_ids)),
+                                   _ref(make_tensor_desc(post)), _ref(make_tensor_desc(cumsum)), _ref(make_tensor_desc(mx)),
+                                   _device_index(ids), _stream_handle(ids))
+    check_rc(rc, "tg_moe_align_block_size")
+    return sorted_ids, expert_ids, post, cumsum, mx
+

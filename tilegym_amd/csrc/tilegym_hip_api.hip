@@ -628,4 +628,40 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
     return TG_OK;
 }
 
+int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
+                                const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
+                                const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,
+                                const tg_tensor* max_expert_count, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(topk_ids, "topk_ids", -1)) || (rc = check_tensor(sorted_token_ids, "sorted_token_ids", 1)) ||
+        (rc = check_tensor(expert_ids, "expert_ids", 1)) || (rc = check_tensor(num_tokens_post_padded, "num_tokens_post_padded", -1)) ||
+        (rc = check_tensor(cumsum, "cumsum", 1)) || (rc = check_tensor(max_expert_count, "max_expert_count", -1)))
+        return rc;
+    if (topk_ids->dtype != TG_I32 && topk_ids->dtype != TG_I64) return fail(TG_ERR_DTYPE, "topk_ids must be int32 or int64");
+    const tg_tensor* outs[5] = {sorted_token_ids, expert_ids, num_tokens_post_padded, cumsum, max_expert_count};
+    for (const tg_tensor* t : outs)
+        if (t->dtype != TG_I32) return fail(TG_ERR_DTYPE, "outputs must be int32");
+    if (block_size < 1) return fail(TG_ERR_INVALID, "block_size must be positive");
+    if (num_experts < 1 || num_experts > 512) return fail(TG_ERR_INVALID, "num_experts must be in [1, 512], got %d", num_experts);
+    const int64_t n = numel(topk_ids);
+    const int64_t cap = n + (int64_t)num_experts * (block_size - 1);
+    if (cap > INT32_MAX) return fail(TG_ERR_INVALID, "too many (token, slot) pairs");
+    const int64_t nblk = cdiv(cap, block_size);
+    if (numel(sorted_token_ids) != cap) return fail(TG_ERR_INVALID, "sorted_token_ids must have %lld elements", (long long)cap);
+    if (numel(expert_ids) < nblk) return fail(TG_ERR_INVALID, "expert_ids must have at least %lld elements", (long long)nblk);
+    if (numel(num_tokens_post_padded) < 1 || numel(max_expert_count) < 1) return fail(TG_ERR_INVALID, "scalar outputs need one element");
+    if (numel(cumsum) != num_experts + 1) return fail(TG_ERR_INVALID, "cumsum must have num_experts + 1 elements");
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipError_t e = tg::run_moe_align(reinterpret_cast<const void*>(topk_ids->ptr), topk_ids->dtype == TG_I64, (int)n, num_experts,
+                                     block_size, reinterpret_cast<int*>(sorted_token_ids->ptr), (int)cap,
+                                     reinterpret_cast<int*>(expert_ids->ptr), (int)numel(expert_ids),
+                                     reinterpret_cast<int*>(num_tokens_post_padded->ptr), reinterpret_cast<int*>(cumsum->ptr),
+                                     reinterpret_cast<int*>(max_expert_count->ptr), reinterpret_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "moe_align launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
+
 }  // extern "C"

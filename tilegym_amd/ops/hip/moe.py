@@ -46,10 +46,20 @@ def invoke_fused_moe_kernel(A, B, C, A_scale, B_scale, topk_weights, topk_ids, s
 
 @register_impl("moe_align_block_size", backend="hip")
 def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int):
-    """Device-side token alignment in torch ops, no host synchronisation; same outputs and buffer
-    sizes as src/tilegym/ops/cutile/moe_align_block.py:205-268: (sorted_ids[numel + E*(bs-1)]
-    pre-filled with the sentinel numel, expert_ids[ceil(that/bs)], num_tokens_post_pad[1],
-    cumsum[E+1] of padded counts, max_expert_cnt[1]).  Stable within an expert."""
+    """Device-side token alignment, no host synchronisation; same outputs and buffer sizes as
+    src/tilegym/ops/cutile/moe_align_block.py:205-268: (sorted_ids[numel + E*(bs-1)] pre-filled
+    with the sentinel numel, expert_ids[ceil(that/bs)], num_tokens_post_pad[1], cumsum[E+1] of
+    padded counts, max_expert_cnt[1]).  Stable within an expert.  One HIP launch for up to 512
+    experts; beyond that the same result from torch device ops."""
+    if not topk_ids.is_cuda:
+        raise RuntimeError("the hip backend works on device tensors only; topk_ids is on " + str(topk_ids.device))
+    if num_experts <= _lib.MOE_ALIGN_MAX_EXPERTS and topk_ids.numel() > 0:
+        return _lib.moe_align_block_size(topk_ids, block_size, num_experts)
+    return _moe_align_torch_ops(topk_ids, block_size, num_experts)
+
+
+def _moe_align_torch_ops(topk_ids: torch.Tensor, block_size: int, num_experts: int):
+    """The same five outputs from torch ops on the tensor's device (used beyond 512 experts)."""
     dev = topk_ids.device
     flat = topk_ids.reshape(-1).to(torch.int64)
     numel = flat.numel()
