@@ -211,7 +211,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="all", choices=["prefill", "decode", "block", "moe", "all"])
+    ap.add_argument("--workload", default="all", choices=["prefill", "decode", "block", "moe", "quant", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time microsecond kernels with plain launches")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -322,9 +322,37 @@ def main():
             torch.cuda.empty_cache()
         detail["moe_grouped"] = shapes
 
-    if "value" not in out:  # block / moe only
+    if args.workload in ("quant", "all"):
+        # the producers either side of the GEMM: 1x128 activation quantizer (HBM-bound) and moe_align_block_size
+        shapes = []
+        for (M, K) in ((8192, 4096), (8192, 14336), (24576, 2048)):
+            xs = [torch.randn(M, K, device=device, dtype=torch.bfloat16) for _ in range(_copies_for(M * K * 3))]
+            fn = lambda i: _lib.fp8_quant_1x128(xs[i % len(xs)], 0.0, False)  # noqa: E731
+            for w in range(max(1, args.warmup)):
+                fn(w)
+            n = max(args.steps, 32)
+            us = _events_ms(fn, n, stream) * 1e3 / n
+            nbytes = M * K * 3 + M * (K // 128) * 4
+            shapes.append({"name": f"act_quant_1x128_bf16_{M}x{K}", "kernel": "act_quant_1x128_kernel", "us": round(us, 2),
+                           "gbs": round(nbytes / us * 1e-3, 1), "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
+                           "note": "includes the torch allocation of the two outputs"})
+            del xs
+            torch.cuda.empty_cache()
+        ids = W.moe_routing(4096, 64, 6, seed=0)[1].to(device)
+        fn = lambda i: _lib.moe_align_block_size(ids, 128, 64)  # noqa: E731
+        for w in range(max(1, args.warmup)):
+            fn(w)
+        n = max(args.steps, 32)
+        us = _events_ms(fn, n, stream) * 1e3 / n
+        shapes.append({"name": "moe_align_block_size_4096x6_E64_bs128", "kernel": "moe_align_kernel", "us": round(us, 2),
+                       "note": "one launch + five torch.empty"})
+        detail["producers"] = shapes
+
+    if "value" not in out:  # block / moe / quant only
         first = next(iter(detail.values()))
         dom = max(first, key=lambda s: s["us"])
+        dom.setdefault("tflops", 0.0)
+        dom.setdefault("frac_mfma", 0.0)
         out.update({"value": dom["tflops"], "ms_per_step": round(dom["us"] * 1e-3, 5),
                     "roofline": {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                                  "frac": dom["frac_mfma"], "traffic": None, "shape": dom["name"]}})
@@ -341,7 +369,8 @@ def main():
                                 "decode": "config 2: Llama-3.1-8B decode projections, M in {1,8,16,64}",
                                 "block": "config 4: block-scaled 12288x5120 / 5120x12288, M in {16,4096}",
                                 "moe": "config 5: DeepSeek-V2-Lite MoE grouped GEMMs",
-                                "all": "config 3 (headline) + configs 2, 4, 5"}[args.workload],
+                                "quant": "producers: 1x128 activation quantizer, moe_align_block_size",
+                                "all": "config 3 (headline) + configs 2, 4, 5 + producers"}[args.workload],
                    "device": props.name, "compute_units": props.multi_processor_count},
     }
     line.update(out)

@@ -155,6 +155,19 @@ int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, i
                                 const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,
                                 const tg_tensor* max_expert_count, int32_t device_id, uint64_t hip_stream);
 
+/*
+ * Per-token 1 x 128 FP8 quantizer (the producer of scale_a for the block-scaled GEMMs):
+ *   scales[m, kb] = amax(x[m, 128*kb : 128*kb+128]) / 448      (rule 0: an all-zero group gets 1.0;
+ *                                                               rule 1: amax is first clamped below by eps)
+ *   q = e4m3fn(clamp(x / scale, -448, 448)), round to nearest even, IEEE divisions.
+ * Replaces src/tilegym/suites/unsloth/cutile/fp8.py:370-385 (act_quant, rule 0) and the row-major fp8 case of
+ * src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:152-272 (rule 1).
+ * x (..., K) bf16 / f16 / f32 contiguous, K % 128 == 0, 16-byte aligned; q same shape e4m3fn;
+ * scales (..., K/128) f32 contiguous.
+ */
+int32_t tg_fp8_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x, float eps,
+                           int32_t rule, int32_t device_id, uint64_t hip_stream);
+
 /* The schedule the most recent GEMM call on this host thread chose: fills out[0..n) with the
  * TG_CFG_* slots (kernel, BLOCK_M, BLOCK_N, SPLIT_K, ROW_GROUPS, WAVES).  Returns slots written. */
 int32_t tg_last_config(int32_t* out, int32_t n);

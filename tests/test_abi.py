@@ -140,6 +140,24 @@ def test_moe_align_argument_validation():
     assert b"sorted_token_ids" in L.tg_last_error() or b"cumsum" in L.tg_last_error()
 
 
+def test_quantizer_argument_validation():
+    L = _lib.load()
+
+    def quant(x, q=None, s=None, rule=0):
+        q = torch.zeros(x.shape, dtype=FP8) if q is None else q
+        s = torch.zeros(x.shape[:-1] + (max(x.shape[-1] // 128, 1),)) if s is None else s
+        ds = [_lib.make_tensor_desc(t) for t in (q, s, x)]
+        return L.tg_fp8_quant_1x128(*[ctypes.byref(d) for d in ds], 1e-10, rule, 0, 0)
+
+    x = torch.zeros(4, 256, dtype=torch.bfloat16)
+    assert quant(torch.zeros(4, 200, dtype=torch.bfloat16)) == -6      # K % 128
+    assert quant(x.to(torch.int32)) == -2
+    assert quant(x, q=torch.zeros(4, 256, dtype=torch.bfloat16)) == -2
+    assert quant(x, s=torch.zeros(4, 3)) == -6
+    assert quant(x, rule=2) == -6
+    assert quant(torch.zeros(0, 256, dtype=torch.bfloat16)) == 0       # nothing to do, no device needed
+
+
 def test_workspace_bytes_and_cfg():
     L = _lib.load()
     cfg, n = _lib.make_cfg(None)

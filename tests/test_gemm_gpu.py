@@ -459,6 +459,47 @@ def test_moe_align_kernel_matches_oracle(device, T, top_k, E, bs, dtype):
     assert all(torch.equal(a, b) for a, b in zip(got, again))
 
 
+# ----------------------------------------------------------------------------- activation quantizers
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 128), (7, 384), (3, 5, 256), (4096, 2048)])
+def test_act_quant_kernels_bit_exact(device, dtype, shape):
+    """Codes and scales, bit for bit, against the oracle: both scale rules, an all-zero group,
+    values that hit +-448, tiny groups (subnormal codes), ties."""
+    from tilegym_amd.suites.flashinfer.ops import per_token_group_quant_8bit
+    from tilegym_amd.suites.unsloth.ops import act_quant
+
+    g = _g(sum(shape))
+    x = torch.randn(shape, generator=g) * torch.exp(torch.randn(shape[:-1] + (1,), generator=g) * 3)
+    flat = x.reshape(-1, 128)
+    flat[0] = 0.0                                   # all-zero group
+    if flat.shape[0] > 2:
+        flat[1] *= 1e-12                            # amax below the flashinfer eps
+        flat[2, :8] = torch.tensor([448.0, -448.0, 224.0, 0.5, 17.0, 19.0, 21.0, 23.0])
+    x = x.clamp(-6e4, 6e4).to(dtype)  # finite in f16
+    for rule, fn, eps in (("unsloth", lambda t: act_quant(t, 128), None),
+                          ("flashinfer", lambda t: per_token_group_quant_8bit(t, 128), 1e-10)):
+        q_ref, s_ref = R.quantize_act_1x128(x, 128, eps)
+        q, s = fn(x.to(device))
+        assert q.dtype == FP8 and s.dtype == torch.float32 and q.shape == x.shape and s.shape == s_ref.shape
+        assert torch.equal(s.cpu().view(torch.int32), s_ref.view(torch.int32)), f"{rule}: scales differ"
+        bad = q.cpu().view(torch.uint8) != q_ref.view(torch.uint8)
+        assert not bad.any(), f"{rule}: {int(bad.sum())} of {bad.numel()} codes differ"
+
+
+def test_quantize_then_gemm_end_to_end(device):
+    """bf16 activations -> HIP quantizer -> block-scaled GEMM, against the oracle on the same bf16 input."""
+    from tilegym_amd.suites.unsloth.ops import act_quant
+
+    g = _g(5)
+    x = torch.randn(96, 512, generator=g).to(torch.bfloat16)
+    case = W.block_scaled_case(8, 384, 512, seed=3)
+    qa_ref, sa_ref = R.quantize_act_1x128(x, 128, None)
+    ref = R.ref_w8a8_block_fp8_matmul(qa_ref, case.b, sa_ref, case.scale_b, None, torch.bfloat16)
+    qa, sa = act_quant(x.to(device), 128)
+    out = w8a8_block_fp8_matmul(qa, case.b.to(device), sa, case.scale_b.to(device), None, torch.bfloat16)
+    check(out, ref, what="quantize + block-scaled GEMM")
+
+
 # ----------------------------------------------------------------------------- group_gemm (list form)
 def test_group_gemm_list_form(device):
     g = _g(12)

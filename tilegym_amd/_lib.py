@@ -102,6 +102,8 @@ def load():
                                   ctypes.c_int32, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     L.tg_moe_align_block_size.restype = ctypes.c_int32
     L.tg_moe_align_block_size.argtypes = [P, ctypes.c_int32, ctypes.c_int32, P, P, P, P, P, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_quant_1x128.restype = ctypes.c_int32
+    L.tg_fp8_quant_1x128.argtypes = [P, P, P, ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     if L.tg_abi_version() != 1:
         raise RuntimeError(f"libtilegym_hip.so ABI version {L.tg_abi_version()} != 1")
     _lib = L
@@ -260,4 +262,16 @@ def moe_align_block_size(topk_ids, block_size: int, num_experts: int):
                                    _device_index(ids), _stream_handle(ids))
     check_rc(rc, "tg_moe_align_block_size")
     return sorted_ids, expert_ids, post, cumsum, mx
+
+
+def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = False):
+    """(q e4m3fn like x, scales (..., K/128) f32) through tg_fp8_quant_1x128."""
+    L = load()
+    x = x.contiguous()
+    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty(x.shape[:-1] + (x.shape[-1] // 128,), dtype=torch.float32, device=x.device)
+    rc = L.tg_fp8_quant_1x128(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+                              float(eps), 1 if flashinfer_rule else 0, _device_index(x), _stream_handle(x))
+    check_rc(rc, "tg_fp8_quant_1x128")
+    return q, scales
 

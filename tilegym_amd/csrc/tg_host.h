@@ -32,6 +32,9 @@ hipError_t run_generic(const GenericParams& p, hipStream_t s);
 // moe_align_block_size in one launch (num_experts <= 512); ids are int32 or int64
 hipError_t run_moe_align(const void* ids, int ids_are_i64, int numel, int E, int block_size, int* sorted_ids, int cap,
                          int* expert_ids, int nblk, int* num_post_pad, int* cumsum, int* max_cnt, hipStream_t s);
+// per-token 1x128 e4m3 quantizer; x_type uses the OutType numbering (f32/f16/bf16)
+hipError_t run_act_quant_1x128(const void* x, int x_type, uint8_t* q, float* scales, int64_t groups, float eps,
+                               int flashinfer_rule, hipStream_t s);
 // dst (cols, rows) <- transpose of src (rows, cols), one byte per element
 hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s);
 

@@ -664,4 +664,30 @@ int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, i
 }
 
 
+int32_t tg_fp8_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x, float eps,
+                           int32_t rule, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(x, "x", -1)) || (rc = check_tensor(q, "q", -1)) || (rc = check_tensor(scales, "scales", -1))) return rc;
+    const int x_type = out_type_of(x->dtype);
+    if (x_type < 0) return fail(TG_ERR_DTYPE, "x must be bf16, f16 or f32");
+    if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
+    if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
+    if (rule != 0 && rule != 1) return fail(TG_ERR_INVALID, "rule must be 0 or 1");
+    if (x->ndim < 1) return fail(TG_ERR_INVALID, "x needs at least one dimension");
+    const int64_t K = x->shape[x->ndim - 1], n = numel(x);
+    if (K % 128 != 0) return fail(TG_ERR_INVALID, "the last dimension (%lld) must be a multiple of 128", (long long)K);
+    if (numel(q) != n) return fail(TG_ERR_INVALID, "q must have the shape of x");
+    if (numel(scales) != n / 128) return fail(TG_ERR_INVALID, "scales must have %lld elements", (long long)(n / 128));
+    if (!aligned16(x->ptr) || (q->ptr & 7) != 0) return fail(TG_ERR_INVALID, "x must be 16-byte and q 8-byte aligned");
+    if (n == 0) return TG_OK;
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipError_t e = tg::run_act_quant_1x128(reinterpret_cast<const void*>(x->ptr), x_type, reinterpret_cast<uint8_t*>(q->ptr),
+                                           reinterpret_cast<float*>(scales->ptr), n / 128, eps, rule,
+                                           reinterpret_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "quantizer launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
 }  // extern "C"

@@ -1,5 +1,7 @@
-"""FP8 (e4m3fn) quantizers on the device, in torch: the producers of the scale layouts the
-GEMMs consume.  Every quantizer clamps to +-448 before the cast (torch's cast does not
+"""FP8 (e4m3fn) quantizers: the producers of the scale layouts the GEMMs consume.  The per-token
+1 x 128 activation quantizers run as one HIP launch for device tensors (bf16 / f16 / f32,
+group size 128); the other forms, and host tensors (synthetic workload generation), use the same
+arithmetic in torch ops.  Every quantizer clamps to +-448 before the cast (torch's cast does not
 saturate) and divides with IEEE division, as the reference's kernels do
 (src/tilegym/suites/unsloth/cutile/fp8.py:105-116,
 src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:52-66)."""
@@ -12,6 +14,11 @@ import torch
 
 FP8 = torch.float8_e4m3fn
 FP8_MAX = 448.0
+
+
+def _hip_1x128_ok(x: torch.Tensor, group: int) -> bool:
+    return (x.is_cuda and group == 128 and x.numel() > 0 and x.dtype in (torch.bfloat16, torch.float16, torch.float32)
+            and x.data_ptr() % 16 == 0)
 
 
 def quantize_per_tensor(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -27,6 +34,9 @@ def act_quant(x: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, tor
     """Per-token 1 x block_size quantization; all-zero block -> scale 1.0
     (src/tilegym/suites/unsloth/cutile/fp8.py:370-385)."""
     assert x.shape[-1] % block_size == 0, "last dim must be divisible by block_size"
+    if _hip_1x128_ok(x, block_size):
+        from . import _lib
+        return _lib.fp8_quant_1x128(x, 0.0, False)
     xb = x.contiguous().float().reshape(-1, block_size)
     amax = xb.abs().amax(dim=-1, keepdim=True)
     s = amax / FP8_MAX
@@ -40,6 +50,9 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128, eps: float
     """Per (token, group) quantization with amax clamped below by eps, row-major scales
     (src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:152-272)."""
     assert x.shape[-1] % group_size == 0 and x.is_contiguous()
+    if not scale_ue8m0 and _hip_1x128_ok(x, group_size):
+        from . import _lib
+        return _lib.fp8_quant_1x128(x, eps, True)
     xb = x.float().reshape(-1, group_size)
     amax = xb.abs().amax(dim=-1, keepdim=True).clamp(min=eps)
     s = amax / FP8_MAX
