@@ -94,24 +94,30 @@ __global__ void __launch_bounds__(64 * kAlignWaves) moe_align_kernel(const IdT* 
     __syncthreads();
 
     // pass 2: stable scatter.  `mine[e]` is this wave's next free rank inside expert e's group.
+    // Lanes holding the same expert are found without a loop over the distinct experts: one ballot
+    // per bit of the expert label, combined into the mask of lanes that agree with this lane on
+    // every bit.  The lowest lane of each such set advances the cursor.
+    int nbits = 0;
+    while ((1 << nbits) < E) ++nbits;
+    const unsigned long long below = (1ull << lane) - 1ull;
     for (int i0 = lo; i0 < hi; i0 += 64) {
         const int i = i0 + lane;
-        long long e = -1;
-        if (i < hi) e = (long long)ids[i];
-        bool todo = e >= 0 && e < E;
-        while (true) {
-            const unsigned long long active = __ballot(todo);
-            if (!active) break;
-            const int leader = __ffsll((long long)active) - 1;
-            const int e0 = __shfl((int)e, leader);
-            const unsigned long long same = __ballot(todo && (int)e == e0);
-            const int base = mine[e0];  // every lane reads the same word
-            if (todo && (int)e == e0) {
-                const int rank = __popcll(same & ((1ull << lane) - 1ull));
-                sorted_ids[pad_start[e0] + base + rank] = i;
-                todo = false;
-            }
-            if (lane == leader) mine[e0] = base + __popcll(same);
+        long long e64 = -1;
+        if (i < hi) e64 = (long long)ids[i];
+        const bool valid = e64 >= 0 && e64 < E;
+        const int e = valid ? (int)e64 : 0;
+        unsigned long long same = __ballot(valid);
+        for (int b = 0; b < nbits; ++b) {
+            const unsigned long long m = __ballot((e >> b) & 1);
+            same &= ((e >> b) & 1) ? m : ~m;
+        }
+        if (valid) {
+            const int base = mine[e];
+            const int rank = __popcll(same & below);
+            sorted_ids[pad_start[e] + base + rank] = i;
+            // every lane of the set has read the cursor before its first lane rewrites it: the
+            // read and the write below are separate LDS instructions of one wave, executed in order
+            if (rank == 0) mine[e] = base + __popcll(same);
         }
     }
 }
