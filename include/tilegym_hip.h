@@ -168,6 +168,22 @@ int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, i
 int32_t tg_fp8_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x, float eps,
                            int32_t rule, int32_t device_id, uint64_t hip_stream);
 
+/*
+ * Between the two MoE GEMMs, one launch: act = silu(x[:, :I]) * x[:, I:], rounded to x's 16-bit type
+ * (the reference's intermediate cache, src/tilegym/ops/moe_interface.py:206-210,272-277; silu_and_mul:
+ * src/tilegym/ops/ops.py:172-193), then quantized 1 x 128 (all-zero group -> scale 1.0).  The reference
+ * casts the activation to fp8 with an all-ones scale (moe_interface.py:279-288); this gives the second
+ * GEMM a real a2_scale.  x (R, 2I) bf16/f16 contiguous, I % 8 == 0; q (R, I) e4m3fn; scales (R, ceil(I/128)) f32.
+ */
+int32_t tg_silu_mul_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x,
+                                int32_t device_id, uint64_t hip_stream);
+
+/*
+ * Top-k combine: out[t, :] = sum_j x[t, j, :] (fp32 sum, one rounding), src/tilegym/ops/moe_interface.py:308-321.
+ * x (T, top_k, H) and out (T, H) bf16 or f16 (same type), contiguous, H % 8 == 0, 16-byte aligned.
+ */
+int32_t tg_moe_sum(const tg_tensor* out, const tg_tensor* x, int32_t device_id, uint64_t hip_stream);
+
 /* The schedule the most recent GEMM call on this host thread chose: fills out[0..n) with the
  * TG_CFG_* slots (kernel, BLOCK_M, BLOCK_N, SPLIT_K, ROW_GROUPS, WAVES).  Returns slots written. */
 int32_t tg_last_config(int32_t* out, int32_t n);

@@ -328,6 +328,39 @@ def ref_fused_moe_gemm(A, B, A_scale, B_scale, topk_weights, topk_ids, mul_route
 # ----------------------------------------------------------------------------
 # comparison (tolerance "relative to output scale")
 # ----------------------------------------------------------------------------
+def ref_silu_mul_quant(x: torch.Tensor):
+    """act = silu(x[:, :I]) * x[:, I:] in fp32, rounded to x's dtype (the reference's intermediate
+    cache, src/tilegym/ops/moe_interface.py:206-210,272-277; silu_and_mul: src/tilegym/ops/ops.py:172-193),
+    then 1 x 128 quantization with a possibly partial last group."""
+    inter = x.shape[1] // 2
+    g, u = x[:, :inter].float(), x[:, inter:].float()
+    act = ((g / (1.0 + torch.exp(-g))) * u).to(x.dtype)
+    pad = (-inter) % 128
+    ap = torch.nn.functional.pad(act.float(), (0, pad))
+    q, s = quantize_act_1x128(ap, 128, None)
+    return q[:, :inter].contiguous(), s, act
+
+
+def ref_fused_experts_fp8(hidden, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, a1_scale=None):
+    """The FP8 MoE layer token by token: quantize -> block-scaled GEMM with the token's experts ->
+    silu * up -> re-quantize -> block-scaled GEMM x routed weight -> fp32 sum over the slots.
+    Order of operations of src/tilegym/ops/moe_interface.py:230-321 and of the torch MoE oracle
+    (tests/ops/test_moe.py:19-66); the FP8 branch itself is covered by no reference test
+    (PARITY UNPINNED against the reference; pinned here by being a composition of the pinned
+    per-op oracles above)."""
+    T, H = hidden.shape
+    k = topk_ids.shape[1]
+    out_dtype = torch.bfloat16 if hidden.dtype == torch.bfloat16 else torch.float16
+    if hidden.dtype == FP8:
+        xq, xs = hidden, a1_scale
+    else:
+        xq, xs = quantize_act_1x128(hidden, 128, None)
+    h1 = ref_fused_moe_gemm(xq, w1, xs, w1_scale, topk_weights, topk_ids, False, k, out_dtype=out_dtype)
+    q2, s2, _ = ref_silu_mul_quant(h1.reshape(T * k, -1))
+    h2 = ref_fused_moe_gemm(q2, w2, s2, w2_scale, topk_weights, topk_ids, True, 1, out_dtype=out_dtype)
+    return h2.reshape(T, k, H).float().sum(dim=1).to(out_dtype)
+
+
 def compare_to_oracle(out: torch.Tensor, ref: torch.Tensor, rtol=2e-2, atol=2e-2):
     """|out - ref| <= atol*sigma_ref + rtol*|ref|, sigma_ref = std of the oracle output.
     Returns (ok, report) with the fields the reference's compare_tensors prints

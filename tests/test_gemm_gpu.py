@@ -500,6 +500,97 @@ def test_quantize_then_gemm_end_to_end(device):
     check(out, ref, what="quantize + block-scaled GEMM")
 
 
+# ----------------------------------------------------------------------------- the MoE layer around the GEMMs
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("R_,I", [(5, 128), (64, 1408), (33, 200), (1, 8)])
+def test_silu_mul_quant_kernel(device, dtype, R_, I):
+    """Dequantized activation within one 16-bit ulp of the oracle's and scales equal to 1e-6 relative (device
+    and host exp differ in the last bit now and then, which can move the 16-bit rounding of one value)."""
+    g = _g(R_ + I)
+    x = (torch.randn(R_, 2 * I, generator=g) * 2).to(dtype)
+    x[0, :8] = 0
+    q_ref, s_ref, act = R.ref_silu_mul_quant(x)
+    q, s = _lib.silu_mul_quant_1x128(x.to(device))
+    assert q.shape == q_ref.shape and s.shape == s_ref.shape
+    assert torch.allclose(s.cpu(), s_ref, rtol=1e-2, atol=0)
+    deq = R.fp8_to_f32(q.cpu()) * s.cpu().repeat_interleave(128, 1)[:, :I]
+    deq_ref = R.fp8_to_f32(q_ref) * s_ref.repeat_interleave(128, 1)[:, :I]
+    step = s_ref.repeat_interleave(128, 1)[:, :I] * 32          # one e4m3 step at the top binade is 32 * scale
+    assert ((deq - deq_ref).abs() <= step + 1e-12).all()
+    same = (q.cpu().view(torch.uint8) == q_ref.view(torch.uint8)).float().mean()
+    assert same > 0.995, f"only {same:.4f} of the codes equal the oracle's"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_moe_sum_kernel(device, dtype):
+    g = _g(8)
+    x = torch.randn(37, 6, 264, generator=g).to(dtype)
+    out = torch.empty(37, 264, dtype=dtype, device=device)
+    _lib.moe_sum(x.to(device), out)
+    acc = x[:, 0].float()
+    for j in range(1, 6):
+        acc = acc + x[:, j].float()
+    assert torch.equal(out.cpu(), acc.to(dtype))
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, "fp8"])
+def test_fused_experts_fp8_small(device, in_dtype):
+    from tilegym_amd.ops import fused_experts_impl, fused_moe
+
+    g = _g(31)
+    T, E, k, H, I = 40, 8, 2, 256, 384
+    dt = torch.bfloat16 if in_dtype == "fp8" else in_dtype
+    hidden = torch.randn(T, H, generator=g).to(dt)
+    w1q, w1s = R.quantize_weight_128x128(torch.randn(E * 2 * I, H, generator=g) * 0.05)
+    w2q, w2s = R.quantize_weight_128x128(torch.randn(E * H, I, generator=g) * 0.05)
+    w1q, w1s = w1q.reshape(E, 2 * I, H), w1s.reshape(E, 2 * I // 128, H // 128)
+    w2q, w2s = w2q.reshape(E, H, I), w2s.reshape(E, H // 128, I // 128)
+    tw, ids = W.moe_routing(T, E, k, seed=4)
+    ids[ids == 5] = 6  # an expert without tokens
+    if in_dtype == "fp8":
+        xq, xs = R.quantize_act_1x128(hidden, 128, None)
+        ref = R.ref_fused_experts_fp8(xq, w1q, w2q, w1s, w2s, tw, ids, a1_scale=xs)
+        # fp8 input: the reference types the output f16 unless the input is bf16 (moe_interface.py:196)
+        out = fused_experts_impl(xq.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device), use_fp8_w8a8=True,
+                                 w1_scale=w1s.to(device), w2_scale=w2s.to(device), a1_scale=xs.to(device))
+        assert out.dtype == torch.float16
+    else:
+        ref = R.ref_fused_experts_fp8(hidden, w1q, w2q, w1s, w2s, tw, ids)
+        out = fused_moe(hidden.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device),
+                        w1_scale=w1s.to(device), w2_scale=w2s.to(device))
+        assert out.dtype == in_dtype
+    # a flipped activation code (host / device exp) moves one input of the second GEMM by one e4m3 step:
+    # within the stated tolerance, not within one output ulp
+    ok, rep = R.compare_to_oracle(out, ref, RTOL, ATOL)
+    assert ok, rep
+    with pytest.raises(NotImplementedError):
+        fused_experts_impl(hidden.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device), use_fp8_w8a8=False)
+
+
+def test_config5_fused_experts_full_size(device):
+    """DeepSeek-V2-Lite MoE layer at full size (4096 tokens, 64 experts, top-6, H 2048, I 1408) through
+    fused_moe; the oracle is evaluated on 24 sampled tokens (a token's output depends on its own row only)."""
+    from tilegym_amd.ops import fused_moe
+
+    up, down = W.moe_grouped_case("gate_up"), W.moe_grouped_case("down")
+    ids, tw = up.extra["topk_ids"], up.extra["topk_weights"]
+    T, H = ids.shape[0], up.b.shape[2]
+    hidden = torch.randn(T, H, generator=_g(9)).to(torch.bfloat16)
+    out = fused_moe(hidden.to(device), up.b.to(device), down.b.to(device), tw.to(device), ids.to(device),
+                    w1_scale=up.b_scale.to(device), w2_scale=down.b_scale.to(device))
+    assert out.shape == (T, H) and torch.isfinite(out.float()).all()
+    rows = _rows_subset(T, 24)
+    ref = R.ref_fused_experts_fp8(hidden[rows], up.b, down.b, up.b_scale, down.b_scale, tw[rows], ids[rows])
+    # Two roundings (16-bit, then e4m3) sit between the GEMMs: an fp32 re-association difference in GEMM1
+    # now and then flips one activation code, i.e. moves one of the 1408 inputs of GEMM2 by an e4m3 step.
+    # Bar for the chained layer: >= 99.9 % of the outputs inside the GEMM tolerance, none beyond 0.1 sigma.
+    ok, rep = R.compare_to_oracle(out[rows.to(device)], ref, RTOL, ATOL)
+    assert rep["matched"] >= 0.999 and rep["max_rel_to_sigma"] <= 0.1, rep
+    again = fused_moe(hidden.to(device), up.b.to(device), down.b.to(device), tw.to(device), ids.to(device),
+                      w1_scale=up.b_scale.to(device), w2_scale=down.b_scale.to(device))
+    assert torch.equal(out, again)
+
+
 # ----------------------------------------------------------------------------- group_gemm (list form)
 def test_group_gemm_list_form(device):
     g = _g(12)

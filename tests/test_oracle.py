@@ -262,6 +262,37 @@ def test_fused_moe_gemm_oracle_against_token_loops():
             assert torch.allclose(got[t, j], want, rtol=1e-5, atol=1e-5)
 
 
+def test_fused_experts_oracle_is_the_composition_of_its_steps():
+    """ref_fused_experts_fp8 against an independent per-token evaluation with dequantized weights:
+    a dropped routed weight, a swapped gate/up half or a wrong slot->expert index fails this."""
+    g = _g(21)
+    T, E, k, H, I = 5, 3, 2, 128, 128
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w1q, w1s = R.quantize_weight_128x128(torch.randn(E * 2 * I, H, generator=g) * 0.1)
+    w2q, w2s = R.quantize_weight_128x128(torch.randn(E * H, I, generator=g) * 0.1)
+    w1q, w1s = w1q.reshape(E, 2 * I, H), w1s.reshape(E, 2, 1)
+    w2q, w2s = w2q.reshape(E, H, I), w2s.reshape(E, 1, 1)
+    ids = torch.tensor([[0, 2], [1, 0], [2, 1], [0, 1], [2, 0]])
+    tw = torch.rand(T, k, generator=g)
+    out = R.ref_fused_experts_fp8(hidden, w1q, w2q, w1s, w2s, tw, ids)
+    xq, xs = R.quantize_act_1x128(hidden, 128, None)
+    x = R.fp8_to_f32(xq) * xs                                   # one group per row
+    want = torch.zeros(T, H)
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            W1 = R.fp8_to_f32(w1q[e]) * w1s[e].repeat_interleave(128, 0)
+            W2 = R.fp8_to_f32(w2q[e]) * w2s[e, 0, 0]
+            h1 = (x[t] @ W1.t()).to(torch.bfloat16).float()
+            act = ((h1[:I] / (1 + torch.exp(-h1[:I]))) * h1[I:]).to(torch.bfloat16)
+            aq, a_s = R.quantize_act_1x128(act.reshape(1, I), 128, None)
+            h2 = ((R.fp8_to_f32(aq) * a_s) @ W2.t() * tw[t, j]).to(torch.bfloat16).float()
+            want[t] += h2[0]
+    assert torch.equal(out, want.to(torch.bfloat16))
+    q, s, act = R.ref_silu_mul_quant(torch.randn(3, 2 * 200, generator=g).to(torch.bfloat16))
+    assert q.shape == (3, 200) and s.shape == (3, 2) and act.shape == (3, 200)
+
+
 def test_compare_to_oracle_flags_errors():
     ref = torch.randn(64, 64, generator=_g(13))
     ok, _ = R.compare_to_oracle(ref.to(torch.bfloat16), ref)

@@ -104,6 +104,10 @@ def load():
     L.tg_moe_align_block_size.argtypes = [P, ctypes.c_int32, ctypes.c_int32, P, P, P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_fp8_quant_1x128.restype = ctypes.c_int32
     L.tg_fp8_quant_1x128.argtypes = [P, P, P, ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_silu_mul_quant_1x128.restype = ctypes.c_int32
+    L.tg_silu_mul_quant_1x128.argtypes = [P, P, P, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_moe_sum.restype = ctypes.c_int32
+    L.tg_moe_sum.argtypes = [P, P, ctypes.c_int32, ctypes.c_uint64]
     if L.tg_abi_version() != 1:
         raise RuntimeError(f"libtilegym_hip.so ABI version {L.tg_abi_version()} != 1")
     _lib = L
@@ -274,4 +278,24 @@ def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = F
                               float(eps), 1 if flashinfer_rule else 0, _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_fp8_quant_1x128")
     return q, scales
+
+
+def silu_mul_quant_1x128(x: torch.Tensor):
+    """x (R, 2I) bf16/f16 -> (q (R, I) e4m3fn, scales (R, ceil(I/128)) f32) through tg_silu_mul_quant_1x128."""
+    L = load()
+    R, two_i = x.shape
+    inter = two_i // 2
+    q = torch.empty(R, inter, dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty(R, -(-inter // 128), dtype=torch.float32, device=x.device)
+    rc = L.tg_silu_mul_quant_1x128(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+                                   _device_index(x), _stream_handle(x))
+    check_rc(rc, "tg_silu_mul_quant_1x128")
+    return q, scales
+
+
+def moe_sum(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out (T, H) <- sum over axis 1 of x (T, top_k, H) through tg_moe_sum."""
+    L = load()
+    rc = L.tg_moe_sum(_ref(make_tensor_desc(out)), _ref(make_tensor_desc(x)), _device_index(x), _stream_handle(x))
+    check_rc(rc, "tg_moe_sum")
 

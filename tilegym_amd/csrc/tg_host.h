@@ -35,6 +35,10 @@ hipError_t run_moe_align(const void* ids, int ids_are_i64, int numel, int E, int
 // per-token 1x128 e4m3 quantizer; x_type uses the OutType numbering (f32/f16/bf16)
 hipError_t run_act_quant_1x128(const void* x, int x_type, uint8_t* q, float* scales, int64_t groups, float eps,
                                int flashinfer_rule, hipStream_t s);
+// q, scales <- quantize_1x128(round16(silu(x[:, :I]) * x[:, I:]));  x (rows, 2I) bf16/f16, I % 8 == 0
+hipError_t run_silu_mul_quant(const void* x, int x_type, uint8_t* q, float* scales, int64_t rows, int I, hipStream_t s);
+// out (tokens, H) <- sum over the top_k axis of x (tokens, top_k, H); bf16/f16, H % 8 == 0
+hipError_t run_moe_sum(const void* x, void* out, int x_type, int64_t tokens, int top_k, int H, hipStream_t s);
 // dst (cols, rows) <- transpose of src (rows, cols), one byte per element
 hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s);
 

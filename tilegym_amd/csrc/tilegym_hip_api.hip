@@ -690,4 +690,49 @@ int32_t tg_fp8_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg
     return TG_OK;
 }
 
+int32_t tg_silu_mul_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x,
+                                int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(x, "x", 2)) || (rc = check_tensor(q, "q", 2)) || (rc = check_tensor(scales, "scales", 2))) return rc;
+    const int x_type = out_type_of(x->dtype);
+    if (x_type != tg::OUT_BF16 && x_type != tg::OUT_F16) return fail(TG_ERR_DTYPE, "x must be bf16 or f16");
+    if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
+    if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
+    const int64_t R = x->shape[0], I = x->shape[1] / 2;
+    if (x->shape[1] % 2 != 0 || I % 8 != 0) return fail(TG_ERR_INVALID, "x must be (R, 2*I) with I a multiple of 8");
+    if (I > INT32_MAX / 4) return fail(TG_ERR_INVALID, "row too long");
+    if (q->shape[0] != R || q->shape[1] != I) return fail(TG_ERR_INVALID, "q must be (%lld, %lld)", (long long)R, (long long)I);
+    if (scales->shape[0] != R || scales->shape[1] != cdiv(I, 128))
+        return fail(TG_ERR_INVALID, "scales must be (%lld, %lld)", (long long)R, (long long)cdiv(I, 128));
+    if (!aligned16(x->ptr) || (q->ptr & 7) != 0) return fail(TG_ERR_INVALID, "x must be 16-byte and q 8-byte aligned");
+    if (R == 0 || I == 0) return TG_OK;
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipError_t e = tg::run_silu_mul_quant(reinterpret_cast<const void*>(x->ptr), x_type, reinterpret_cast<uint8_t*>(q->ptr),
+                                          reinterpret_cast<float*>(scales->ptr), R, (int)I, reinterpret_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "silu_mul_quant launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
+int32_t tg_moe_sum(const tg_tensor* out, const tg_tensor* x, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(x, "x", 3)) || (rc = check_tensor(out, "out", 2))) return rc;
+    const int x_type = out_type_of(x->dtype);
+    if ((x_type != tg::OUT_BF16 && x_type != tg::OUT_F16) || out->dtype != x->dtype)
+        return fail(TG_ERR_DTYPE, "x and out must both be bf16 or both f16");
+    const int64_t T = x->shape[0], k = x->shape[1], H = x->shape[2];
+    if (out->shape[0] != T || out->shape[1] != H) return fail(TG_ERR_INVALID, "out must be (%lld, %lld)", (long long)T, (long long)H);
+    if (k < 1 || k > INT32_MAX || H > INT32_MAX || H % 8 != 0) return fail(TG_ERR_INVALID, "top_k must be positive and H a multiple of 8");
+    if (!aligned16(x->ptr) || !aligned16(out->ptr)) return fail(TG_ERR_INVALID, "x and out must be 16-byte aligned");
+    if (T == 0 || H == 0) return TG_OK;
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipError_t e = tg::run_moe_sum(reinterpret_cast<const void*>(x->ptr), reinterpret_cast<void*>(out->ptr), x_type, T, (int)k, (int)H,
+                                   reinterpret_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "moe_sum launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
 }  // extern "C"

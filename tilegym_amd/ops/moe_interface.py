@@ -1,4 +1,4 @@
-"""MoE entry points with the reference's signatures (src/tilegym/ops/moe_interface.py:14-79)."""
+"""MoE entry points with the reference's signatures (src/tilegym/ops/moe_interface.py:14-370)."""
 
 from __future__ import annotations
 
@@ -41,3 +41,97 @@ def moe_align_block_size(
     """Sort (token, k) slots by expert and pad every expert to a multiple of block_size
     (src/tilegym/ops/moe_interface.py:21-28, src/tilegym/ops/cutile/moe_align_block.py:205-268)."""
     raise NotImplementedError(f"moe_align_block_size is not implemented for this backend: {get_current_backend()}")
+
+
+def fused_experts_impl(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    inplace: bool = False,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+):
+    """The FP8 (use_fp8_w8a8) MoE layer, same signature and chunking as
+    src/tilegym/ops/moe_interface.py:116-322:
+        align -> GEMM1 (gate+up) -> silu(gate) * up -> GEMM2 (down, x routed weight) -> sum over top-k.
+
+    hidden_states (T, H): bf16 / f16 (quantized 1 x 128 on the device here), or e4m3fn together with
+    a1_scale (T, H/128).  w1 (E, 2I, H) and w2 (E, H, I) e4m3fn with w1_scale (E, 2I/128, H/128) and
+    w2_scale (E, H/128, ceil(I/128)).  Returns (T, H) bf16 for bf16 input, else f16.
+
+    Two deliberate differences from the reference's FP8 branch: the activation between the GEMMs is
+    re-quantized 1 x 128 with its own scales (the reference casts it to fp8 under an all-ones a2_scale,
+    moe_interface.py:276-288), and no backend-specific config keys are needed (the reference reads
+    config["BLOCK_SIZE_N"], which only its tilecpp branch defines)."""
+    from .. import _lib, quant
+    from .hip.moe import FP8
+
+    if use_int8_w8a16 or not use_fp8_w8a8:
+        raise NotImplementedError("the hip backend implements the use_fp8_w8a8 MoE path only")
+    assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
+    assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert hidden_states.dtype in [torch.float8_e4m3fn, torch.float32, torch.float16, torch.bfloat16]
+    assert w1.dtype == FP8 and w2.dtype == FP8, "use_fp8_w8a8 needs float8_e4m3fn expert weights"
+    if not hidden_states.is_cuda:
+        raise RuntimeError("the hip backend works on device tensors only")
+    device = hidden_states.device
+    w1, w2, topk_weights, topk_ids = (t if t.is_cuda else t.to(device) for t in (w1, w2, topk_weights, topk_ids))
+    if hidden_states.dtype == FP8:
+        assert a1_scale is not None, "fp8 hidden_states need a1_scale (T, H/128)"
+        if inplace:
+            raise ValueError("inplace needs a 16-bit hidden_states tensor")
+
+    num_tokens, H = hidden_states.shape
+    E, N, _ = w1.shape
+    top_k = topk_ids.shape[1]
+    assert N % 2 == 0 and w2.shape[2] == N // 2 and w2.shape[1] == H
+    out_dtype = torch.bfloat16 if hidden_states.dtype == torch.bfloat16 else torch.float16
+    CHUNK_SIZE = 32768
+    M = min(num_tokens, CHUNK_SIZE)
+    cache1 = torch.empty((M, top_k, N), device=device, dtype=out_dtype)
+    cache3 = torch.empty((M, top_k, H), device=device, dtype=out_dtype)
+    out = hidden_states if inplace else torch.empty((num_tokens, H), device=device, dtype=out_dtype)
+    config = {"BLOCK_SIZE_M": 128}
+
+    for chunk in range((num_tokens // CHUNK_SIZE) + 1):
+        lo, hi = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
+        n = hi - lo
+        if n <= 0:
+            break
+        cur = hidden_states[lo:hi]
+        ids, weights = topk_ids[lo:hi].contiguous(), topk_weights[lo:hi].contiguous()
+        c1, c3 = cache1[:n], cache3[:n]
+        if cur.dtype == FP8:
+            xq, xs = cur, a1_scale[lo:hi]
+        else:
+            xq, xs = quant.act_quant(cur if cur.dtype != torch.float32 else cur.to(out_dtype), 128)
+        sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids, config["BLOCK_SIZE_M"], E)
+        invoke_fused_moe_kernel(xq, w1, c1, xs, w1_scale, weights, ids, sorted_ids, expert_ids, post,
+                                False, top_k, config, compute_type=out_dtype, use_fp8_w8a8=True)
+        q2, s2 = _lib.silu_mul_quant_1x128(c1.view(n * top_k, N))
+        invoke_fused_moe_kernel(q2, w2, c3, s2, w2_scale, weights, ids, sorted_ids, expert_ids, post,
+                                True, 1, config, compute_type=out_dtype, use_fp8_w8a8=True)
+        if top_k == 1:
+            out[lo:hi] = c3[:, 0]
+        else:
+            _lib.moe_sum(c3, out[lo:hi])
+    return out
+
+
+def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk_weights: torch.Tensor,
+              topk_ids: torch.Tensor, **kwargs) -> torch.Tensor:
+    """Unified MoE entry point (src/tilegym/ops/moe_interface.py:325-370).  The reference's form runs the
+    16-bit path; here the expert weights are FP8, so the block scales travel as keyword arguments:
+    ``fused_moe(h, w1, w2, tw, ids, w1_scale=..., w2_scale=..., a1_scale=None)``."""
+    return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, use_fp8_w8a8=True,
+                              w1_scale=kwargs.get("w1_scale"), w2_scale=kwargs.get("w2_scale"),
+                              a1_scale=kwargs.get("a1_scale"))
+
