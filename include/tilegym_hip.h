@@ -140,6 +140,20 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
                         const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream);
 
 /*
+ * A list of independent FP8 GEMMs, C_i <- (sa_i * A_i) @ (sb_i * op(B_i)), i < count, in one launch when
+ * every problem has (N,K) weights (trans_b != 0), K_i % 128 == 0 and 16-byte aligned operands; any other
+ * list is run problem by problem with tg_fp8_gemm's schedules (same results).
+ * Replaces the launch half of tilegym.ops.group_gemm, src/tilegym/ops/cutile/group_gemm.py:170-197.
+ * c, a, b: arrays of `count` descriptor pointers; scale_a, scale_b: NULL, or arrays whose entries are NULL or
+ * one-element f32 tensors.  All c_i share one dtype (bf16 / f16 / f32).  workspace: as for tg_fp8_gemm
+ * (only used on the problem-by-problem route).
+ */
+int32_t tg_fp8_group_gemm(const tg_tensor* const* c, const tg_tensor* const* a, const tg_tensor* const* b,
+                          const tg_tensor* const* scale_a, const tg_tensor* const* scale_b, int32_t count,
+                          int32_t trans_b, const tg_tensor* workspace, const int32_t* cfg, int32_t ncfg,
+                          int32_t device_id, uint64_t hip_stream);
+
+/*
  * moe_align_block_size: group the (token, slot) pairs of a top-k routing by expert and pad every
  * group to a multiple of block_size, in one launch and without host synchronisation.
  * Replaces src/tilegym/ops/cutile/moe_align_block.py:205-268 (four launches) and

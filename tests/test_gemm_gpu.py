@@ -610,6 +610,28 @@ def test_group_gemm_list_form(device):
     assert default[0].dtype == FP8
 
 
+@pytest.mark.parametrize("tile", [None, (64, 128), (128, 128), (256, 256)])
+def test_group_gemm_single_launch(device, tile):
+    """(N,K) weights with K % 128 == 0: the whole list is one launch of the tiled kernel; ragged M and N,
+    an empty problem, more problems than one launch carries (40), per-problem scales."""
+    g = _g(13)
+    shapes = [(64, 128, 256), (130, 72, 128), (8, 264, 512), (0, 128, 128), (300, 520, 384)] + [(17 + i, 136, 128) for i in range(44)]
+    As = [fp8_randn((m, k), g) for m, n, k in shapes]
+    Bs = [fp8_randn((n, k), g, 0.1) for m, n, k in shapes]
+    sa = [0.25 + 0.01 * i for i in range(len(shapes))]
+    sb = [torch.tensor([1.0 + 0.5 * (i % 3)]) for i in range(len(shapes))]
+    kc = None if tile is None else {"BLOCK_M": tile[0], "BLOCK_N": tile[1]}
+    outs = group_gemm([x.to(device) for x in As], [x.to(device) for x in Bs], transpose_b=True, out_dtype=torch.bfloat16,
+                      scales_a=sa, scales_b=[t.to(device) for t in sb], kernel_configs=kc)
+    cfg = used("tiled")
+    if tile is not None:
+        assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == tile
+    for i, (A, B, o) in enumerate(zip(As, Bs, outs)):
+        assert o.shape == (A.shape[0], B.shape[0])
+        if A.shape[0]:
+            check(o, R.ref_gemm_per_tensor(A, B, torch.tensor([sa[i]]), sb[i], trans_b=True), what=f"problem {i}")
+
+
 # ----------------------------------------------------------------------------- BASELINE configs at full size
 def _rows_subset(M, count, seed=0):
     if M <= count:

@@ -108,6 +108,10 @@ def load():
     L.tg_silu_mul_quant_1x128.argtypes = [P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_moe_sum.restype = ctypes.c_int32
     L.tg_moe_sum.argtypes = [P, P, ctypes.c_int32, ctypes.c_uint64]
+    PP = ctypes.POINTER(P)
+    L.tg_fp8_group_gemm.restype = ctypes.c_int32
+    L.tg_fp8_group_gemm.argtypes = [PP, PP, PP, PP, PP, ctypes.c_int32, ctypes.c_int32, P, I32P, ctypes.c_int32,
+                                    ctypes.c_int32, ctypes.c_uint64]
     if L.tg_abi_version() != 1:
         raise RuntimeError(f"libtilegym_hip.so ABI version {L.tg_abi_version()} != 1")
     _lib = L
@@ -298,4 +302,37 @@ def moe_sum(x: torch.Tensor, out: torch.Tensor) -> None:
     L = load()
     rc = L.tg_moe_sum(_ref(make_tensor_desc(out)), _ref(make_tensor_desc(x)), _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_moe_sum")
+
+
+def _desc_array(tensors):
+    """list of tensors (entries may be None) -> (array of descriptor pointers, keep-alive list)."""
+    P = ctypes.POINTER(TgTensor)
+    descs = [make_tensor_desc(t) for t in tensors]
+    arr = (P * len(tensors))(*[ctypes.pointer(d) if d is not None else P() for d in descs])
+    return arr, descs
+
+
+def fp8_group_gemm(cs, As, Bs, scales_a=None, scales_b=None, trans_b=True, kernel_configs=None) -> None:
+    """Lists of problems through tg_fp8_group_gemm (one launch when the list qualifies)."""
+    L = load()
+    n = len(As)
+    cfg, ncfg = make_cfg(kernel_configs)
+    dev = _device_index(As[0])
+    PP = ctypes.POINTER(ctypes.POINTER(TgTensor))
+    c_arr, k1 = _desc_array(cs)
+    a_arr, k2 = _desc_array(As)
+    b_arr, k3 = _desc_array(Bs)
+    sa_arr, k4 = _desc_array(scales_a) if scales_a is not None else (None, None)
+    sb_arr, k5 = _desc_array(scales_b) if scales_b is not None else (None, None)
+    need = 0
+    if not trans_b:
+        for a, b in zip(As, Bs):
+            need = max(need, workspace_bytes(a.shape[0], b.shape[1], a.shape[1], False, cfg, ncfg))
+    ws = workspace_for(As[0].device, need) if need else None
+    rc = L.tg_fp8_group_gemm(ctypes.cast(c_arr, PP), ctypes.cast(a_arr, PP), ctypes.cast(b_arr, PP),
+                             ctypes.cast(sa_arr, PP) if sa_arr is not None else None,
+                             ctypes.cast(sb_arr, PP) if sb_arr is not None else None,
+                             n, 1 if trans_b else 0, _ref(make_tensor_desc(ws)), cfg, ncfg, dev, _stream_handle(As[0]))
+    del k1, k2, k3, k4, k5
+    check_rc(rc, "tg_fp8_group_gemm")
 

@@ -210,8 +210,10 @@ __device__ __forceinline__ void pipeline_hint_scaled() {
     __builtin_amdgcn_sched_group_barrier(TG_SGB_VALU, 4 * TM, 0);
 }
 
+// Body of the tiled kernel for workgroup `bid` of problem `p` (the kernels below only differ in
+// how a workgroup finds its problem).
 template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>
-__global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_gemm_tile_kernel(const GemmParams p) {
+__device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const int bid) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body is device-only assembly; the host pass only needs the stub
     constexpr int NT = 64 * WGM * WGN;
     constexpr int NW = WGM * WGN;
@@ -258,7 +260,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     int post_pad = 0;
     if constexpr (GROUP == GROUP_DENSE) {
         const int tiles_m = (p.M + BM - 1) / BM;
-        const int pid = xcd_remap(blockIdx.x, tiles_m * tiles_n);
+        const int pid = xcd_remap(bid, tiles_m * tiles_n);
         constexpr int GM = 8;
         const int width = GM * tiles_n;
         const int group = pid / width, first_m = group * GM;
@@ -270,8 +272,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     } else if constexpr (GROUP == GROUP_RAGGED) {
         const int total_mt = ragged_count_tiles(p.m_indptr, p.E, BM, lane);
         const int nblk = total_mt * tiles_n;
-        if ((int)blockIdx.x >= nblk) return;
-        const int pid = xcd_remap(blockIdx.x, nblk);
+        if (bid >= nblk) return;
+        const int pid = xcd_remap(bid, nblk);
         tile_m = pid / tiles_n;
         tile_n = pid % tiles_n;
         int e, t_in_e;
@@ -289,8 +291,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
         post_pad = min(p.num_post_pad[0], p.em_capacity);
         const int total_mt = (post_pad + BM - 1) / BM;
         const int nblk = total_mt * tiles_n;
-        if ((int)blockIdx.x >= nblk) return;
-        const int pid = xcd_remap(blockIdx.x, nblk);
+        if (bid >= nblk) return;
+        const int pid = xcd_remap(bid, nblk);
         tile_m = pid / tiles_n;
         tile_n = pid % tiles_n;
         m0 = tile_m * BM;  // position in the sorted slot sequence
@@ -562,6 +564,43 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     }
 
 #endif
+}
+
+template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>
+__global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_gemm_tile_kernel(const GemmParams p) {
+    fp8_gemm_tile_body<BM, BN, WGM, WGN, BLOCKSCALE, GROUP, SPLIT>(p, (int)blockIdx.x);
+}
+
+// A list of independent per-tensor-scaled GEMMs in one launch (tilegym.ops.group_gemm,
+// src/tilegym/ops/cutile/group_gemm.py:170-197).  The problems travel in the kernel arguments;
+// a workgroup finds the problem that owns its tile with a scan over the tile prefix and then runs
+// the dense body on it.
+template <int BM, int BN, int WGM, int WGN>
+__global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_gemm_tile_list_kernel(const GemmList gl) {
+    const int bid = (int)blockIdx.x;
+    int i = 0, start = 0;
+    while (i + 1 < gl.count && bid >= gl.prob[i].tile_end) {
+        start = gl.prob[i].tile_end;
+        ++i;
+    }
+    GemmParams p{};
+    p.A = gl.prob[i].A; p.B = gl.prob[i].B; p.C = gl.prob[i].C;
+    p.As = gl.prob[i].As; p.Bs = gl.prob[i].Bs;
+    p.M = gl.prob[i].M; p.N = gl.prob[i].N; p.K = gl.prob[i].K;
+    p.kblocks = p.K / kKBlock; p.nblocks = (p.N + 127) / 128;
+    p.alpha = gl.alpha; p.beta = 0.f;
+    p.out_type = gl.out_type;
+    p.vec_store = gl.prob[i].vec_store;
+    p.split_k = 1; p.ksteps_per_split = p.kblocks;
+    p.E = 1; p.top_k = 1;
+    fp8_gemm_tile_body<BM, BN, WGM, WGN, false, GROUP_DENSE, false>(p, bid - start);
+}
+
+template <int BM, int BN, int WGM, int WGN>
+inline hipError_t launch_tile_list(const GemmList& gl, int grid_x, hipStream_t stream) {
+    auto kern = fp8_gemm_tile_list_kernel<BM, BN, WGM, WGN>;
+    hipLaunchKernelGGL(kern, dim3(grid_x, 1, 1), dim3(64 * WGM * WGN, 1, 1), 0, stream, gl);
+    return hipGetLastError();
 }
 
 template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>

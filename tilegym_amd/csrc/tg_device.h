@@ -45,6 +45,26 @@ struct GemmParams {
     int top_k, num_valid, block_m, em_capacity;
 };
 
+// A list of independent per-tensor-scaled NT GEMMs handed to one launch in the kernel arguments.
+constexpr int kListMax = 40;
+struct ListProblem {
+    const uint8_t* A;
+    const uint8_t* B;
+    void* C;
+    const float* As;
+    const float* Bs;
+    int M, N, K;
+    int tile_end;   // exclusive prefix of BM x BN tiles over the list
+    int vec_store;
+    int pad;
+};
+struct GemmList {
+    int count, out_type;
+    float alpha;
+    int pad;
+    ListProblem prob[kListMax];
+};
+
 // One 16x16x128 e4m3 x e4m3 MFMA with fp32 accumulation.  `w` supplies the 16 rows of the
 // result (lane l: row l%16, K bytes of K-group l/16), `x` supplies the 16 columns; lane l
 // receives column l%16, rows 4*(l/16)..+3.  With both scale operands zero the compiler

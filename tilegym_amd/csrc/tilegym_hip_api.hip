@@ -735,4 +735,85 @@ int32_t tg_moe_sum(const tg_tensor* out, const tg_tensor* x, int32_t device_id, 
     return TG_OK;
 }
 
+int32_t tg_fp8_group_gemm(const tg_tensor* const* c, const tg_tensor* const* a, const tg_tensor* const* b,
+                          const tg_tensor* const* scale_a, const tg_tensor* const* scale_b, int32_t count,
+                          int32_t trans_b, const tg_tensor* workspace, const int32_t* cfg, int32_t ncfg,
+                          int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    if (count < 0) return fail(TG_ERR_INVALID, "negative count");
+    if (count == 0) return TG_OK;
+    if (!c || !a || !b) return fail(TG_ERR_NULL, "null descriptor array");
+    // ---- can the whole list go out as one launch?
+    bool one_launch = trans_b != 0 && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0 && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1;
+    int32_t rc;
+    int32_t out_dtype = -1;
+    int64_t max_m = 0;
+    for (int i = 0; i < count; ++i) {
+        if ((rc = check_tensor(a[i], "a[i]", 2)) || (rc = check_tensor(b[i], "b[i]", 2)) || (rc = check_tensor(c[i], "c[i]", 2))) return rc;
+        if (a[i]->dtype != TG_F8E4M3FN || b[i]->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7)");
+        if (out_type_of(c[i]->dtype) < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16 or f32");
+        if (out_dtype < 0) out_dtype = c[i]->dtype;
+        if (c[i]->dtype != out_dtype) one_launch = false;
+        const int64_t M = a[i]->shape[0], K = a[i]->shape[1];
+        const int64_t N = trans_b ? b[i]->shape[0] : b[i]->shape[1], Kb = trans_b ? b[i]->shape[1] : b[i]->shape[0];
+        if (K != Kb) return fail(TG_ERR_INVALID, "problem %d: K dimensions must match: %lld != %lld", i, (long long)K, (long long)Kb);
+        if (c[i]->shape[0] != M || c[i]->shape[1] != N) return fail(TG_ERR_INVALID, "problem %d: c must be (%lld, %lld)", i, (long long)M, (long long)N);
+        for (const tg_tensor* const* sc : {scale_a, scale_b}) {
+            if (sc && sc[i]) {
+                if ((rc = check_tensor(sc[i], "scale", -1))) return rc;
+                if (sc[i]->dtype != TG_F32 || numel(sc[i]) != 1) return fail(TG_ERR_INVALID, "problem %d: scales must be one-element f32 tensors", i);
+            }
+        }
+        if (K <= 0 || K % 128 != 0 || K > 65536 || !aligned16(a[i]->ptr) || !aligned16(b[i]->ptr) || M * K >= kOffsetLimit ||
+            N * K >= kOffsetLimit || M > INT32_MAX || N > INT32_MAX)
+            one_launch = false;
+        if (M > max_m) max_m = M;
+    }
+    if (!one_launch) {
+        for (int i = 0; i < count; ++i) {
+            rc = tg_fp8_gemm(c[i], a[i], b[i], scale_a ? scale_a[i] : nullptr, scale_b ? scale_b[i] : nullptr, 0, trans_b, 1.0f, 0.0f,
+                             workspace, cfg, ncfg, device_id, hip_stream);
+            if (rc) return rc;
+        }
+        return TG_OK;
+    }
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
+    if (!((bm == 256 && bn == 256) || (bm == 128 && bn == 128) || (bm == 64 && bn == 128))) {
+        int64_t big = 0;
+        for (int i = 0; i < count; ++i) big += cdiv(a[i]->shape[0], 256) * cdiv(b[i]->shape[0], 256);
+        if (max_m <= 64) { bm = 64; bn = 128; }
+        else if (big >= 200) { bm = 256; bn = 256; }
+        else { bm = 128; bn = 128; }
+    }
+    Schedule s{1, bm, bn, 1, -1, -1, -1};
+    remember(s);
+    for (int first = 0; first < count; first += tg::kListMax) {
+        tg::GemmList gl{};
+        gl.out_type = out_type_of(out_dtype);
+        gl.alpha = 1.0f;
+        int tiles = 0;
+        for (int i = first; i < count && i < first + tg::kListMax; ++i) {
+            const int64_t M = a[i]->shape[0], N = b[i]->shape[0], K = a[i]->shape[1];
+            if (M == 0 || N == 0) continue;
+            tg::ListProblem& q = gl.prob[gl.count++];
+            q.A = reinterpret_cast<const uint8_t*>(a[i]->ptr);
+            q.B = reinterpret_cast<const uint8_t*>(b[i]->ptr);
+            q.C = reinterpret_cast<void*>(c[i]->ptr);
+            q.As = (scale_a && scale_a[i]) ? reinterpret_cast<const float*>(scale_a[i]->ptr) : nullptr;
+            q.Bs = (scale_b && scale_b[i]) ? reinterpret_cast<const float*>(scale_b[i]->ptr) : nullptr;
+            q.M = (int)M; q.N = (int)N; q.K = (int)K;
+            tiles += (int)(cdiv(M, bm) * cdiv(N, bn));
+            q.tile_end = tiles;
+            q.vec_store = ((N % 4) == 0 && aligned16(c[i]->ptr)) ? 1 : 0;
+        }
+        if (gl.count == 0 || tiles == 0) continue;
+        hipError_t e = tg::run_tile_list(bm, bn, gl, tiles, stream);
+        if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "list kernel launch failed: %s", hipGetErrorString(e));
+    }
+    return TG_OK;
+}
+
 }  // extern "C"

@@ -167,19 +167,48 @@ def ragged_block_scaled_bmm(a, b, a_scale, b_scale, m_indptr, max_m, max_m_devic
 
 @register_impl("group_gemm", backend="hip")
 def group_gemm(group_A, group_B, static_persistent=True, use_tma=True, transpose_b=False, **kwargs):
-    """List of GEMMs (src/tilegym/ops/cutile/group_gemm.py:170-197): one launch per group, all
-    on the current stream; outputs in ``A.dtype`` unless ``out_dtype`` is given."""
+    """List of GEMMs (src/tilegym/ops/cutile/group_gemm.py:170-197) through tg_fp8_group_gemm: one
+    launch for (N,K) weights with K % 128 == 0, otherwise problem by problem; all on the current
+    stream; outputs in ``A.dtype`` unless ``out_dtype`` is given.  ``scales_a`` / ``scales_b``:
+    optional lists of per-tensor scales (one-element tensors, floats or None)."""
     if not group_A or not group_B:
         raise ValueError("group_A and group_B must not be empty")
     if len(group_A) != len(group_B):
         raise ValueError(f"group_A and group_B must have same length, got {len(group_A)} and {len(group_B)}")
-    scales_a: Optional[List] = kwargs.get("scales_a")
-    scales_b: Optional[List] = kwargs.get("scales_b")
+    transpose_b = bool(transpose_b)
+    out_dtype = kwargs.get("out_dtype")
+    cast_back = None
+    if out_dtype is None:
+        cast_back = group_A[0].dtype
+        out_dtype = torch.float32
+    if out_dtype not in _OUT_DTYPES:
+        raise NotImplementedError(f"out_dtype {out_dtype} not supported")
+    dev = group_A[0].device
+    if not group_A[0].is_cuda:
+        raise RuntimeError("the hip backend works on device tensors only")
     outs = []
-    for i, (A, B) in enumerate(zip(group_A, group_B)):
-        outs.append(matmul(A, B, False, bool(transpose_b),
-                           scale_a=None if scales_a is None else scales_a[i],
-                           scale_b=None if scales_b is None else scales_b[i],
-                           out_dtype=kwargs.get("out_dtype"),
-                           kernel_configs=kwargs.get("kernel_configs")))
-    return outs
+    for A, B in zip(group_A, group_B):
+        _require_fp8(A, B)
+        if A.dim() != 2 or B.dim() != 2:
+            raise ValueError("group_gemm expects 2-D operands")
+        N, KB = (B.shape if transpose_b else (B.shape[1], B.shape[0]))
+        assert A.shape[1] == KB, f"Incompatible matrices: K dimension of A is {A.shape[1]}, K dimension of B is {KB}"
+        assert A.is_contiguous() and B.is_contiguous(), "operands must be contiguous"
+        outs.append(torch.empty((A.shape[0], N), device=dev, dtype=out_dtype))
+
+    def as_tensors(scales):
+        if scales is None:
+            return None
+        res = []
+        for sc in scales:
+            if sc is None:
+                res.append(None)
+            elif isinstance(sc, torch.Tensor):
+                res.append(sc.reshape(-1)[:1].float().contiguous())
+            else:
+                res.append(torch.full((1,), float(sc), dtype=torch.float32, device=dev))
+        return res
+
+    _lib.fp8_group_gemm(outs, list(group_A), list(group_B), as_tensors(kwargs.get("scales_a")),
+                        as_tensors(kwargs.get("scales_b")), transpose_b, kwargs.get("kernel_configs"))
+    return [o.to(cast_back) for o in outs] if cast_back is not None else outs
