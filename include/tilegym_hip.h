@@ -63,7 +63,7 @@ enum {
     TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (64/128/256)            */
     TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (128/256)               */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
-    TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4)         */
+    TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4); stream kernel: LDS buffers per wave (1/2) */
     TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); pipe kernel: loader waves (4/8) */
     TG_CFG_COUNT = 8
 };

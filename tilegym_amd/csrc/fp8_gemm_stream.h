@@ -97,15 +97,28 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p
     // next piece's direct loads would have to wait for them).  Larger M: one K step ahead.
     constexpr bool PRELOAD = MT == 1;
     v4i pa_lo[PRELOAD ? SPC : 1], pa_hi[PRELOAD ? SPC : 1];
+    // block scales of a whole piece travel with the preloaded activations: fetched before the wait
+    // for the weights, not between the MFMAs
+    float psc[(PRELOAD && BLOCKSCALE) ? SPC : 1];
     auto preload_act = [&](int c) {
         if constexpr (PRELOAD) {
 #pragma unroll
             for (int s = 0; s < SPC; ++s) load_act(c * SPC + s, &pa_lo[s], &pa_hi[s]);
+            if constexpr (BLOCKSCALE) {
+#pragma unroll
+                for (int s = 0; s < SPC; ++s) {
+                    const int ks = min(c * SPC + s, p.kblocks - 1);
+                    const float sb = bs_ptr ? bs_ptr[ks] : 1.0f;
+                    psc[s] = (p.As ? p.As[(int64_t)arow[0] * p.kblocks + ks] : 1.0f) * sb;
+                }
+            }
         }
     };
-    auto mma_step = [&](int ks, v8i wf, const v8i* af) {
+    auto mma_step = [&](int ks, v8i wf, const v8i* af, int s_in_piece) {
         float sc[MT];
-        if constexpr (BLOCKSCALE) {
+        if constexpr (BLOCKSCALE && PRELOAD) {
+            sc[0] = psc[s_in_piece];
+        } else if constexpr (BLOCKSCALE) {
             const float sb = bs_ptr ? bs_ptr[ks] : 1.0f;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
@@ -133,7 +146,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p
                     const v8i wf = join(*reinterpret_cast<const v4i*>(base + ((j0 ^ li) << 4)),
                                         *reinterpret_cast<const v4i*>(base + ((j1 ^ li) << 4)));
                     const v8i af = join(pa_lo[s], pa_hi[s]);
-                    mma_step(ks0 + s, wf, &af);
+                    mma_step(ks0 + s, wf, &af, s);
                 }
             }
         } else {
@@ -147,7 +160,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p
                 const int j0 = s * 8 + lg, j1 = j0 + 4;
                 const v8i wf = join(*reinterpret_cast<const v4i*>(base + ((j0 ^ li) << 4)),
                                     *reinterpret_cast<const v4i*>(base + ((j1 ^ li) << 4)));
-                mma_step(ks0 + s, wf, af);
+                mma_step(ks0 + s, wf, af, 0);
             }
         }
     };

@@ -404,7 +404,11 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
         const int64_t pieces = cdiv(K, 1024);
         if (s.split_k > 1) p.ksteps_per_split = (int)cdiv(pieces, s.split_k);
         const int64_t per_wave = cdiv(s.split_k > 1 ? p.ksteps_per_split : pieces, 4);
-        const int nbuf = (per_wave >= 2 && s.mt == 1) ? 2 : 1;
+        int nbuf = cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS);  // stream kernel: LDS buffers per wave
+        // measured: one 16 KiB buffer per wave and two workgroups per compute unit beat two buffers and
+        // one workgroup, except for long K where they tie
+        if (nbuf != 1 && nbuf != 2) nbuf = (per_wave >= 3 && s.mt == 1 && !block_scaled) ? 2 : 1;
+        if (s.mt != 1) nbuf = 1;
         hipError_t e = tg::run_stream(s.mt, nbuf, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "stream kernel launch failed: %s", hipGetErrorString(e));
         if (s.split_k > 1 && tg::run_splitk_reduce(p, block_scaled, stream) != hipSuccess)
