@@ -141,6 +141,22 @@ def test_per_tensor_stream(device, M, N, K, split):
     check(out, ref, what=f"stream M={M} N={N} K={K} split={split}")
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 1), (264, 2064, 1), (128, 16384, 4), (72, 512, 1), (4096, 3072, 2)])
+def test_per_tensor_stream_wide(device, M, N, K, split):
+    """64 weight rows per workgroup with the activation piece shared through LDS: ragged N (also inside a
+    workgroup's 64 rows), K tails inside a 1 KiB piece, split-K, every M up to 16."""
+    g = _g(M * 13 + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
+    ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split})
+    cfg = used("stream")
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split
+    check(out, ref, what=f"stream wide M={M} N={N} K={K} split={split}")
+
+
 def test_decode_auto_schedule_and_determinism(device):
     case = W.llama_decode_case(16, "o")
     ref = R.ref_gemm_per_tensor(case.a, case.b, case.scale_a, case.scale_b, trans_b=True)

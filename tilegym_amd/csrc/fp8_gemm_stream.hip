@@ -13,4 +13,6 @@ hipError_t run_stream(int mt, int nbuf, bool bs, const GemmParams& p, int gx, in
     return hipErrorInvalidConfiguration;
 }
 
+hipError_t run_stream_wide(const GemmParams& p, int gx, int gy, hipStream_t s) { return launch_stream_wide(p, gx, gy, s); }
+
 }  // namespace tg
