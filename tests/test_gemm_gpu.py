@@ -157,6 +157,19 @@ def test_per_tensor_stream_wide(device, M, N, K, split):
     check(out, ref, what=f"stream wide M={M} N={N} K={K} split={split}")
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("N,K,split", [(640, 1024, 1), (264, 2304, 1), (1152, 5120, 2), (128, 12288, 6)])
+def test_block_scaled_stream_wide(device, M, N, K, split):
+    case = W.block_scaled_case(M, N, K, seed=M + N)
+    ref = R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16)
+    d = case.to(device)
+    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16,
+                                kernel_configs={"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split})
+    cfg = used("stream")
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split
+    check(out, ref, what=f"block-scaled stream wide M={M} N={N} K={K} split={split}")
+
+
 def test_decode_auto_schedule_and_determinism(device):
     case = W.llama_decode_case(16, "o")
     ref = R.ref_gemm_per_tensor(case.a, case.b, case.scale_a, case.scale_b, trans_b=True)

@@ -235,7 +235,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p
 #endif
 }
 
-// Wide variant for M <= 16 and many weight rows (per-tensor scales): a workgroup owns 64 weight
+// Wide variant for M <= 16 and many weight rows: a workgroup owns 64 weight
 // rows, wave w the rows 16w .. 16w+15 over the workgroup's whole K range, so no cross-wave
 // reduction is needed -- and all four waves multiply the SAME activation piece, which is fetched
 // once per workgroup into a shared 16 KiB LDS buffer with the same row-wise direct loads as the
@@ -245,6 +245,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p
 // Here the activations cost a quarter of the weights' load instructions, each over full lines.
 // Only rows < M of the activation buffer are filled; the other columns of the MFMA result are
 // never stored.
+template <bool BLOCKSCALE>
 __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int NW = 4;
@@ -289,11 +290,28 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmPar
         }
     };
 
+    // block scales: the wave's 16 weight rows lie in one 128-row block (one scalar per K step), the
+    // activation scale belongs to the lane's column (row li of A); both are fetched per piece
+    // before the wait for the weights
+    const float* bs_ptr = nullptr;
+    const float* as_ptr = nullptr;
+    if constexpr (BLOCKSCALE) {
+        bs_ptr = p.Bs ? p.Bs + (int64_t)min(n_base / 128, p.nblocks - 1) * p.kblocks : nullptr;
+        as_ptr = p.As ? p.As + (int64_t)min(li, M - 1) * p.kblocks : nullptr;
+    }
     v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
     constexpr int kWaitMine = 0x0070;  // vmcnt(0) lgkmcnt(0)
     constexpr int kWaitLds = 0xC07F;   // lgkmcnt(0)
     for (int c = c_begin; c < c_end; ++c) {
         issue(c);
+        float psc[BLOCKSCALE ? SPC : 1];
+        if constexpr (BLOCKSCALE) {
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) {
+                const int ks = min(c * SPC + s, p.kblocks - 1);
+                psc[s] = (as_ptr ? as_ptr[ks] : 1.0f) * (bs_ptr ? bs_ptr[ks] : 1.0f);
+            }
+        }
         __builtin_amdgcn_s_waitcnt(kWaitMine);
         __builtin_amdgcn_s_barrier();  // every wave's share of the activation piece has landed
         const uint8_t* wb = my_buf + li * kStreamChunk;
@@ -305,7 +323,8 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmPar
                 const int j0 = ((s * 8 + lg) ^ li) << 4, j1 = ((s * 8 + 4 + lg) ^ li) << 4;
                 const v8i wf = join(*reinterpret_cast<const v4i*>(wb + j0), *reinterpret_cast<const v4i*>(wb + j1));
                 const v8i af = join(*reinterpret_cast<const v4i*>(ab + j0), *reinterpret_cast<const v4i*>(ab + j1));
-                acc = mfma_e4m3(wf, af, acc);
+                if constexpr (BLOCKSCALE) acc += mfma_e4m3(wf, af, v4f{0.f, 0.f, 0.f, 0.f}) * psc[s];
+                else acc = mfma_e4m3(wf, af, acc);
             }
         }
         __builtin_amdgcn_s_waitcnt(kWaitLds);
@@ -320,14 +339,17 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmPar
         return;
     }
     float scale = p.alpha;
-    if (p.As) scale *= p.As[0];
-    if (p.Bs) scale *= p.Bs[0];
+    if constexpr (!BLOCKSCALE) {
+        if (p.As) scale *= p.As[0];
+        if (p.Bs) scale *= p.Bs[0];
+    }
     store4(p.C, p.out_type, m, col, N, acc * scale, p.beta, vec_ok);
 #endif
 }
 
+template <bool BLOCKSCALE>
 inline hipError_t launch_stream_wide(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
-    hipLaunchKernelGGL(fp8_gemm_stream_wide_kernel, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
+    hipLaunchKernelGGL(fp8_gemm_stream_wide_kernel<BLOCKSCALE>, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -13,6 +13,8 @@ hipError_t run_stream(int mt, int nbuf, bool bs, const GemmParams& p, int gx, in
     return hipErrorInvalidConfiguration;
 }
 
-hipError_t run_stream_wide(const GemmParams& p, int gx, int gy, hipStream_t s) { return launch_stream_wide(p, gx, gy, s); }
+hipError_t run_stream_wide(bool bs, const GemmParams& p, int gx, int gy, hipStream_t s) {
+    return bs ? launch_stream_wide<true>(p, gx, gy, s) : launch_stream_wide<false>(p, gx, gy, s);
+}
 
 }  // namespace tg

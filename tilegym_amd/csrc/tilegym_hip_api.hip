@@ -175,18 +175,17 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // blocks to fill the chip without a second pass; ROW_GROUPS = 4 asks for it explicitly
         const int want_rg = cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS);
         const int64_t wide_wgs = cdiv(N, 64);
-        // without a second pass when the row blocks alone fill the chip; for long K (>= 8 pieces) also
-        // with K split over ~448 workgroups of >= 2 pieces each (measured: wins on 4096 x 14336, loses
-        // on 4096 x 4096 and 6144 x 4096 where the reduction pass costs more than it saves)
-        const bool wide_auto = N >= 16384 || (pieces >= 8 && wide_wgs * (pieces / 2) >= 320);
-        if (!block_scaled && M <= 16 && (want_rg == 4 || (want_rg < 0 && wide_auto))) {
+        // without a second pass when the row blocks alone fill the chip; otherwise K is split over ~448
+        // workgroups, which pays a reduction pass (~3 us): measured to win from ~50 MB of weights on
+        // (4096 x 14336, 12288 x 5120, 5120 x 12288) and to lose on 4096 x 4096 and 6144 x 4096
+        int64_t wide_split = cdiv(448, wide_wgs);
+        if (wide_split > pieces) wide_split = pieces;
+        const bool wide_auto = N >= 16384 || (N * K >= ((int64_t)48 << 20) && wide_wgs * wide_split >= 320);
+        if (M <= 16 && (want_rg == 4 || (want_rg < 0 && wide_auto))) {
             s.row_groups = 4;
             if (want_split > 1) s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, want_split);
-            else if (want_split < 0 && wide_wgs < 384 && pieces >= 4) {
-                int64_t want = cdiv(448, wide_wgs);
-                if (want > pieces / 2) want = pieces / 2;
-                if (want > 1) s.split_k = pick_split(wide_wgs, 512, pieces, 2, M, N, partial_bytes_avail, (int)want);
-            }
+            else if (want_split < 0 && wide_wgs < 384 && wide_split > 1)
+                s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, (int)wide_split);
             return s;
         }
         if (want_split > 1 || (want_split < 0 && wgs * 4 * 4 <= kTargetWaves && pieces >= 16))
@@ -427,7 +426,7 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
         // one workgroup, except for long K where they tie
         if (nbuf != 1 && nbuf != 2) nbuf = (per_wave >= 3 && s.mt == 1 && !block_scaled) ? 2 : 1;
         if (s.mt != 1) nbuf = 1;
-        hipError_t e = s.row_groups == 4 ? tg::run_stream_wide(p, (int)cdiv(N, 64), s.split_k, stream)
+        hipError_t e = s.row_groups == 4 ? tg::run_stream_wide(block_scaled, p, (int)cdiv(N, 64), s.split_k, stream)
                                          : tg::run_stream(s.mt, nbuf, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "stream kernel launch failed: %s", hipGetErrorString(e));
         if (s.split_k > 1 && tg::run_splitk_reduce(p, block_scaled, stream) != hipSuccess)
