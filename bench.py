@@ -39,7 +39,7 @@ ROTATE_BYTES = 640 << 20
 # HBM bytes per launch (reads + writes) from the hardware counters FETCH_SIZE and WRITE_SIZE, collected in
 # two profiler passes of this program and scaled by what the same counters read for --calibrate-copy's
 # elementwise add of known size (reads x2.000, writes x1.000); figures and commands are in
-# profiles/fp8_gemm_tile_kernel_prefill_pmc.txt and profiles/fp8_gemm_stream_kernel_decode_pmc.txt.
+# profiles/fp8_gemm_tile_kernel_prefill_pmc.txt and profiles/fp8_gemm_stream_wide_kernel_decode_pmc.txt.
 # Decode entries are the average over M = 1, 8, 16 of one projection (same grid).
 KIB = 1024
 MEASURED_TRAFFIC = {
@@ -47,9 +47,16 @@ MEASURED_TRAFFIC = {
     "c3_prefill_gate_up_M8192": (688551.8 * 2 + 458752.0) * KIB,
     "c2_decode_qkv": (12497.2 * 2 + 100.0) * KIB,
     "c2_decode_o": (8370.3 * 2 + 66.7) * KIB,
-    "c2_decode_gate_up": (57712.5 * 2 + 466.7) * KIB,
-    "c2_decode_down": (29204.2 * 2 + 66.7) * KIB,
+    "c2_decode_gate_up": (57522.9 * 2 + 467.1) * KIB,
+    "c2_decode_down": (29179.7 * 2 + 933.6) * KIB,
 }
+
+
+def kernel_symbol(shape):
+    """Device function a measured shape ran (the stream kernel's 64-row form is a kernel of its own)."""
+    if shape["kernel"] == "stream" and shape["row_groups"] == 4:
+        return "fp8_gemm_stream_wide_kernel"
+    return KERNEL_SYMBOLS[shape["kernel"]]
 
 
 def measured_traffic(shape_name):
@@ -153,7 +160,9 @@ def measure_shape(runner, steps, warmup, stream, use_graph):
     ms = None
     launches = steps
     if use_graph:
-        per_graph = max(runner.copies, 8)
+        # a whole number of passes over the operand copies: a graph that stopped part-way through the
+        # rotation would start its next replay on copies the previous one had just read
+        per_graph = runner.copies * max(1, -(-8 // runner.copies))
         replays = max(1, steps // per_graph)
         ms = _graph_ms(runner, per_graph, replays, stream)
         launches = per_graph * replays
@@ -291,7 +300,7 @@ def main():
             "us_per_step": round(tot_us, 2),
             "frac_hbm_M_le_16": round(sum(s["bytes"] for s in small) / sum(s["us"] for s in small) * 1e-3 / PEAK_HBM_GBS, 4),
             "roofline": {"bound": "hbm", "achieved": dom["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
-                         "traffic": measured_traffic(dom["name"]), "kernel": KERNEL_SYMBOLS[dom["kernel"]] + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
+                         "traffic": measured_traffic(dom["name"]), "kernel": kernel_symbol(dom) + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
         }
         detail["decode"] = shapes
         if "value" in out:

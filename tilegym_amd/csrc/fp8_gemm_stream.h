@@ -53,7 +53,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p
             const uint32_t voff = (uint32_t)n * (uint32_t)K + j * 16;
             const uint32_t dst = my_lds + buf * BUF + r * kStreamChunk;
             if (k0 + j * 16 < K) {
-                direct_load_b128(rsrc_b, dst, voff, k0);
+                direct_load_b128_nt(rsrc_b, dst, voff, k0);
             } else {  // past the end of K: zeros
                 *reinterpret_cast<v4i*>(my_buf + buf * BUF + r * kStreamChunk + lane * 16) = v4i{0, 0, 0, 0};
             }
@@ -276,7 +276,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmPar
         for (int r = 0; r < 16; ++r) {
             const int n = min(n_base + r, N - 1);
             const int j = lane ^ r;
-            if (k0 + j * 16 < K) direct_load_b128(rsrc_b, my_lds + r * kStreamChunk, (uint32_t)n * (uint32_t)K + j * 16, k0);
+            if (k0 + j * 16 < K) direct_load_b128_nt(rsrc_b, my_lds + r * kStreamChunk, (uint32_t)n * (uint32_t)K + j * 16, k0);
             else *reinterpret_cast<v4i*>(my_buf + r * kStreamChunk + lane * 16) = v4i{0, 0, 0, 0};
         }
 #pragma unroll
