@@ -293,7 +293,7 @@ def test_block_scaled_reference_test_shapes(device, M, N, K):
     check(out, ref, tight=1e-4, what="block-scaled f32")
 
 
-@pytest.mark.parametrize("bm,bn", [(128, 128), (128, 256), (64, 128)])
+@pytest.mark.parametrize("bm,bn", [(256, 256), (128, 128), (128, 256), (64, 128)])
 @pytest.mark.parametrize("M,N,K", [(300, 640, 384), (129, 136, 256)])
 def test_block_scaled_tiled_configs_and_edges(device, bm, bn, M, N, K):
     case = W.block_scaled_case(M, N, K, seed=M)
@@ -370,7 +370,7 @@ def test_ragged_reference_test_shapes(device, groups, m, n, k):
     check(out, ref, what="ragged aligned")
 
 
-@pytest.mark.parametrize("bm,bn", [(128, 128), (128, 256), (64, 128)])
+@pytest.mark.parametrize("bm,bn", [(256, 256), (128, 128), (128, 256), (64, 128)])
 def test_ragged_unaligned_empty_and_single_experts(device, bm, bn):
     sizes = [5, 0, 131, 64, 0, 0, 257, 1, 77]
     a, b, a_s, b_s, ptr = _ragged_inputs(sizes, 392, 256, 17, total_extra=6)
@@ -420,7 +420,7 @@ def test_ragged_fallback_for_odd_k(device):
 
 
 # ----------------------------------------------------------------------------- MoE token gather
-@pytest.mark.parametrize("block_m", [64, 128, 16])
+@pytest.mark.parametrize("block_m", [64, 128, 16, 256])
 @pytest.mark.parametrize("mul_w", [False, True])
 def test_moe_gather_gemm(device, block_m, mul_w):
     g = _g(block_m)

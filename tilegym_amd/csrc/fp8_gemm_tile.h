@@ -343,7 +343,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // logical chunk (l%8) ^ swz16(row) = (l%8) ^ (l/8).
     const int lrow = lane >> 3;
     const int lj = (lane & 7) ^ swz16(lrow);
-    const bool loader = wave < NL;
+    // (with NL == NW every wave loads: no test, and so no branch inside the K loop)
+    const bool loader = NL == NW || wave < NL;
     uint32_t a_off[A_IT], b_off[B_IT];
 #pragma unroll
     for (int i = 0; i < A_IT; ++i) {
@@ -444,24 +445,38 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     };
     auto mma = [&](const uint8_t* cB) {
         if constexpr (BLOCKSCALE) {
-            // The 16x16 products of column tile tn are scaled and added while the MFMAs of
-            // column tile tn+1 run: MFMA and VALU work overlap instead of alternating.
-            v4f part[2][TM];
-#pragma unroll
-            for (int tn = 0; tn < TN; ++tn) {
+            // One MFMA (into a zeroed 16x16 product), then the four scale-and-add operations of the
+            // product issued two MFMAs earlier: the matrix pipe works on the MFMA for 32 clocks while
+            // the wave issues 16 clocks of VALU work behind it, and a product is complete (two MFMA
+            // slots old) when it is read.  Three product registers rotate.  The scheduling fence after
+            // every such pair keeps the compiler from collecting the VALU work behind the last MFMA
+            // (where the matrix pipe would idle); the weight fragment of column tile tn+1 is fetched
+            // during column tile tn.
+            constexpr int NJ = TN * TM;
+            v4f part[3];
+            v8i wf[2];
+            auto read_w = [&](int tn) {
                 const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
-                const v8i wf = join(*reinterpret_cast<const v4i*>(base + frag0),
-                                    *reinterpret_cast<const v4i*>(base + frag1));
+                wf[tn & 1] = join(*reinterpret_cast<const v4i*>(base + frag0), *reinterpret_cast<const v4i*>(base + frag1));
+            };
+            read_w(0);
 #pragma unroll
-                for (int tm = 0; tm < TM; ++tm)
-                    part[tn & 1][tm] = mfma_e4m3(wf, af[tm], v4f{0.f, 0.f, 0.f, 0.f});
-                if (tn > 0) {
-#pragma unroll
-                    for (int tm = 0; tm < TM; ++tm) acc[tn - 1][tm] += part[(tn - 1) & 1][tm] * sc[tm];
-                }
+            for (int j = 0; j < NJ; ++j) {
+                const int tn = j / TM, tm = j % TM;
+                part[j % 3] = mfma_e4m3(wf[tn & 1], af[tm], v4f{0.f, 0.f, 0.f, 0.f});
+                if (tm == 0 && tn + 1 < TN) read_w(tn + 1);
+                if (j >= 2) acc[(j - 2) / TM][(j - 2) % TM] += part[(j - 2) % 3] * sc[(j - 2) % TM];
+                __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) acc[TN - 1][tm] += part[(TN - 1) & 1][tm] * sc[tm];
+            for (int j = NJ - 2; j < NJ; ++j) acc[j / TM][j % TM] += part[j % 3] * sc[j % TM];
+            // Pin the scale-and-add results here: without a use in this block the compiler sinks the
+            // whole VALU chain behind the next conditional (a later K step's loader test), keeps every
+            // 16x16 product alive until then and spills.  No instruction is emitted.
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm) asm volatile("" : "+v"(acc[tn][tm]));
         } else {
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
@@ -501,7 +516,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     issue_b(ks, sB0);
     issue_s(ks, sS0);
     issue_a(min(ks + 1, last), sA1);
-    if (loader) __builtin_amdgcn_s_waitcnt(kWaitAllButA);
+    __builtin_amdgcn_s_waitcnt(kWaitAllButA);  // a wave without loads in flight passes at once
     lds_barrier();
     auto step = [&](int k, uint8_t* cA, uint8_t* cB, float* cS, uint8_t* oB, float* oS) {
         issue_b(min(k + 1, last), oB);
@@ -512,8 +527,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         issue_a(min(k + 2, last), cA);
         mma(cB);
         if constexpr (!BLOCKSCALE) pipeline_hint<TM, TN, A_IT>();
-        else pipeline_hint_scaled<TM, TN, A_IT>();
-        if (loader) __builtin_amdgcn_s_waitcnt(kWaitAllButA);
+        __builtin_amdgcn_s_waitcnt(kWaitAllButA);
         lds_barrier();
     };
     int i = 0;

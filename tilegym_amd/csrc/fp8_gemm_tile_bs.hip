@@ -10,6 +10,7 @@ hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p,
         return split ? launch_tile<BM, BN, WGM, WGN, true, GROUP_DENSE, true>(p, gx, gy, s)      \
                      : launch_tile<BM, BN, WGM, WGN, true, GROUP_DENSE, false>(p, gx, gy, s);    \
     }
+    TG_CASE(256, 256, 4, 2)
     TG_CASE(128, 128, 2, 2)
     TG_CASE(128, 256, 2, 4)
     TG_CASE(64, 128, 1, 4)

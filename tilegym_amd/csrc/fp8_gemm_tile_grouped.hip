@@ -12,6 +12,7 @@ hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p
                    ? launch_tile<BM, BN, WGM, WGN, true, GROUP_RAGGED, false>(p, gx, 1, s)       \
                    : launch_tile<BM, BN, WGM, WGN, true, GROUP_GATHER, false>(p, gx, 1, s);      \
     }
+    TG_CASE(256, 256, 4, 2)
     TG_CASE(128, 128, 2, 2)
     TG_CASE(128, 256, 2, 4)
     TG_CASE(64, 128, 1, 4)

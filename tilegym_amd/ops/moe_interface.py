@@ -99,7 +99,9 @@ def fused_experts_impl(
     cache1 = torch.empty((M, top_k, N), device=device, dtype=out_dtype)
     cache3 = torch.empty((M, top_k, H), device=device, dtype=out_dtype)
     out = hidden_states if inplace else torch.empty((num_tokens, H), device=device, dtype=out_dtype)
-    config = {"BLOCK_SIZE_M": 128}
+    # rows per expert decide the row tile of the grouped GEMMs: 256 once an expert sees >= 192 routed
+    # rows on average (measured on the 64-expert workload), else 128
+    config = {"BLOCK_SIZE_M": 256 if (M * top_k) // max(E, 1) >= 192 else 128}
 
     for chunk in range((num_tokens // CHUNK_SIZE) + 1):
         lo, hi = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
