@@ -417,7 +417,11 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         const int k0 = kstep * kKBlock;
         const uint32_t dst = lds_address(dB) + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < B_IT; ++i) direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
+        for (int i = 0; i < B_IT; ++i) {
+            // the 64-row tile serves M <= 64: one row tile, every weight byte is read once
+            if constexpr (BM == 64) direct_load_b128_nt(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
+            else direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
+        }
     };
     const v4i rsrc_s = make_rsrc(p.As);
     auto issue_s = [&](int kstep, float* dS) {
