@@ -140,6 +140,24 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
                         const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream);
 
 /*
+ * First GEMM of the FP8 MoE layer with its activation fused into the epilogue:
+ *   for every routed slot id:  h = (A[id / top_k] * a_scale) @ (B[e] * b_scale)^T        (2*I columns, rounded to `act_dtype`)
+ *                              act = act_dtype(silu(h[:I]) * h[I:])
+ *                              q[id], scales[id] = 1x128 e4m3 quantization of act (all-zero group -> scale 1)
+ * i.e. tg_fp8_moe_gemm followed by tg_silu_mul_quant_1x128, bit for bit, without the (T*top_k, 2*I) intermediate.
+ * Replaces the GEMM1 + SiLU-and-multiply steps of fused_experts_impl, src/tilegym/ops/moe_interface.py:252-277
+ * (activation: src/tilegym/ops/ops.py:172-193).
+ * b (E, 2*I, K) e4m3 with I % 128 == 0 and K % 128 == 0; q (num_valid, I) e4m3; scales (num_valid, I/128) f32;
+ * act_dtype: TG_BF16 or TG_F16; block_m (the moe_align block size) must be a multiple of 256; the other
+ * arguments as for tg_fp8_moe_gemm.  Shapes outside these limits return TG_ERR_INVALID: call the two-step form.
+ */
+int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* a, const tg_tensor* b,
+                                   const tg_tensor* a_scale, const tg_tensor* b_scale,
+                                   const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
+                                   const tg_tensor* num_tokens_post_padded, int32_t top_k, int32_t block_m,
+                                   int32_t act_dtype, int32_t device_id, uint64_t hip_stream);
+
+/*
  * A list of independent FP8 GEMMs, C_i <- (sa_i * A_i) @ (sb_i * op(B_i)), i < count, in one launch when
  * every problem has (N,K) weights (trans_b != 0), K_i % 128 == 0 and 16-byte aligned operands; any other
  * list is run problem by problem with tg_fp8_gemm's schedules (same results).

@@ -118,6 +118,41 @@ def test_grouped_argument_validation():
     assert moe(expert_ids=torch.zeros(1, dtype=torch.int32)) == -6
 
 
+def test_moe_gemm_silu_quant_argument_validation():
+    L = _lib.load()
+    T, K, E, I, top_k = 6, 256, 2, 128, 2
+
+    def call(q=None, scales=None, a=None, b=None, a_s=None, b_s=None, sorted_ids=None, expert_ids=None, block_m=256,
+             top_k=top_k, act=_lib._DTYPE_CODES[torch.bfloat16]):
+        q = torch.zeros(T * top_k, I).to(FP8) if q is None else q
+        scales = torch.zeros(T * top_k, I // 128) if scales is None else scales
+        a = torch.zeros(T, K).to(FP8) if a is None else a
+        b = torch.zeros(E, 2 * I, K).to(FP8) if b is None else b
+        a_s = torch.ones(T, K // 128) if a_s is None else a_s
+        b_s = torch.ones(E, 2 * I // 128, K // 128) if b_s is None else b_s
+        sorted_ids = torch.zeros(512, dtype=torch.int32) if sorted_ids is None else sorted_ids
+        expert_ids = torch.zeros(2, dtype=torch.int32) if expert_ids is None else expert_ids
+        post = torch.tensor([512], dtype=torch.int32)
+        ds = [_lib.make_tensor_desc(t) for t in (q, scales, a, b, a_s, b_s, sorted_ids, expert_ids, post)]
+        return L.tg_fp8_moe_gemm_silu_quant(*[ctypes.byref(d) for d in ds], top_k, block_m, act, 0, 0)
+
+    assert call(block_m=128) == -6                                          # row tile of the fused form
+    assert call(top_k=0) == -6
+    assert call(act=_lib._DTYPE_CODES[torch.float32]) == -2                 # 16-bit intermediate type only
+    assert call(q=torch.zeros(T * top_k, I, dtype=torch.bfloat16)) == -2
+    assert call(q=torch.zeros(T * top_k, 2 * I).to(FP8)) == -6              # q holds I columns, not 2I
+    assert call(scales=torch.zeros(T * top_k, 2)) == -6
+    assert call(b=torch.zeros(E, 2 * I + 128, K).to(FP8)) == -6             # I % 128
+    assert call(a_s=torch.ones(T, 1)) == -6
+    assert call(b_s=torch.ones(E, 1, K // 128)) == -6
+    assert call(expert_ids=torch.zeros(1, dtype=torch.int32)) == -6
+    assert call(sorted_ids=torch.zeros(512, dtype=torch.int64)) == -2
+    assert call(q=torch.zeros(0, I).to(FP8), scales=torch.zeros(0, 1)) == 0  # nothing to do, no device needed
+    assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * I, K), 128)
+    assert _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * I, K), 256)
+    assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * 200, K), 256)
+
+
 def test_moe_align_argument_validation():
     L = _lib.load()
 

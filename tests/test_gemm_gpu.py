@@ -551,6 +551,62 @@ def test_silu_mul_quant_kernel(device, dtype, R_, I):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,top_k,H,I", [(64, 4, 2, 256, 128), (300, 8, 2, 512, 384), (700, 3, 1, 128, 1408)])
+def test_moe_gemm_silu_quant_equals_the_two_steps(device, dtype, T, E, top_k, H, I):
+    """GEMM1 with the activation and the 1x128 re-quantization in its epilogue returns the very bits of
+    GEMM1 (256-row blocks) followed by the stand-alone activation kernel, and stays within that kernel's
+    bar against the oracle (src/tilegym/ops/moe_interface.py:252-277, src/tilegym/ops/ops.py:172-193)."""
+    g = _g(T + I)
+    A = fp8_randn((T, H), g)
+    B = fp8_randn((E, 2 * I, H), g, 0.5)
+    a_s = torch.rand(T, H // 128, generator=g) * 0.05 + 0.01
+    b_s = torch.rand(E, 2 * I // 128, H // 128, generator=g) + 0.1
+    w, ids = W.moe_routing(T, E, top_k, seed=3)
+    if E > 2:
+        ids[ids == 1] = 2  # an expert without tokens
+    Ad, Bd, asd, bsd = A.to(device), B.to(device), a_s.to(device), b_s.to(device)
+    sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids.to(device), 256, E)
+    C = torch.zeros(T, top_k, 2 * I, dtype=dtype, device=device)
+    invoke_fused_moe_kernel(Ad, Bd, C, asd, bsd, w.to(device), ids.to(device), sorted_ids, expert_ids, post,
+                            False, top_k, {"BLOCK_SIZE_M": 256}, compute_type=dtype, use_fp8_w8a8=True)
+    q2, s2 = _lib.silu_mul_quant_1x128(C.view(T * top_k, 2 * I))
+    assert _lib.moe_gemm_silu_quant_ok(Bd, 256)
+    q, s = _lib.fp8_moe_gemm_silu_quant(Ad, Bd, asd, bsd, sorted_ids, expert_ids, post, top_k, 256, T * top_k, dtype)
+    used("tiled")
+    assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+    # against the oracle: its GEMM1 output rounded to the 16-bit type, then its activation + quantization
+    ref_c = R.ref_fused_moe_gemm(A, B, a_s, b_s, w, ids, False, top_k, out_dtype=dtype).reshape(T * top_k, 2 * I)
+    q_ref, s_ref, _ = R.ref_silu_mul_quant(ref_c)
+    assert torch.allclose(s.cpu(), s_ref, rtol=2e-2, atol=0)
+    deq = R.fp8_to_f32(q.cpu()) * s.cpu().repeat_interleave(128, 1)
+    deq_ref = R.fp8_to_f32(q_ref) * s_ref.repeat_interleave(128, 1)
+    step = s_ref.repeat_interleave(128, 1) * 32
+    # an fp32 re-association difference in the GEMM can move a 16-bit rounding of gate or up, hence two steps
+    assert ((deq - deq_ref).abs() <= 2 * step + 1e-12).float().mean() > 0.9999
+
+
+def test_fused_experts_fp8_fused_activation_path(device):
+    """Enough rows per expert for 256-row blocks: fused_moe takes the GEMM1 + activation + quantization
+    entry point; checked against the oracle of the whole layer."""
+    from tilegym_amd.ops import fused_moe
+
+    g = _g(32)
+    T, E, k, H, I = 600, 4, 2, 256, 384
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w1q, w1s = R.quantize_weight_128x128(torch.randn(E * 2 * I, H, generator=g) * 0.05)
+    w2q, w2s = R.quantize_weight_128x128(torch.randn(E * H, I, generator=g) * 0.05)
+    w1q, w1s = w1q.reshape(E, 2 * I, H), w1s.reshape(E, 2 * I // 128, H // 128)
+    w2q, w2s = w2q.reshape(E, H, I), w2s.reshape(E, H // 128, I // 128)
+    tw, ids = W.moe_routing(T, E, k, seed=5)
+    assert (T * k) // E >= 192 and _lib.moe_gemm_silu_quant_ok(w1q, 256)
+    ref = R.ref_fused_experts_fp8(hidden, w1q, w2q, w1s, w2s, tw, ids)
+    out = fused_moe(hidden.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device),
+                    w1_scale=w1s.to(device), w2_scale=w2s.to(device))
+    ok, rep = R.compare_to_oracle(out, ref, RTOL, ATOL)
+    assert rep["matched"] >= 0.999 and rep["max_rel_to_sigma"] <= 0.1, rep
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_moe_sum_kernel(device, dtype):
     g = _g(8)
     x = torch.randn(37, 6, 264, generator=g).to(dtype)

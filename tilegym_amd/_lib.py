@@ -100,6 +100,9 @@ def load():
     L.tg_fp8_moe_gemm.restype = ctypes.c_int32
     L.tg_fp8_moe_gemm.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_int32, ctypes.c_int32,
                                   ctypes.c_int32, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_moe_gemm_silu_quant.restype = ctypes.c_int32
+    L.tg_fp8_moe_gemm_silu_quant.argtypes = [P, P, P, P, P, P, P, P, P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                                             ctypes.c_int32, ctypes.c_uint64]
     L.tg_moe_align_block_size.restype = ctypes.c_int32
     L.tg_moe_align_block_size.argtypes = [P, ctypes.c_int32, ctypes.c_int32, P, P, P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_fp8_quant_1x128.restype = ctypes.c_int32
@@ -244,6 +247,28 @@ def fp8_moe_gemm(c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids, expe
     rc = L.tg_fp8_moe_gemm(*[_ref(d) for d in ds], int(bool(mul_routed_weight)), int(top_k),
                            int(block_m), cfg, ncfg, dev, _stream_handle(a))
     check_rc(rc, "tg_fp8_moe_gemm")
+
+
+def moe_gemm_silu_quant_ok(b, block_m) -> bool:
+    """Shapes the fused GEMM1 + SiLU-multiply + 1x128 quantization entry point accepts."""
+    two_i, k = b.shape[1], b.shape[2]
+    return two_i % 256 == 0 and k % 128 == 0 and 128 <= k <= 65536 and block_m % 256 == 0
+
+
+def fp8_moe_gemm_silu_quant(a, b, a_scale, b_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                            top_k, block_m, num_valid, act_dtype):
+    """tg_fp8_moe_gemm_silu_quant: returns (q (num_valid, I) e4m3, scales (num_valid, I/128) f32)."""
+    import torch
+    L = load()
+    dev = _device_index(a)
+    inter = b.shape[1] // 2
+    q = torch.empty((num_valid, inter), dtype=torch.float8_e4m3fn, device=a.device)
+    scales = torch.empty((num_valid, inter // 128), dtype=torch.float32, device=a.device)
+    ds = [make_tensor_desc(t) for t in (q, scales, a, b, a_scale, b_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)]
+    rc = L.tg_fp8_moe_gemm_silu_quant(*[_ref(d) for d in ds], int(top_k), int(block_m), _DTYPE_CODES[act_dtype], dev,
+                                      _stream_handle(a))
+    check_rc(rc, "tg_fp8_moe_gemm_silu_quant")
+    return q, scales
 
 
 MOE_ALIGN_MAX_EXPERTS = 512

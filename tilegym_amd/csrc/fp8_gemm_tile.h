@@ -247,6 +247,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     static_assert(WTM * PCOLS * 4 * (NW / 4) <= OBJ && PCOLS >= 16, "epilogue slice fits");
     static_assert(!BLOCKSCALE || (WTN <= 128 && 128 % WTN == 0), "one weight scale per wave");
     static_assert(!SPLIT || GROUP == GROUP_DENSE, "split-K is dense only");
+    // fused activation epilogue (MoE gate/up GEMM): a tile is 128 gate columns + the 128 matching up columns
+    constexpr bool ACT = GROUP == GROUP_GATHER_ACT;
+    static_assert(!ACT || (BLOCKSCALE && BM == 256 && BN == 256 && WGM == 4 && WGN == 2), "fused activation: block-scaled 256x256 only");
 
     __shared__ __align__(1024) uint8_t sA0[BM * kKBlock];
     __shared__ __align__(1024) uint8_t sA1[BM * kKBlock];
@@ -263,7 +266,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = wave / WGM;
-    const int tiles_n = (p.N + BN - 1) / BN;
+    const int tiles_n = ACT ? p.inter / 128 : (p.N + BN - 1) / BN;
     const int K = p.K;
 
     // ---------------------------------------------------------------- which tile
@@ -314,7 +317,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         Bbase += (int64_t)e * p.N * K;
         if (Bsbase) Bsbase += (int64_t)e * p.nblocks * p.kblocks;
     }
-    const int n0 = tile_n * BN;
+    const int n0 = ACT ? tile_n * 128 : tile_n * BN;  // ACT: first gate column of the tile
 
     if constexpr (GROUP != GROUP_DENSE) {
         for (int r = tid; r < BM; r += NT) {
@@ -356,7 +359,10 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     }
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
-        const int n = min(n0 + (i * NL + (wave % NL)) * 8 + lrow, p.N - 1);
+        const int br = (i * NL + (wave % NL)) * 8 + lrow;  // slab row
+        int n;
+        if constexpr (ACT) n = br < 128 ? n0 + br : p.inter + n0 + (br - 128);  // gate rows, then the up rows
+        else n = min(n0 + br, p.N - 1);
         b_off[i] = (uint32_t)n * (uint32_t)K + lj * 16;
     }
 
@@ -375,7 +381,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         constexpr int NBT = (BN + 127) / 128;
         for (int idx = tid; idx < NBT * p.kblocks; idx += NT) {
             const int j = idx / p.kblocks, kb = idx % p.kblocks;
-            const int nb = min(n0 / 128 + j, p.nblocks - 1);
+            const int nb = ACT ? (j == 0 ? n0 / 128 : (p.inter + n0) / 128) : min(n0 / 128 + j, p.nblocks - 1);
             sBs[j][kb] = Bsbase ? Bsbase[(int64_t)nb * p.kblocks + kb] : 1.0f;
         }
         const int r = min(wave * 64 + lane, BM - 1);
@@ -542,6 +548,88 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     if (i < nsteps) step(ks + i, sA0, sB0, sS0, sB1, sS1);
     __builtin_amdgcn_s_waitcnt(kWaitAll);
     __syncthreads();
+
+    // ---------------------------------------------------------------- fused activation epilogue
+    // Wave (wm, 0) holds the tile's 128 gate columns of rows 64*wm .. 64*wm+63, wave (wm, 1) the
+    // matching up columns.  In four passes of 32 columns every wave stages its slice through LDS
+    // (fp32, 8 KiB per wave; the passes alternate between the A and the B slabs, so one barrier per
+    // pass suffices), then the two waves of a row group take 32 rows each, read gate and up of the
+    // same elements and compute, exactly as the stand-alone kernel does on the stored GEMM output:
+    //   g = T(acc_gate), u = T(acc_up), act = T(g * sigmoid(g) * u)          (T = the 16-bit type)
+    // A row's 128 activations sit in 4 lanes x 4 passes; after the last pass the row maximum is
+    // reduced over those lanes, the scale (amax / 448, 1 for an all-zero group) is formed with an
+    // IEEE division and the codes are written 8 bytes per lane and pass.
+    if constexpr (ACT) {
+        constexpr int APC = 32, APASS = WTN / APC;  // staged columns per pass
+        float actv[APASS][2][8];
+        const int rsel = wn * 32;                   // this wave's half of the 64 rows
+        const int arr = lane >> 2, ac8 = (lane & 3) * 8;
+#pragma unroll
+        for (int ps = 0; ps < APASS; ++ps) {
+            uint8_t* const set_lo = (ps & 1) ? sB0 : sA0;  // waves 0..3 (gate), 4 x 8 KiB
+            uint8_t* const set_hi = (ps & 1) ? sB1 : sA1;  // waves 4..7 (up)
+            uint8_t* const mine = (wn == 0 ? set_lo : set_hi) + wm * (WTM * APC * 4);
+#pragma unroll
+            for (int t = 0; t < APC / 16; ++t)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm) {
+                    const int r = tm * 16 + li;
+                    const int u = (t * 4 + lg) ^ (r & 7);
+                    *reinterpret_cast<v4f*>(mine + r * (APC * 4) + u * 16) = acc[ps * (APC / 16) + t][tm];
+                }
+            __syncthreads();
+            const uint8_t* gsrc = set_lo + wm * (WTM * APC * 4);
+            const uint8_t* usrc = set_hi + wm * (WTM * APC * 4);
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                const int r = rsel + it * 16 + arr;
+                const int u0 = (ac8 >> 2) ^ (r & 7), u1 = ((ac8 >> 2) + 1) ^ (r & 7);
+                const v4f g0 = *reinterpret_cast<const v4f*>(gsrc + r * (APC * 4) + u0 * 16);
+                const v4f g1 = *reinterpret_cast<const v4f*>(gsrc + r * (APC * 4) + u1 * 16);
+                const v4f p0 = *reinterpret_cast<const v4f*>(usrc + r * (APC * 4) + u0 * 16);
+                const v4f p1 = *reinterpret_cast<const v4f*>(usrc + r * (APC * 4) + u1 * 16);
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const float ga = q < 4 ? g0[q & 3] : g1[q & 3], ua = q < 4 ? p0[q & 3] : p1[q & 3];
+                    if (p.act_is_bf16) actv[ps][it][q] = silu_mul_round<__bf16>((float)(__bf16)ga, (float)(__bf16)ua);
+                    else actv[ps][it][q] = silu_mul_round<_Float16>((float)(_Float16)ga, (float)(_Float16)ua);
+                }
+            }
+        }
+        uint8_t* const qout = reinterpret_cast<uint8_t*>(p.C);
+        const int groups_per_row = p.inter / 128;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            float amax = 0.f;
+#pragma unroll
+            for (int ps = 0; ps < APASS; ++ps)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) amax = fmaxf(amax, fabsf(actv[ps][it][q]));
+            amax = fmaxf(amax, __shfl_xor(amax, 1));
+            amax = fmaxf(amax, __shfl_xor(amax, 2));
+            const float sc1 = amax == 0.f ? 1.0f : amax / 448.0f;
+            const int rt = wm * WTM + rsel + it * 16 + arr;
+            const int dst = s_dst[rt];
+            if (dst < 0) continue;
+#pragma unroll
+            for (int ps = 0; ps < APASS; ++ps) {
+                int packed[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    float c[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) c[i] = fminf(fmaxf(actv[ps][it][4 * h + i] / sc1, -448.0f), 448.0f);
+                    int w = 0;
+                    w = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], w, false);
+                    w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
+                    packed[h] = w;
+                }
+                *reinterpret_cast<v2i*>(qout + (int64_t)dst * p.inter + n0 + ps * APC + ac8) = v2i{packed[0], packed[1]};
+            }
+            if ((lane & 3) == 0) p.act_scales[(int64_t)dst * groups_per_row + tile_n] = sc1;
+        }
+        return;
+    }
 
     // ---------------------------------------------------------------- epilogue
     // Every wave is past the last barrier, so the stage buffers are free: wave w stages through

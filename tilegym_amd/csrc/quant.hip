@@ -93,10 +93,7 @@ __global__ void __launch_bounds__(256) silu_mul_quant_kernel(const T* __restrict
         const v8f_q up = load8<T>(x + row * (2 * (int64_t)I) + I + col);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            // sigmoid with the hardware exponential and reciprocal (about 2 ulp in fp32, far below the
-            // 16-bit rounding that follows); the quantization below keeps its IEEE divisions
-            const float sl = gate[i] * __builtin_amdgcn_rcpf(1.0f + __expf(-gate[i]));
-            act[i] = (float)(T)(sl * up[i]);
+            act[i] = silu_mul_round<T>(gate[i], up[i]);  // the quantization below keeps its IEEE divisions
         }
     }
     float amax = 0.f;

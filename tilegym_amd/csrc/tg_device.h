@@ -17,7 +17,9 @@ constexpr int kKBlock = 128;    // bytes of K consumed by one 16x16x128 MFMA = t
 enum OutType { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2 };  // same numbering as the ABI dtype codes
 
 // How rows of the activation operand are found.
-enum GroupMode { GROUP_DENSE = 0, GROUP_RAGGED = 1, GROUP_GATHER = 2 };
+// GROUP_GATHER_ACT: the gather form for a (E, 2I, K) gate/up weight whose epilogue produces
+// act = silu(gate) * up, quantized 1 x 128 to e4m3, instead of the GEMM output.
+enum GroupMode { GROUP_DENSE = 0, GROUP_RAGGED = 1, GROUP_GATHER = 2, GROUP_GATHER_ACT = 3 };
 
 struct GemmParams {
     const uint8_t* A;   // activations, (M,K) row-major, e4m3
@@ -43,6 +45,12 @@ struct GemmParams {
     const int* num_post_pad;  // gather: (1)
     const float* row_weight;  // gather: (num_valid) or null
     int top_k, num_valid, block_m, em_capacity;
+    // GROUP_GATHER_ACT: I (gate rows are B[e][0:I], up rows B[e][I:2I]); C is then the (num_valid, I)
+    // e4m3 activation and act_scales its (num_valid, I/128) fp32 scales; act_is_bf16 says which
+    // 16-bit type the GEMM output and the activation are rounded to on the way
+    int inter;
+    float* act_scales;
+    int act_is_bf16;
 };
 
 // A list of independent per-tensor-scaled NT GEMMs handed to one launch in the kernel arguments.
@@ -144,6 +152,20 @@ __device__ __forceinline__ int xcd_remap(int pid, int nblk) {
     int q = nblk / X, r = nblk % X;
     int x = pid % X, idx = pid / X;
     return x * q + (x < r ? x : r) + idx;
+}
+
+// silu(gate) * up rounded to the 16-bit type T, with gate and up already values of T.  The sigmoid uses
+// the hardware exponential and reciprocal (about 2 ulp in fp32, far below the 16-bit rounding that
+// follows).  The fp32 product is rounded on its own and only then converted: the empty asm keeps the
+// compiler from folding multiply and conversion into one mixed-precision FMA, which rounds once (and
+// gives a zero product the sign of its zero addend), so that every kernel that calls this returns the
+// same bits as separate fp32 multiply and conversion steps do.
+template <typename T>
+__device__ __forceinline__ float silu_mul_round(float gate, float up) {
+    const float sl = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate));
+    float prod = sl * up;
+    asm volatile("" : "+v"(prod));
+    return (float)(T)prod;
 }
 
 }  // namespace tg

@@ -657,6 +657,87 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
     return TG_OK;
 }
 
+int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* a, const tg_tensor* b,
+                                   const tg_tensor* a_scale, const tg_tensor* b_scale,
+                                   const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
+                                   const tg_tensor* num_tokens_post_padded, int32_t top_k, int32_t block_m,
+                                   int32_t act_dtype, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(a, "a", 2)) || (rc = check_tensor(b, "b", 3)) || (rc = check_tensor(q, "q", 2)) ||
+        (rc = check_tensor(scales, "scales", 2)) || (rc = check_tensor(a_scale, "a_scale", 2)) ||
+        (rc = check_tensor(b_scale, "b_scale", 3)) || (rc = check_tensor(sorted_token_ids, "sorted_token_ids", 1)) ||
+        (rc = check_tensor(expert_ids, "expert_ids", 1)) || (rc = check_tensor(num_tokens_post_padded, "num_tokens_post_padded", -1)))
+        return rc;
+    if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN || q->dtype != TG_F8E4M3FN)
+        return fail(TG_ERR_DTYPE, "a, b and q must be float8_e4m3fn (dtype code 7)");
+    if (scales->dtype != TG_F32 || a_scale->dtype != TG_F32 || b_scale->dtype != TG_F32)
+        return fail(TG_ERR_DTYPE, "scales, a_scale and b_scale must be f32");
+    if (act_dtype != TG_BF16 && act_dtype != TG_F16) return fail(TG_ERR_DTYPE, "act_dtype must be bf16 or f16");
+    if (sorted_token_ids->dtype != TG_I32 || expert_ids->dtype != TG_I32 || num_tokens_post_padded->dtype != TG_I32)
+        return fail(TG_ERR_DTYPE, "sorted_token_ids, expert_ids and num_tokens_post_padded must be int32");
+    const int64_t T = a->shape[0], K = a->shape[1], E = b->shape[0], N = b->shape[1], I = N / 2;
+    if (b->shape[2] != K) return fail(TG_ERR_INVALID, "K dimensions must match: %lld != %lld", (long long)K, (long long)b->shape[2]);
+    if (N % 2 || I % 128 || I == 0) return fail(TG_ERR_INVALID, "b must hold 2*I rows per expert with I a positive multiple of 128 (got %lld)", (long long)N);
+    if (K % 128 || K == 0 || K > 65536) return fail(TG_ERR_INVALID, "K must be a multiple of 128 in [128, 65536]");
+    if (top_k <= 0) return fail(TG_ERR_INVALID, "top_k must be positive");
+    if (block_m <= 0 || block_m % 256) return fail(TG_ERR_INVALID, "block_m must be a positive multiple of 256 for the fused form");
+    const int64_t num_valid = q->shape[0];
+    if (q->shape[1] != I) return fail(TG_ERR_INVALID, "q must have %lld columns", (long long)I);
+    if (num_valid > T * top_k) return fail(TG_ERR_INVALID, "q has %lld rows but a provides only %lld slots", (long long)num_valid, (long long)(T * top_k));
+    if (scales->shape[0] != num_valid || scales->shape[1] != I / 128)
+        return fail(TG_ERR_INVALID, "scales must be (%lld, %lld)", (long long)num_valid, (long long)(I / 128));
+    if (a_scale->shape[0] != T || a_scale->shape[1] != K / 128) return fail(TG_ERR_INVALID, "a_scale must be (%lld, %lld)", (long long)T, (long long)(K / 128));
+    if (b_scale->shape[0] != E || b_scale->shape[1] != N / 128 || b_scale->shape[2] != K / 128)
+        return fail(TG_ERR_INVALID, "b_scale must be (%lld, %lld, %lld)", (long long)E, (long long)(N / 128), (long long)(K / 128));
+    if (!contiguous(q) || !contiguous(scales) || !contiguous(a) || !contiguous(b) || !contiguous(a_scale) || !contiguous(b_scale))
+        return fail(TG_ERR_INVALID, "all tensors must be contiguous");
+    if (numel(num_tokens_post_padded) < 1) return fail(TG_ERR_INVALID, "num_tokens_post_padded must hold one element");
+    const int64_t EM = sorted_token_ids->shape[0];
+    if (expert_ids->shape[0] * block_m < EM)
+        return fail(TG_ERR_INVALID, "expert_ids too short: %lld blocks of %d for %lld slots", (long long)expert_ids->shape[0], block_m, (long long)EM);
+    if (T > INT32_MAX || N > INT32_MAX || E > INT32_MAX || T * K >= kOffsetLimit || N * K >= kOffsetLimit)
+        return fail(TG_ERR_INVALID, "extent too large for the fused form");
+    if (!aligned16(a->ptr) || !aligned16(b->ptr) || (q->ptr % 8) != 0) return fail(TG_ERR_INVALID, "a and b must be 16-byte aligned, q 8-byte aligned");
+    if (num_valid == 0 || EM == 0) return TG_OK;
+
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+
+    tg::GemmParams p{};
+    p.A = reinterpret_cast<const uint8_t*>(a->ptr);
+    p.B = reinterpret_cast<const uint8_t*>(b->ptr);
+    p.C = reinterpret_cast<void*>(q->ptr);
+    p.As = reinterpret_cast<const float*>(a_scale->ptr);
+    p.Bs = reinterpret_cast<const float*>(b_scale->ptr);
+    p.M = (int)num_valid; p.N = (int)N; p.K = (int)K;
+    p.kblocks = (int)(K / 128); p.nblocks = (int)(N / 128);
+    p.alpha = 1.0f; p.beta = 0.0f;
+    p.out_type = act_dtype == TG_BF16 ? tg::OUT_BF16 : tg::OUT_F16;
+    p.split_k = 1;
+    p.ksteps_per_split = p.kblocks;
+    p.E = (int)E;
+    p.sorted_ids = reinterpret_cast<const int*>(sorted_token_ids->ptr);
+    p.expert_ids = reinterpret_cast<const int*>(expert_ids->ptr);
+    p.num_post_pad = reinterpret_cast<const int*>(num_tokens_post_padded->ptr);
+    p.top_k = top_k;
+    p.num_valid = (int)num_valid;
+    p.block_m = block_m;
+    p.em_capacity = (int)EM;
+    p.inter = (int)I;
+    p.act_scales = reinterpret_cast<float*>(scales->ptr);
+    p.act_is_bf16 = act_dtype == TG_BF16 ? 1 : 0;
+
+    Schedule s{1, 256, 256, 1, -1, -1, -1};
+    remember(s);
+    const int64_t gx = cdiv(EM, 256) * (I / 128);
+    if (gx > INT32_MAX) return fail(TG_ERR_INVALID, "too many tiles");
+    hipError_t e = tg::run_tile_moe_act(p, (int)gx, stream);
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "fused MoE kernel launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
 int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
                                 const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
                                 const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,

@@ -96,12 +96,13 @@ def fused_experts_impl(
     out_dtype = torch.bfloat16 if hidden_states.dtype == torch.bfloat16 else torch.float16
     CHUNK_SIZE = 32768
     M = min(num_tokens, CHUNK_SIZE)
-    cache1 = torch.empty((M, top_k, N), device=device, dtype=out_dtype)
+    cache1 = None
     cache3 = torch.empty((M, top_k, H), device=device, dtype=out_dtype)
     out = hidden_states if inplace else torch.empty((num_tokens, H), device=device, dtype=out_dtype)
     # rows per expert decide the row tile of the grouped GEMMs: 256 once an expert sees >= 192 routed
     # rows on average (measured on the 64-expert workload), else 128
     config = {"BLOCK_SIZE_M": 256 if (M * top_k) // max(E, 1) >= 192 else 128}
+    fuse_act = _lib.moe_gemm_silu_quant_ok(w1, config["BLOCK_SIZE_M"]) and w1_scale is not None
 
     for chunk in range((num_tokens // CHUNK_SIZE) + 1):
         lo, hi = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
@@ -110,15 +111,25 @@ def fused_experts_impl(
             break
         cur = hidden_states[lo:hi]
         ids, weights = topk_ids[lo:hi].contiguous(), topk_weights[lo:hi].contiguous()
-        c1, c3 = cache1[:n], cache3[:n]
+        c3 = cache3[:n]
+        if not fuse_act:
+            if cache1 is None:
+                cache1 = torch.empty((M, top_k, N), device=device, dtype=out_dtype)
+            c1 = cache1[:n]
         if cur.dtype == FP8:
             xq, xs = cur, a1_scale[lo:hi]
         else:
             xq, xs = quant.act_quant(cur if cur.dtype != torch.float32 else cur.to(out_dtype), 128)
         sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids, config["BLOCK_SIZE_M"], E)
-        invoke_fused_moe_kernel(xq, w1, c1, xs, w1_scale, weights, ids, sorted_ids, expert_ids, post,
-                                False, top_k, config, compute_type=out_dtype, use_fp8_w8a8=True)
-        q2, s2 = _lib.silu_mul_quant_1x128(c1.view(n * top_k, N))
+        if fuse_act:
+            # GEMM1 with SiLU(gate) * up and the 1x128 re-quantization in its epilogue: same bits as the
+            # two steps below, without writing and re-reading the (n * top_k, 2I) intermediate
+            q2, s2 = _lib.fp8_moe_gemm_silu_quant(xq, w1, xs, w1_scale, sorted_ids, expert_ids, post, top_k,
+                                                  config["BLOCK_SIZE_M"], n * top_k, out_dtype)
+        else:
+            invoke_fused_moe_kernel(xq, w1, c1, xs, w1_scale, weights, ids, sorted_ids, expert_ids, post,
+                                    False, top_k, config, compute_type=out_dtype, use_fp8_w8a8=True)
+            q2, s2 = _lib.silu_mul_quant_1x128(c1.view(n * top_k, N))
         invoke_fused_moe_kernel(q2, w2, c3, s2, w2_scale, weights, ids, sorted_ids, expert_ids, post,
                                 True, 1, config, compute_type=out_dtype, use_fp8_w8a8=True)
         if top_k == 1:
