@@ -341,6 +341,25 @@ def main():
             del r
             torch.cuda.empty_cache()
         detail["moe_grouped"] = shapes
+        # the whole FP8 MoE layer those GEMMs sit in (fused_moe: align, 1x128 activation quantizer, GEMM1 with the
+        # SiLU-multiply + re-quantization epilogue, GEMM2 with the routed weights, top-k sum)
+        from tilegym_amd.ops import fused_moe
+        up, down = W.moe_grouped_case("gate_up"), W.moe_grouped_case("down")
+        ids, tw = up.extra["topk_ids"].to(device), up.extra["topk_weights"].to(device)
+        T, H, I = ids.shape[0], up.b.shape[2], down.b.shape[2]
+        hidden = torch.randn(T, H, device=device).to(torch.bfloat16)
+        w1, w2, s1, s2 = up.b.to(device), down.b.to(device), up.b_scale.to(device), down.b_scale.to(device)
+        fn = lambda i: fused_moe(hidden, w1, w2, tw, ids, w1_scale=s1, w2_scale=s2)  # noqa: E731
+        for w in range(max(2, args.warmup)):
+            fn(w)
+        n = max(args.steps, 20)
+        us = _events_ms(fn, n, stream) * 1e3 / n
+        flops = 2.0 * T * ids.shape[1] * (2 * I * H + H * I)
+        detail["moe_layer"] = [{"name": f"c5_fused_moe_T{T}_E{w1.shape[0]}_top{ids.shape[1]}_H{H}_I{I}", "us": round(us, 2),
+                                "tflops": round(flops / us * 1e-6, 1), "frac_mfma": round(flops / us * 1e-6 / PEAK_FP8_TFLOPS, 4),
+                                "note": "five launches per call, outputs allocated by torch inside the timed region"}]
+        del hidden, w1, w2, s1, s2
+        torch.cuda.empty_cache()
 
     if args.workload in ("quant", "all"):
         # the producers either side of the GEMM: 1x128 activation quantizer (HBM-bound) and moe_align_block_size

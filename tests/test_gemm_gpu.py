@@ -465,11 +465,13 @@ def test_moe_fc2_shape_top_k_1(device):
 
 @pytest.mark.parametrize("T,top_k,E,bs,dtype", [(4, 3, 4, 4, torch.int64), (1, 1, 1, 16, torch.int32), (77, 6, 64, 16, torch.int64),
                                                  (4096, 6, 64, 128, torch.int32), (1000, 2, 512, 64, torch.int64),
-                                                 (333, 8, 8, 1, torch.int32), (50, 4, 600, 32, torch.int64)])
+                                                 (333, 8, 8, 1, torch.int32), (50, 4, 600, 32, torch.int64),
+                                                 (7001, 6, 160, 256, torch.int32), (1025, 1, 3, 64, torch.int64)])
 def test_moe_align_kernel_matches_oracle(device, T, top_k, E, bs, dtype):
     """All five outputs, bit for bit, against the oracle (stable order inside an expert, sentinel
-    fill, padded prefix sums); empty experts, one expert, block size 1, int32 and int64 ids, and
-    more experts than the one-launch kernel takes (torch device ops then)."""
+    fill, padded prefix sums); empty experts, one expert, block size 1, int32 and int64 ids, one to
+    the largest number of workgroups (one per 1024 ids, at most 32), slices that end inside the last
+    workgroup, and more experts than the one-launch kernel takes (torch device ops then)."""
     g = _g(T + E)
     ids = torch.randint(0, E, (T, top_k), generator=g)
     if E >= 8:
