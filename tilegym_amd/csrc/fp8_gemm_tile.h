@@ -24,6 +24,8 @@
 // src/tilegym/suites/flashinfer/cutile/gemm/ragged_block_scaled_bmm.py:71-91) and gather
 // (sorted_token_ids / expert_ids, the contract of src/tilegym/ops/tilecpp/moe.cuh:72-225).
 #pragma once
+#include <type_traits>
+
 #include "tg_device.h"
 
 namespace tg {
@@ -86,6 +88,8 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 // conflict free with this XOR (8 clocks per 1 KiB wave-read, the LDS's full rate); additive
 // variants are 2-way conflicted.
 __device__ __forceinline__ int swz16(int r) { return r & 7; }
+// chunk swizzle of the weight slab: row bits 0, 1 and 3
+__device__ __forceinline__ int swz_w(int r) { return (r & 3) | ((r >> 1) & 4); }
 
 // Number of BM-row tiles over all experts (every lane returns the same value).
 __device__ __forceinline__ int ragged_count_tiles(const int* indptr, int E, int BM, int lane) {
@@ -235,16 +239,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     constexpr int NL = NW == 8 ? 4 : NW;  // waves that issue the direct global->LDS loads
     constexpr int RPP = 8 * NL;           // slab rows filled per pass of the loader waves
     constexpr int A_IT = BM / RPP, B_IT = BN / RPP;
-    // epilogue slices: PCOLS columns of the wave tile at a time, fp32, through one LDS object
-    constexpr int OBJ = (BM < BN ? BM : BN) * kKBlock;  // bytes of the smaller stage object
-    constexpr int PC0 = WTN < 64 ? WTN : 64;
-    constexpr int PCOLS = (WTM * PC0 * 4 * (NW / 4) <= OBJ) ? PC0 : PC0 / 2;
-    constexpr int TNG = PCOLS / 16, PASSES = TN / TNG;
-    constexpr int UNITS = PCOLS / 4;  // 16-byte units per staged row
-    static_assert(NW == 4 || NW == 8, "epilogue staging: NW/4 waves share one LDS object");
-    static_assert(BM % RPP == 0 && BN % RPP == 0, "loader shape");
-    static_assert(WTM % 16 == 0 && WTN % 16 == 0 && TN % TNG == 0, "wave tile");
-    static_assert(WTM * PCOLS * 4 * (NW / 4) <= OBJ && PCOLS >= 16, "epilogue slice fits");
+    static_assert(NW == 4 || NW == 8, "wave grid");
+    static_assert(BM % RPP == 0 && BN % RPP == 0 && NL % 2 == 0, "loader shape");
+    static_assert(WTM % 16 == 0 && WTN % 32 == 0, "wave tile: column tiles are taken in pairs");
     static_assert(!BLOCKSCALE || (WTN <= 128 && 128 % WTN == 0), "one weight scale per wave");
     static_assert(!SPLIT || GROUP == GROUP_DENSE, "split-K is dense only");
     // fused activation epilogue (MoE gate/up GEMM): a tile is 128 gate columns + the 128 matching up columns
@@ -262,6 +259,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     __shared__ float sBs[BLOCKSCALE ? (BN + 127) / 128 : 1][BLOCKSCALE ? kMaxKBlocks : 1];
     __shared__ int s_src[GROUP == GROUP_DENSE ? 1 : BM];
     __shared__ int s_dst[GROUP == GROUP_DENSE ? 1 : BM];
+    // routed weight of each tile row (gather GEMM with mul_routed_weight), fetched once with the row
+    // maps: a load inside the epilogue's row loop would put a global-memory latency on every iteration
+    __shared__ float s_w[GROUP == GROUP_GATHER ? BM : 1];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -334,6 +334,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
             }
             s_src[r] = src;
             s_dst[r] = dst;
+            if constexpr (GROUP == GROUP_GATHER) s_w[r] = (p.row_weight && dst >= 0) ? p.row_weight[dst] : 1.0f;
         }
         __syncthreads();
     }
@@ -346,6 +347,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // logical chunk (l%8) ^ swz16(row) = (l%8) ^ (l/8).
     const int lrow = lane >> 3;
     const int lj = (lane & 7) ^ swz16(lrow);
+    // weight slab: its own swizzle (see the fragment addresses below).  Row 8g + lrow with g = i*NL + wave:
+    // NL is even, so bit 3 of the row is the parity of the loader wave.
+    const int ljb = (lane & 7) ^ swz_w(((wave & 1) << 3) | lrow);
     // (with NL == NW every wave loads: no test, and so no branch inside the K loop)
     const bool loader = NL == NW || wave < NL;
     uint32_t a_off[A_IT], b_off[B_IT];
@@ -363,12 +367,22 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         int n;
         if constexpr (ACT) n = br < 128 ? n0 + br : p.inter + n0 + (br - 128);  // gate rows, then the up rows
         else n = min(n0 + br, p.N - 1);
-        b_off[i] = (uint32_t)n * (uint32_t)K + lj * 16;
+        b_off[i] = (uint32_t)n * (uint32_t)K + ljb * 16;
     }
 
     const int li = lane & 15, lg = lane >> 4;
     const uint32_t frag0 = li * kKBlock + ((lg ^ swz16(li)) << 4);
     const uint32_t frag1 = frag0 ^ 64;
+    // Weight fragments.  Row r of column tile tn (the MFMA's 16 output columns) is slab row
+    //   (tn/2)*32 + (r/4)*8 + (tn%2)*4 + r%4
+    // instead of tn*16 + r: a lane's four accumulator columns 4*lg .. 4*lg+3 of tiles 2t and 2t+1 are then
+    // the eight CONSECUTIVE output columns 32t + 8*lg .. +7, which the epilogue stores straight from
+    // registers as one 16-byte write.  The slab's chunk swizzle uses row bits 0, 1 and 3 (the bits that
+    // vary over a fragment's sixteen rows besides the repeated one), so the reads stay conflict-free.
+    const int wrow = ((li >> 2) << 3) | (li & 3);
+    const uint32_t wfrag0 = wrow * kKBlock + ((lg ^ swz_w(wrow)) << 4);
+    const uint32_t wfrag1 = wfrag0 ^ 64;
+    auto w_tile_row = [](int tn) { return (tn >> 1) * 32 + (tn & 1) * 4; };
     const uint32_t a_frag_base = wm * WTM * kKBlock, b_frag_base = wn * WTN * kKBlock;
 
     // block scales: the activation scales of a K step travel with its slabs (one 4-byte direct
@@ -466,8 +480,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
             v4f part[3];
             v8i wf[2];
             auto read_w = [&](int tn) {
-                const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
-                wf[tn & 1] = join(*reinterpret_cast<const v4i*>(base + frag0), *reinterpret_cast<const v4i*>(base + frag1));
+                const uint8_t* base = cB + b_frag_base + w_tile_row(tn) * kKBlock;
+                wf[tn & 1] = join(*reinterpret_cast<const v4i*>(base + wfrag0), *reinterpret_cast<const v4i*>(base + wfrag1));
             };
             read_w(0);
 #pragma unroll
@@ -490,9 +504,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         } else {
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
-                const uint8_t* base = cB + b_frag_base + tn * 16 * kKBlock;
-                const v8i wf = join(*reinterpret_cast<const v4i*>(base + frag0),
-                                    *reinterpret_cast<const v4i*>(base + frag1));
+                const uint8_t* base = cB + b_frag_base + w_tile_row(tn) * kKBlock;
+                const v8i wf = join(*reinterpret_cast<const v4i*>(base + wfrag0),
+                                    *reinterpret_cast<const v4i*>(base + wfrag1));
 #pragma unroll
                 for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
             }
@@ -574,7 +588,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
 #pragma unroll
                 for (int tm = 0; tm < TM; ++tm) {
                     const int r = tm * 16 + li;
-                    const int u = (t * 4 + lg) ^ (r & 7);
+                    const int u = (lg * 2 + t) ^ (r & 7);  // columns 8*lg + 4*t .. +3 of the pass
                     *reinterpret_cast<v4f*>(mine + r * (APC * 4) + u * 16) = acc[ps * (APC / 16) + t][tm];
                 }
             __syncthreads();
@@ -632,55 +646,44 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     }
 
     // ---------------------------------------------------------------- epilogue
-    // Every wave is past the last barrier, so the stage buffers are free: wave w stages through
-    // the w-th of them.  A staged row holds PCOLS fp32; 16-byte unit u of row r sits at unit
-    // position u ^ (r % UNITS) so that both the accumulator writes (16 lanes = 16 rows, same
-    // unit) and the row-wise reads spread over the banks.
+    // Straight from the accumulators: for every pair of column tiles a lane holds eight consecutive
+    // output columns of row 16*tm + li (see the weight fragment addresses), i.e. one 16-byte store of
+    // bf16/f16 or two of fp32; the four lanes of a row cover 32 consecutive columns.
     float scale = p.alpha;
     if constexpr (!BLOCKSCALE) {
         if (p.As) scale *= p.As[0];
         if (p.Bs) scale *= p.Bs[0];
     }
     const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;  // 8-wide rows stay 16-byte aligned
-    uint8_t* stage_buf = (wave & 3) == 0 ? sA0 : (wave & 3) == 1 ? sA1 : (wave & 3) == 2 ? sB0 : sB1;
-    stage_buf += (wave >> 2) * (WTM * PCOLS * 4);
     const int64_t MN = (int64_t)p.M * p.N;
-
+    int dsts[TM];
+    float rws[TM];
 #pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
+    for (int tm = 0; tm < TM; ++tm) {
+        const int rt = wm * WTM + tm * 16 + li;  // row inside the workgroup tile
+        if constexpr (GROUP == GROUP_DENSE) dsts[tm] = rt < rows_valid ? m0 + rt : -1;
+        else dsts[tm] = s_dst[rt];
+        rws[tm] = scale;
+        if constexpr (GROUP == GROUP_GATHER) rws[tm] *= s_w[rt];
+    }
+    auto emit = [&](auto type_tag) {
+        constexpr int OT = decltype(type_tag)::value;
 #pragma unroll
-        for (int t = 0; t < TNG; ++t)
+        for (int tp = 0; tp < TN / 2; ++tp) {
+            const int col = n0 + wn * WTN + tp * 32 + lg * 8;
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm) {
-                const int r = tm * 16 + li;
-                const int u = (t * 4 + lg) ^ (r & (UNITS - 1));
-                *reinterpret_cast<v4f*>(stage_buf + r * (PCOLS * 4) + u * 16) = acc[ps * TNG + t][tm];
-            }
-        // rolled: 8 columns per lane, PCOLS/8 lanes per row
-        constexpr int LPR = PCOLS / 8, RPI = 64 / LPR;
-        const int rr = lane / LPR, c8 = (lane % LPR) * 8;
-        const int col = n0 + wn * WTN + ps * PCOLS + c8;
-        for (int it = 0; it < WTM / RPI; ++it) {
-            const int r = it * RPI + rr;
-            const int rt = wm * WTM + r;  // row inside the workgroup tile
-            const int u0 = (c8 >> 2) ^ (r & (UNITS - 1)), u1 = ((c8 >> 2) + 1) ^ (r & (UNITS - 1));
-            v4f lo = *reinterpret_cast<const v4f*>(stage_buf + r * (PCOLS * 4) + u0 * 16);
-            v4f hi = *reinterpret_cast<const v4f*>(stage_buf + r * (PCOLS * 4) + u1 * 16);
-            int dst;
-            if constexpr (GROUP == GROUP_DENSE) dst = rt < rows_valid ? m0 + rt : -1;
-            else dst = s_dst[rt];
-            if (dst < 0 || col >= p.N) continue;
-            if constexpr (SPLIT) {
-                store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, dst, col, p.N, lo, hi, 0.f, vec_ok);
-            } else {
-                float rs = scale;
-                if constexpr (GROUP == GROUP_GATHER) {
-                    if (p.row_weight) rs *= p.row_weight[dst];
-                }
-                store8(p.C, p.out_type, dst, col, p.N, lo * rs, hi * rs, p.beta, vec_ok);
+                if (dsts[tm] < 0 || col >= p.N) continue;
+                if constexpr (SPLIT)
+                    store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, dsts[tm], col, p.N, acc[2 * tp][tm], acc[2 * tp + 1][tm], 0.f, vec_ok);
+                else
+                    store8(p.C, OT, dsts[tm], col, p.N, acc[2 * tp][tm] * rws[tm], acc[2 * tp + 1][tm] * rws[tm], p.beta, vec_ok);
             }
         }
-    }
+    };
+    if (SPLIT || p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
+    else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
+    else emit(std::integral_constant<int, OUT_F16>{});
 
 #endif
 }
