@@ -365,7 +365,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     for (int i = 0; i < B_IT; ++i) {
         const int br = (i * NL + (wave % NL)) * 8 + lrow;  // slab row
         int n;
-        if constexpr (ACT) n = br < 128 ? n0 + br : p.inter + n0 + (br - 128);  // gate rows, then the up rows
+        // fused activation: wave column wn owns slab rows 128*wn .. +127 = 64 gate rows, then the 64 up rows of the same columns
+        if constexpr (ACT) n = ((br >> 6) & 1) * p.inter + n0 + (br >> 7) * 64 + (br & 63);
         else n = min(n0 + br, p.N - 1);
         b_off[i] = (uint32_t)n * (uint32_t)K + ljb * 16;
     }
@@ -451,12 +452,21 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         }
     };
     float sc[TM];
+    float sc_up[ACT ? TM : 1];  // fused activation: column tiles TN/2 .. TN-1 are up columns, with their own weight block
     auto read_scales = [&](int kstep, const float* cS) {
         if constexpr (BLOCKSCALE) {
-            const float bs = sBs[(wn * WTN) / 128][kstep];
+            const float bs = sBs[ACT ? 0 : (wn * WTN) / 128][kstep];
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) sc[tm] = cS[wm * WTM + tm * 16 + li] * bs;
+            for (int tm = 0; tm < TM; ++tm) {
+                const float as = cS[wm * WTM + tm * 16 + li];
+                sc[tm] = as * bs;
+                if constexpr (ACT) sc_up[tm] = as * sBs[1][kstep];
+            }
         }
+    };
+    auto scale_of = [&](int tn, int tm) -> float {
+        if constexpr (ACT) return tn >= TN / 2 ? sc_up[tm] : sc[tm];
+        else return sc[tm];
     };
     v8i af[TM];
     auto read_a = [&](const uint8_t* cA) {
@@ -489,11 +499,11 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
                 const int tn = j / TM, tm = j % TM;
                 part[j % 3] = mfma_e4m3(wf[tn & 1], af[tm], v4f{0.f, 0.f, 0.f, 0.f});
                 if (tm == 0 && tn + 1 < TN) read_w(tn + 1);
-                if (j >= 2) acc[(j - 2) / TM][(j - 2) % TM] += part[(j - 2) % 3] * sc[(j - 2) % TM];
+                if (j >= 2) acc[(j - 2) / TM][(j - 2) % TM] += part[(j - 2) % 3] * scale_of((j - 2) / TM, (j - 2) % TM);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int j = NJ - 2; j < NJ; ++j) acc[j / TM][j % TM] += part[j % 3] * sc[j % TM];
+            for (int j = NJ - 2; j < NJ; ++j) acc[j / TM][j % TM] += part[j % 3] * scale_of(j / TM, j % TM);
             // Pin the scale-and-add results here: without a use in this block the compiler sinks the
             // whole VALU chain behind the next conditional (a later K step's loader test), keeps every
             // 16x16 product alive until then and spills.  No instruction is emitted.
@@ -564,83 +574,81 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     __syncthreads();
 
     // ---------------------------------------------------------------- fused activation epilogue
-    // Wave (wm, 0) holds the tile's 128 gate columns of rows 64*wm .. 64*wm+63, wave (wm, 1) the
-    // matching up columns.  In four passes of 32 columns every wave stages its slice through LDS
-    // (fp32, 8 KiB per wave; the passes alternate between the A and the B slabs, so one barrier per
-    // pass suffices), then the two waves of a row group take 32 rows each, read gate and up of the
-    // same elements and compute, exactly as the stand-alone kernel does on the stored GEMM output:
+    // Wave (wm, wn) holds, for rows 64*wm .. +63, gate columns 64*wn .. +63 of the tile in column tiles
+    // 0..3 and the matching up columns in column tiles 4..7: a lane has gate and up of the same 16
+    // elements of each of its four rows in registers and computes, exactly as the stand-alone kernel
+    // does on the stored GEMM output,
     //   g = T(acc_gate), u = T(acc_up), act = T(g * sigmoid(g) * u)          (T = the 16-bit type)
-    // A row's 128 activations sit in 4 lanes x 4 passes; after the last pass the row maximum is
-    // reduced over those lanes, the scale (amax / 448, 1 for an all-zero group) is formed with an
-    // IEEE division and the codes are written 8 bytes per lane and pass.
+    // The maximum of a row's 128 activations (4 lanes x 2 waves) goes through two shuffles and one LDS
+    // exchange; then scale = amax / 448 (1 for an all-zero group), codes = e4m3(act / scale), written
+    // 8 bytes per lane and column-tile pair.
     if constexpr (ACT) {
-        constexpr int APC = 32, APASS = WTN / APC;  // staged columns per pass
-        float actv[APASS][2][8];
-        const int rsel = wn * 32;                   // this wave's half of the 64 rows
-        const int arr = lane >> 2, ac8 = (lane & 3) * 8;
+        float actv[TM][TN / 4][8];
+        float* const amax_mine = wn == 0 ? sS0 : sS1;  // the scale stages are idle now
+        // (one branch on the type around all 64 elements of the lane, so that their chains interleave)
+        auto activate = [&](auto type_tag) {
+            using T = decltype(type_tag);
 #pragma unroll
-        for (int ps = 0; ps < APASS; ++ps) {
-            uint8_t* const set_lo = (ps & 1) ? sB0 : sA0;  // waves 0..3 (gate), 4 x 8 KiB
-            uint8_t* const set_hi = (ps & 1) ? sB1 : sA1;  // waves 4..7 (up)
-            uint8_t* const mine = (wn == 0 ? set_lo : set_hi) + wm * (WTM * APC * 4);
+            for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-            for (int t = 0; t < APC / 16; ++t)
+                for (int tp = 0; tp < TN / 4; ++tp)
 #pragma unroll
-                for (int tm = 0; tm < TM; ++tm) {
-                    const int r = tm * 16 + li;
-                    const int u = (lg * 2 + t) ^ (r & 7);  // columns 8*lg + 4*t .. +3 of the pass
-                    *reinterpret_cast<v4f*>(mine + r * (APC * 4) + u * 16) = acc[ps * (APC / 16) + t][tm];
-                }
-            __syncthreads();
-            const uint8_t* gsrc = set_lo + wm * (WTM * APC * 4);
-            const uint8_t* usrc = set_hi + wm * (WTM * APC * 4);
+                    for (int q = 0; q < 8; ++q) {
+                        const float ga = acc[2 * tp + (q >> 2)][tm][q & 3], ua = acc[TN / 2 + 2 * tp + (q >> 2)][tm][q & 3];
+                        actv[tm][tp][q] = silu_mul_round<T>((float)(T)ga, (float)(T)ua);
+                    }
+        };
+        if (p.act_is_bf16) activate(__bf16{});
+        else activate(_Float16{});
 #pragma unroll
-            for (int it = 0; it < 2; ++it) {
-                const int r = rsel + it * 16 + arr;
-                const int u0 = (ac8 >> 2) ^ (r & 7), u1 = ((ac8 >> 2) + 1) ^ (r & 7);
-                const v4f g0 = *reinterpret_cast<const v4f*>(gsrc + r * (APC * 4) + u0 * 16);
-                const v4f g1 = *reinterpret_cast<const v4f*>(gsrc + r * (APC * 4) + u1 * 16);
-                const v4f p0 = *reinterpret_cast<const v4f*>(usrc + r * (APC * 4) + u0 * 16);
-                const v4f p1 = *reinterpret_cast<const v4f*>(usrc + r * (APC * 4) + u1 * 16);
+        for (int tm = 0; tm < TM; ++tm) {
+            float amax = 0.f;
 #pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    const float ga = q < 4 ? g0[q & 3] : g1[q & 3], ua = q < 4 ? p0[q & 3] : p1[q & 3];
-                    if (p.act_is_bf16) actv[ps][it][q] = silu_mul_round<__bf16>((float)(__bf16)ga, (float)(__bf16)ua);
-                    else actv[ps][it][q] = silu_mul_round<_Float16>((float)(_Float16)ga, (float)(_Float16)ua);
-                }
-            }
+            for (int tp = 0; tp < TN / 4; ++tp)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) amax = fmaxf(amax, fabsf(actv[tm][tp][q]));
+            amax = fmaxf(amax, __shfl_xor(amax, 16));
+            amax = fmaxf(amax, __shfl_xor(amax, 32));
+            if (lg == 0) amax_mine[wm * WTM + tm * 16 + li] = amax;
         }
+        __syncthreads();
         uint8_t* const qout = reinterpret_cast<uint8_t*>(p.C);
         const int groups_per_row = p.inter / 128;
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            float amax = 0.f;
-#pragma unroll
-            for (int ps = 0; ps < APASS; ++ps)
-#pragma unroll
-                for (int q = 0; q < 8; ++q) amax = fmaxf(amax, fabsf(actv[ps][it][q]));
-            amax = fmaxf(amax, __shfl_xor(amax, 1));
-            amax = fmaxf(amax, __shfl_xor(amax, 2));
+        for (int tm = 0; tm < TM; ++tm) {
+            const int rt = wm * WTM + tm * 16 + li;
+            const float amax = fmaxf(sS0[rt], sS1[rt]);
             const float sc1 = amax == 0.f ? 1.0f : amax / 448.0f;
-            const int rt = wm * WTM + rsel + it * 16 + arr;
             const int dst = s_dst[rt];
             if (dst < 0) continue;
+            const ScaleDivider div(sc1);
+            if (div.fast) {
 #pragma unroll
-            for (int ps = 0; ps < APASS; ++ps) {
+                for (int tp = 0; tp < TN / 4; ++tp)
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) actv[tm][tp][q] = div.quotient(actv[tm][tp][q]);
+            } else {
+#pragma unroll
+                for (int tp = 0; tp < TN / 4; ++tp)
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) actv[tm][tp][q] = actv[tm][tp][q] / sc1;
+            }
+#pragma unroll
+            for (int tp = 0; tp < TN / 4; ++tp) {
                 int packed[2];
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     float c[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) c[i] = fminf(fmaxf(actv[ps][it][4 * h + i] / sc1, -448.0f), 448.0f);
+                    for (int i = 0; i < 4; ++i) c[i] = fminf(fmaxf(actv[tm][tp][4 * h + i], -448.0f), 448.0f);
                     int w = 0;
                     w = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], w, false);
                     w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
                     packed[h] = w;
                 }
-                *reinterpret_cast<v2i*>(qout + (int64_t)dst * p.inter + n0 + ps * APC + ac8) = v2i{packed[0], packed[1]};
+                *reinterpret_cast<v2i*>(qout + (int64_t)dst * p.inter + n0 + wn * 64 + tp * 32 + lg * 8) = v2i{packed[0], packed[1]};
             }
-            if ((lane & 3) == 0) p.act_scales[(int64_t)dst * groups_per_row + tile_n] = sc1;
+            if (wn == 0 && lg == 0) p.act_scales[(int64_t)dst * groups_per_row + tile_n] = sc1;
         }
         return;
     }

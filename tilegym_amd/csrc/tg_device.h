@@ -164,8 +164,32 @@ template <typename T>
 __device__ __forceinline__ float silu_mul_round(float gate, float up) {
     const float sl = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate));
     float prod = sl * up;
-    asm volatile("" : "+v"(prod));
+    asm("" : "+v"(prod));  // not volatile: the pins of different elements need no order among themselves
     return (float)(T)prod;
 }
+
+// a / s for many a and one s, bit-equal to the IEEE division `a / s`.  For a divisor well inside the
+// exponent range this is the compiler's own expansion of a float division without the operand
+// pre-scaling and the special-case fix-up, which only act on extreme exponents (reciprocal estimate,
+// one Newton step, then two residual corrections of the quotient; the reciprocal is shared by all
+// numerators).  Where the pre-scaling would act on a tiny quotient (|a / s| < 2^-90) the result may
+// differ in its last bits; every caller rounds the quotient to e4m3, where all such values are zero
+// of the same sign.  For other divisors (zero, subnormal, huge, inf, nan) `fast` is false and the caller
+// divides plainly; the test is per divisor so that a caller branches once for all its numerators.
+struct ScaleDivider {
+    float s, r;
+    bool fast;
+    __device__ __forceinline__ explicit ScaleDivider(float scale) : s(scale) {
+        fast = scale >= 0x1p-100f && scale <= 0x1p100f;
+        const float r0 = __builtin_amdgcn_rcpf(scale);
+        r = __builtin_fmaf(__builtin_fmaf(-scale, r0, 1.0f), r0, r0);
+    }
+    // valid while `fast` holds; a zero numerator keeps its sign as in the plain division
+    __device__ __forceinline__ float quotient(float a) const {
+        const float q0 = a * r;
+        const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, a), r, q0);
+        return __builtin_copysignf(__builtin_fmaf(__builtin_fmaf(-s, q1, a), r, q1), a);
+    }
+};
 
 }  // namespace tg
