@@ -384,7 +384,12 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     const uint32_t wfrag0 = wrow * kKBlock + ((lg ^ swz_w(wrow)) << 4);
     const uint32_t wfrag1 = wfrag0 ^ 64;
     auto w_tile_row = [](int tn) { return (tn >> 1) * 32 + (tn & 1) * 4; };
-    const uint32_t a_frag_base = wm * WTM * kKBlock, b_frag_base = wn * WTN * kKBlock;
+    // Rows: wave row wm owns the 16-row groups wm, wm + WGM, wm + 2*WGM, ... of the tile (not a contiguous
+    // block of rows), so that a tile whose valid rows are a prefix -- the last row tile of an expert or
+    // of the problem -- spreads them evenly over the waves and every wave can skip the same share of
+    // its MFMAs (see `n_tm` below).
+    auto tile_row = [&](int tm) { return (tm * WGM + wm) * 16; };
+    const uint32_t a_frag_base = wm * 16 * kKBlock, b_frag_base = wn * WTN * kKBlock;
 
     // block scales: the activation scales of a K step travel with its slabs (one 4-byte direct
     // load per slab row into sS0/sS1, issued by the first BM/64 loader waves), the weight scale
@@ -453,12 +458,13 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     };
     float sc[TM];
     float sc_up[ACT ? TM : 1];  // fused activation: column tiles TN/2 .. TN-1 are up columns, with their own weight block
-    auto read_scales = [&](int kstep, const float* cS) {
-        if constexpr (BLOCKSCALE) {
+    auto read_scales = [&](auto ntm_tag, int kstep, const float* cS) {
+        constexpr int NTM = decltype(ntm_tag)::value;
+        if constexpr (BLOCKSCALE && NTM > 0) {
             const float bs = sBs[ACT ? 0 : (wn * WTN) / 128][kstep];
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) {
-                const float as = cS[wm * WTM + tm * 16 + li];
+            for (int tm = 0; tm < NTM; ++tm) {
+                const float as = cS[tile_row(tm) + li];
                 sc[tm] = as * bs;
                 if constexpr (ACT) sc_up[tm] = as * sBs[1][kstep];
             }
@@ -469,16 +475,20 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         else return sc[tm];
     };
     v8i af[TM];
-    auto read_a = [&](const uint8_t* cA) {
+    auto read_a = [&](auto ntm_tag, const uint8_t* cA) {
+        constexpr int NTM = decltype(ntm_tag)::value;
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
-            const uint8_t* base = cA + a_frag_base + tm * 16 * kKBlock;
+        for (int tm = 0; tm < NTM; ++tm) {
+            const uint8_t* base = cA + a_frag_base + tm * (WGM * 16 * kKBlock);
             af[tm] = join(*reinterpret_cast<const v4i*>(base + frag0),
                           *reinterpret_cast<const v4i*>(base + frag1));
         }
     };
-    auto mma = [&](const uint8_t* cB) {
-        if constexpr (BLOCKSCALE) {
+    auto mma = [&](auto ntm_tag, const uint8_t* cB) {
+        constexpr int NTM = decltype(ntm_tag)::value;  // this wave's row groups that hold valid rows
+        if constexpr (NTM == 0) {
+            return;
+        } else if constexpr (BLOCKSCALE) {
             // One MFMA (into a zeroed 16x16 product), then the four scale-and-add operations of the
             // product issued two MFMAs earlier: the matrix pipe works on the MFMA for 32 clocks while
             // the wave issues 16 clocks of VALU work behind it, and a product is complete (two MFMA
@@ -486,7 +496,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
             // every such pair keeps the compiler from collecting the VALU work behind the last MFMA
             // (where the matrix pipe would idle); the weight fragment of column tile tn+1 is fetched
             // during column tile tn.
-            constexpr int NJ = TN * TM;
+            constexpr int NJ = TN * NTM;
             v4f part[3];
             v8i wf[2];
             auto read_w = [&](int tn) {
@@ -496,21 +506,21 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
             read_w(0);
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
-                const int tn = j / TM, tm = j % TM;
+                const int tn = j / NTM, tm = j % NTM;
                 part[j % 3] = mfma_e4m3(wf[tn & 1], af[tm], v4f{0.f, 0.f, 0.f, 0.f});
                 if (tm == 0 && tn + 1 < TN) read_w(tn + 1);
-                if (j >= 2) acc[(j - 2) / TM][(j - 2) % TM] += part[(j - 2) % 3] * scale_of((j - 2) / TM, (j - 2) % TM);
+                if (j >= 2) acc[(j - 2) / NTM][(j - 2) % NTM] += part[(j - 2) % 3] * scale_of((j - 2) / NTM, (j - 2) % NTM);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int j = NJ - 2; j < NJ; ++j) acc[j / TM][j % TM] += part[j % 3] * scale_of(j / TM, j % TM);
+            for (int j = NJ - 2; j < NJ; ++j) acc[j / NTM][j % NTM] += part[j % 3] * scale_of(j / NTM, j % NTM);
             // Pin the scale-and-add results here: without a use in this block the compiler sinks the
             // whole VALU chain behind the next conditional (a later K step's loader test), keeps every
             // 16x16 product alive until then and spills.  No instruction is emitted.
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-                for (int tm = 0; tm < TM; ++tm) asm volatile("" : "+v"(acc[tn][tm]));
+                for (int tm = 0; tm < NTM; ++tm) asm volatile("" : "+v"(acc[tn][tm]));
         } else {
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
@@ -518,7 +528,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
                 const v8i wf = join(*reinterpret_cast<const v4i*>(base + wfrag0),
                                     *reinterpret_cast<const v4i*>(base + wfrag1));
 #pragma unroll
-                for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
+                for (int tm = 0; tm < NTM; ++tm) acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
             }
         }
     };
@@ -552,29 +562,52 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     issue_a(min(ks + 1, last), sA1);
     __builtin_amdgcn_s_waitcnt(kWaitAllButA);  // a wave without loads in flight passes at once
     lds_barrier();
-    auto step = [&](int k, uint8_t* cA, uint8_t* cB, float* cS, uint8_t* oB, float* oS) {
-        issue_b(min(k + 1, last), oB);
-        issue_s(min(k + 1, last), oS);
-        read_a(cA);
-        read_scales(k, cS);
-        lds_barrier();
-        issue_a(min(k + 2, last), cA);
-        mma(cB);
-        if constexpr (!BLOCKSCALE) pipeline_hint<TM, TN, A_IT>();
-        __builtin_amdgcn_s_waitcnt(kWaitAllButA);
-        lds_barrier();
+    // The loop exists once per number of row groups a wave may have to compute (NTM = 0 .. TM): the
+    // waves of a workgroup can run different copies, every copy issues the same loads and barriers.
+    auto k_loop = [&](auto ntm_tag) {
+        constexpr int NTM = decltype(ntm_tag)::value;
+        auto step = [&](int k, uint8_t* cA, uint8_t* cB, float* cS, uint8_t* oB, float* oS) {
+            issue_b(min(k + 1, last), oB);
+            issue_s(min(k + 1, last), oS);
+            read_a(ntm_tag, cA);
+            read_scales(ntm_tag, k, cS);
+            lds_barrier();
+            issue_a(min(k + 2, last), cA);
+            mma(ntm_tag, cB);
+            if constexpr (!BLOCKSCALE && NTM > 0) pipeline_hint<NTM, TN, A_IT>();
+            __builtin_amdgcn_s_waitcnt(kWaitAllButA);
+            lds_barrier();
+        };
+        int i = 0;
+        for (; i + 1 < nsteps; i += 2) {
+            step(ks + i, sA0, sB0, sS0, sB1, sS1);
+            step(ks + i + 1, sA1, sB1, sS1, sB0, sS0);
+        }
+        if (i < nsteps) step(ks + i, sA0, sB0, sS0, sB1, sS1);
     };
-    int i = 0;
-    for (; i + 1 < nsteps; i += 2) {
-        step(ks + i, sA0, sB0, sS0, sB1, sS1);
-        step(ks + i + 1, sA1, sB1, sS1, sB0, sS0);
+    // Row groups of this wave that hold at least one valid row, counted up to the last such group (the
+    // valid rows of a tile are a prefix wherever the row maps come from this library's own alignment;
+    // any other map only costs the skipped work).  Dense problems skip nothing: one copy of the loop.
+    if constexpr (GROUP == GROUP_DENSE) {
+        k_loop(std::integral_constant<int, TM>{});
+    } else {
+        static_assert(TM == 4, "dispatch below");
+        int n_tm = 0;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+            if (__ballot(s_dst[tile_row(tm) + li] >= 0) != 0) n_tm = tm + 1;
+        n_tm = __builtin_amdgcn_readfirstlane(n_tm);
+        if (n_tm == 4) k_loop(std::integral_constant<int, 4>{});
+        else if (n_tm == 3) k_loop(std::integral_constant<int, 3>{});
+        else if (n_tm == 2) k_loop(std::integral_constant<int, 2>{});
+        else if (n_tm == 1) k_loop(std::integral_constant<int, 1>{});
+        else k_loop(std::integral_constant<int, 0>{});
     }
-    if (i < nsteps) step(ks + i, sA0, sB0, sS0, sB1, sS1);
     __builtin_amdgcn_s_waitcnt(kWaitAll);
     __syncthreads();
 
     // ---------------------------------------------------------------- fused activation epilogue
-    // Wave (wm, wn) holds, for rows 64*wm .. +63, gate columns 64*wn .. +63 of the tile in column tiles
+    // Wave (wm, wn) holds, for its four 16-row groups, gate columns 64*wn .. +63 of the tile in column tiles
     // 0..3 and the matching up columns in column tiles 4..7: a lane has gate and up of the same 16
     // elements of each of its four rows in registers and computes, exactly as the stand-alone kernel
     // does on the stored GEMM output,
@@ -609,14 +642,14 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
                 for (int q = 0; q < 8; ++q) amax = fmaxf(amax, fabsf(actv[tm][tp][q]));
             amax = fmaxf(amax, __shfl_xor(amax, 16));
             amax = fmaxf(amax, __shfl_xor(amax, 32));
-            if (lg == 0) amax_mine[wm * WTM + tm * 16 + li] = amax;
+            if (lg == 0) amax_mine[tile_row(tm) + li] = amax;
         }
         __syncthreads();
         uint8_t* const qout = reinterpret_cast<uint8_t*>(p.C);
         const int groups_per_row = p.inter / 128;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
-            const int rt = wm * WTM + tm * 16 + li;
+            const int rt = tile_row(tm) + li;
             const float amax = fmaxf(sS0[rt], sS1[rt]);
             const float sc1 = amax == 0.f ? 1.0f : amax / 448.0f;
             const int dst = s_dst[rt];
@@ -668,7 +701,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     float rws[TM];
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
-        const int rt = wm * WTM + tm * 16 + li;  // row inside the workgroup tile
+        const int rt = tile_row(tm) + li;  // row inside the workgroup tile
         if constexpr (GROUP == GROUP_DENSE) dsts[tm] = rt < rows_valid ? m0 + rt : -1;
         else dsts[tm] = s_dst[rt];
         rws[tm] = scale;
