@@ -709,11 +709,12 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     }
     auto emit = [&](auto type_tag) {
         constexpr int OT = decltype(type_tag)::value;
+        // (row group outermost: the two 64-byte halves of an output line are written back to back)
 #pragma unroll
-        for (int tp = 0; tp < TN / 2; ++tp) {
-            const int col = n0 + wn * WTN + tp * 32 + lg * 8;
+        for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm) {
+            for (int tp = 0; tp < TN / 2; ++tp) {
+                const int col = n0 + wn * WTN + tp * 32 + lg * 8;
                 if (dsts[tm] < 0 || col >= p.N) continue;
                 if constexpr (SPLIT)
                     store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, dsts[tm], col, p.N, acc[2 * tp][tm], acc[2 * tp + 1][tm], 0.f, vec_ok);
