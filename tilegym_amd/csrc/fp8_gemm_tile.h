@@ -259,8 +259,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     __shared__ float sBs[BLOCKSCALE ? (BN + 127) / 128 : 1][BLOCKSCALE ? kMaxKBlocks : 1];
     __shared__ int s_src[GROUP == GROUP_DENSE ? 1 : BM];
     __shared__ int s_dst[GROUP == GROUP_DENSE ? 1 : BM];
-    // routed weight of each tile row (gather GEMM with mul_routed_weight), fetched once with the row
-    // maps: a load inside the epilogue's row loop would put a global-memory latency on every iteration
+    // routed weight of each tile row (gather GEMM with mul_routed_weight), fetched once per tile: a load
+    // inside the epilogue's row loop would put a global-memory latency on every iteration
     __shared__ float s_w[GROUP == GROUP_GATHER ? BM : 1];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -319,48 +319,22 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     }
     const int n0 = ACT ? tile_n * 128 : tile_n * BN;  // ACT: first gate column of the tile
 
-    if constexpr (GROUP != GROUP_DENSE) {
-        for (int r = tid; r < BM; r += NT) {
-            int src, dst;
-            if constexpr (GROUP == GROUP_RAGGED) {
-                src = m0 + min(r, rows_valid - 1);
-                dst = r < rows_valid ? m0 + r : -1;
-            } else {
-                const int idx = m0 + r;
-                const int id = idx < post_pad ? p.sorted_ids[idx] : p.num_valid;
-                const bool ok = id >= 0 && id < p.num_valid;
-                src = ok ? id / p.top_k : 0;
-                dst = ok ? id : -1;
-            }
-            s_src[r] = src;
-            s_dst[r] = dst;
-            if constexpr (GROUP == GROUP_GATHER) s_w[r] = (p.row_weight && dst >= 0) ? p.row_weight[dst] : 1.0f;
-        }
-        __syncthreads();
+    int ks = 0, ks_end = p.kblocks;
+    if constexpr (SPLIT) {
+        ks = blockIdx.y * p.ksteps_per_split;
+        ks_end = min(ks + p.ksteps_per_split, p.kblocks);
     }
 
-    // ---------------------------------------------------------------- loader set-up
-    // The first NL waves of the workgroup issue every direct load (one loader per SIMD when there
-    // are two waves per SIMD: while a loader waits for room in the memory pipeline, the other
-    // wave of its SIMD keeps the matrix pipe fed).  Pass i of loader w fills the 8-row group
-    // g = i*NL + w: lane l lands at row 8g + l/8, chunk position l%8, and therefore fetches
-    // logical chunk (l%8) ^ swz16(row) = (l%8) ^ (l/8).
+    // ---------------------------------------------------------------- weight slab of the first K step
+    // Requested before anything else: it needs only the tile's column and expert, so its trip to memory
+    // overlaps the row maps and scale tables fetched below (which the activation loads must wait for).
     const int lrow = lane >> 3;
-    const int lj = (lane & 7) ^ swz16(lrow);
     // weight slab: its own swizzle (see the fragment addresses below).  Row 8g + lrow with g = i*NL + wave:
     // NL is even, so bit 3 of the row is the parity of the loader wave.
     const int ljb = (lane & 7) ^ swz_w(((wave & 1) << 3) | lrow);
     // (with NL == NW every wave loads: no test, and so no branch inside the K loop)
     const bool loader = NL == NW || wave < NL;
-    uint32_t a_off[A_IT], b_off[B_IT];
-#pragma unroll
-    for (int i = 0; i < A_IT; ++i) {
-        const int r = (i * NL + (wave % NL)) * 8 + lrow;
-        int src;
-        if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
-        else src = s_src[r];
-        a_off[i] = (uint32_t)src * (uint32_t)K + lj * 16;
-    }
+    uint32_t b_off[B_IT];
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
         const int br = (i * NL + (wave % NL)) * 8 + lrow;  // slab row
@@ -369,6 +343,75 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         if constexpr (ACT) n = ((br >> 6) & 1) * p.inter + n0 + (br >> 7) * 64 + (br & 63);
         else n = min(n0 + br, p.N - 1);
         b_off[i] = (uint32_t)n * (uint32_t)K + ljb * 16;
+    }
+    const v4i rsrc_b = make_rsrc(Bbase);
+    auto issue_b = [&](int kstep, uint8_t* dB) {
+        if (!loader) return;
+        const int k0 = kstep * kKBlock;
+        const uint32_t dst = lds_address(dB) + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) {
+            // the 64-row tile serves M <= 64: one row tile, every weight byte is read once
+            if constexpr (BM == 64) direct_load_b128_nt(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
+            else direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
+        }
+    };
+    issue_b(ks, sB0);
+
+    // ---------------------------------------------------------------- row maps and scale tables
+    // Both come from global memory; the slot ids are requested first and used last, so that the two
+    // round trips (and the weight slab's) overlap.  One barrier publishes all of it.
+    static_assert(BM <= NT, "one tile row per thread");
+    int slot_id = 0;
+    if constexpr (GROUP == GROUP_GATHER || GROUP == GROUP_GATHER_ACT) {
+        const int idx = m0 + tid;
+        slot_id = (tid < BM && idx < post_pad) ? p.sorted_ids[idx] : p.num_valid;
+    }
+    if constexpr (BLOCKSCALE) {
+        // weight block scales of this tile's column blocks for every K step
+        constexpr int NBT = (BN + 127) / 128;
+        for (int idx = tid; idx < NBT * p.kblocks; idx += NT) {
+            const int j = idx / p.kblocks, kb = idx % p.kblocks;
+            const int nb = ACT ? (j == 0 ? n0 / 128 : (p.inter + n0) / 128) : min(n0 / 128 + j, p.nblocks - 1);
+            sBs[j][kb] = Bsbase ? Bsbase[(int64_t)nb * p.kblocks + kb] : 1.0f;
+        }
+        if (!p.As) {  // no activation scales: ones
+            for (int r2 = tid; r2 < BM; r2 += NT) sS0[r2] = sS1[r2] = 1.0f;
+        }
+    }
+    if constexpr (GROUP != GROUP_DENSE) {
+        if (tid < BM) {
+            const int r = tid;
+            int src, dst;
+            if constexpr (GROUP == GROUP_RAGGED) {
+                src = m0 + min(r, rows_valid - 1);
+                dst = r < rows_valid ? m0 + r : -1;
+            } else {
+                const bool ok = slot_id >= 0 && slot_id < p.num_valid;
+                src = ok ? slot_id / p.top_k : 0;
+                dst = ok ? slot_id : -1;
+            }
+            s_src[r] = src;
+            s_dst[r] = dst;
+        }
+    }
+    if constexpr (BLOCKSCALE || GROUP != GROUP_DENSE) __syncthreads();
+
+    // ---------------------------------------------------------------- loader set-up
+    // The first NL waves of the workgroup issue every direct load (one loader per SIMD when there
+    // are two waves per SIMD: while a loader waits for room in the memory pipeline, the other
+    // wave of its SIMD keeps the matrix pipe fed).  Pass i of loader w fills the 8-row group
+    // g = i*NL + w: lane l lands at row 8g + l/8, chunk position l%8, and therefore fetches
+    // logical chunk (l%8) ^ swz16(row) = (l%8) ^ (l/8).
+    const int lj = (lane & 7) ^ swz16(lrow);
+    uint32_t a_off[A_IT];
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+        const int r = (i * NL + (wave % NL)) * 8 + lrow;
+        int src;
+        if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
+        else src = s_src[r];
+        a_off[i] = (uint32_t)src * (uint32_t)K + lj * 16;
     }
 
     const int li = lane & 15, lg = lane >> 4;
@@ -398,27 +441,11 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     constexpr int S_WAVES = (BM + 63) / 64;
     static_assert(!BLOCKSCALE || S_WAVES <= NL, "scale rows are fetched by the loader waves");
     if constexpr (BLOCKSCALE) {
-        constexpr int NBT = (BN + 127) / 128;
-        for (int idx = tid; idx < NBT * p.kblocks; idx += NT) {
-            const int j = idx / p.kblocks, kb = idx % p.kblocks;
-            const int nb = ACT ? (j == 0 ? n0 / 128 : (p.inter + n0) / 128) : min(n0 / 128 + j, p.nblocks - 1);
-            sBs[j][kb] = Bsbase ? Bsbase[(int64_t)nb * p.kblocks + kb] : 1.0f;
-        }
         const int r = min(wave * 64 + lane, BM - 1);
         int src;
         if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
         else src = s_src[r];
         s_off = (uint32_t)src * (uint32_t)p.kblocks * 4u;
-        if (!p.As) {  // no activation scales: ones
-            for (int r2 = tid; r2 < BM; r2 += NT) sS0[r2] = sS1[r2] = 1.0f;
-        }
-        __syncthreads();
-    }
-
-    int ks = 0, ks_end = p.kblocks;
-    if constexpr (SPLIT) {
-        ks = blockIdx.y * p.ksteps_per_split;
-        ks_end = min(ks + p.ksteps_per_split, p.kblocks);
     }
 
     v4f acc[TN][TM];
@@ -430,24 +457,13 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // Direct global->LDS loads of one K step, as buffer loads: 32-bit per-lane offset + scalar
     // K offset, no 64-bit address arithmetic in the loop.  K is a multiple of 128 here (the host
     // sends other K to the fallback kernel), so every lane's 16 bytes are in range.
-    const v4i rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(Bbase);
+    const v4i rsrc_a = make_rsrc(p.A);
     auto issue_a = [&](int kstep, uint8_t* dA) {
         if (!loader) return;
         const int k0 = kstep * kKBlock;
         const uint32_t dst = lds_address(dA) + wave * 1024;
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) direct_load_b128(rsrc_a, dst + i * NL * 1024, a_off[i], k0);
-    };
-    auto issue_b = [&](int kstep, uint8_t* dB) {
-        if (!loader) return;
-        const int k0 = kstep * kKBlock;
-        const uint32_t dst = lds_address(dB) + wave * 1024;
-#pragma unroll
-        for (int i = 0; i < B_IT; ++i) {
-            // the 64-row tile serves M <= 64: one row tile, every weight byte is read once
-            if constexpr (BM == 64) direct_load_b128_nt(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
-            else direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
-        }
     };
     const v4i rsrc_s = make_rsrc(p.As);
     auto issue_s = [&](int kstep, float* dS) {
@@ -556,8 +572,16 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // Steps past the end are clamped to the last step: they re-fetch it into an idle slab, which
     // keeps the loop body free of branches.
     const int nsteps = ks_end - ks, last = ks_end - 1;
-    issue_a(ks, sA0);
-    issue_b(ks, sB0);
+    // Routed weight of each tile row (thread t holds row t's): needed by the epilogue only, so it is
+    // requested now, rides through the K loop in a register and goes to LDS after the loop.
+    float row_w = 1.0f;
+    if constexpr (GROUP == GROUP_GATHER) {
+        if (tid < BM && p.row_weight) {
+            const int dst = s_dst[tid];
+            if (dst >= 0) row_w = p.row_weight[dst];
+        }
+    }
+    issue_a(ks, sA0);  // (the weight slab of this step is in flight since the top of the kernel)
     issue_s(ks, sS0);
     issue_a(min(ks + 1, last), sA1);
     __builtin_amdgcn_s_waitcnt(kWaitAllButA);  // a wave without loads in flight passes at once
@@ -604,6 +628,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         else k_loop(std::integral_constant<int, 0>{});
     }
     __builtin_amdgcn_s_waitcnt(kWaitAll);
+    if constexpr (GROUP == GROUP_GATHER) {
+        if (tid < BM) s_w[tid] = row_w;
+    }
     __syncthreads();
 
     // ---------------------------------------------------------------- fused activation epilogue
