@@ -88,6 +88,7 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 // conflict free with this XOR (8 clocks per 1 KiB wave-read, the LDS's full rate); additive
 // variants are 2-way conflicted.
 __device__ __forceinline__ int swz16(int r) { return r & 7; }
+constexpr int kScaleChunk = 8;  // K steps per chunk of the activation-scale table
 // chunk swizzle of the weight slab: row bits 0, 1 and 3
 __device__ __forceinline__ int swz_w(int r) { return (r & 3) | ((r >> 1) & 4); }
 
@@ -253,8 +254,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     __shared__ __align__(1024) uint8_t sB0[BN * kKBlock];
     __shared__ __align__(1024) uint8_t sB1[BN * kKBlock];
     // per-stage activation scales of the slab rows (block-scaled kernels only)
-    __shared__ __align__(256) float sS0[BLOCKSCALE ? BM : 1];
-    __shared__ __align__(256) float sS1[BLOCKSCALE ? BM : 1];
+    __shared__ __align__(256) float sTab[BLOCKSCALE ? 2 * BM * kScaleChunk : 1];
     // weight block scales of this tile's column blocks for every K step (fetched once)
     __shared__ float sBs[BLOCKSCALE ? (BN + 127) / 128 : 1][BLOCKSCALE ? kMaxKBlocks : 1];
     __shared__ int s_src[GROUP == GROUP_DENSE ? 1 : BM];
@@ -376,7 +376,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
             sBs[j][kb] = Bsbase ? Bsbase[(int64_t)nb * p.kblocks + kb] : 1.0f;
         }
         if (!p.As) {  // no activation scales: ones
-            for (int r2 = tid; r2 < BM; r2 += NT) sS0[r2] = sS1[r2] = 1.0f;
+            for (int r2 = tid; r2 < 2 * BM * kScaleChunk; r2 += NT) sTab[r2] = 1.0f;
         }
     }
     if constexpr (GROUP != GROUP_DENSE) {
@@ -434,20 +434,19 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     auto tile_row = [&](int tm) { return (tm * WGM + wm) * 16; };
     const uint32_t a_frag_base = wm * 16 * kKBlock, b_frag_base = wn * WTN * kKBlock;
 
-    // block scales: the activation scales of a K step travel with its slabs (one 4-byte direct
-    // load per slab row into sS0/sS1, issued by the first BM/64 loader waves), the weight scale
-    // is one scalar per wave and K step.
-    uint32_t s_off = 0;
-    constexpr int S_WAVES = (BM + 63) / 64;
-    static_assert(!BLOCKSCALE || S_WAVES <= NL, "scale rows are fetched by the loader waves");
-    if constexpr (BLOCKSCALE) {
-        const int r = min(wave * 64 + lane, BM - 1);
-        int src;
-        if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
-        else src = s_src[r];
-        s_off = (uint32_t)src * (uint32_t)p.kblocks * 4u;
-    }
-
+    // Block scales.  The weight scale is one scalar per wave and K step (table sBs).  The activation
+    // scales (one per tile row and K step) come in chunks of kScaleChunk = 8 K steps through a
+    // double-buffered LDS table: one 4-byte direct load covers 8 rows x 8 consecutive K steps, i.e. 8
+    // runs of 32 contiguous bytes -- fetching one K step for 64 rows would touch 64 cache lines per
+    // instruction, eight times what a slab load does.  Chunk c+1 is requested while chunk c is in use,
+    // one 8-row group per loader wave and K step.  Lane l of the load for row group g lands at float
+    // 64*g + l of the chunk's buffer; it fetches row 8g + l/8 at chunk step (l%8 - l/8) % 8, so step s of
+    // row r sits at position (s + r) % 8 of the row's eight floats and the 16 rows a fragment's lanes
+    // read in one K step spread over the banks.
+    constexpr int S_GROUPS = BM / 8;                     // 8-row groups of the tile
+    constexpr int S_PHASES = (S_GROUPS + NL - 1) / NL;   // K steps a chunk's loads are spread over
+    static_assert(S_PHASES <= kScaleChunk, "a chunk is fetched within the chunk before it");
+    const int s_kbi = ((lane & 7) - (lane >> 3)) & 7;    // chunk step this lane fetches
     v4f acc[TN][TM];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
@@ -466,21 +465,34 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         for (int i = 0; i < A_IT; ++i) direct_load_b128(rsrc_a, dst + i * NL * 1024, a_off[i], k0);
     };
     const v4i rsrc_s = make_rsrc(p.As);
-    auto issue_s = [&](int kstep, float* dS) {
+    // direct load of row group ph*NL + wave of chunk `chunk` (K steps ks + 8*chunk ..), if this wave has one
+    auto issue_s = [&](int chunk, int ph) {
         if constexpr (BLOCKSCALE) {
-            if (p.As && wave < S_WAVES && (BM >= 64 || lane < BM))
-                direct_load_b32(rsrc_s, lds_address(dS) + wave * 256, s_off, kstep * 4);
+            const int g = ph * NL + wave;
+            if (p.As && loader && g < S_GROUPS) {
+                const int r = g * 8 + (lane >> 3);
+                int src;
+                if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
+                else src = s_src[r];
+                const int kb = min(ks + chunk * kScaleChunk + s_kbi, p.kblocks - 1);
+                const uint32_t off = ((uint32_t)src * (uint32_t)p.kblocks + (uint32_t)kb) * 4u;
+                direct_load_b32(rsrc_s, lds_address(sTab) + ((chunk & 1) * BM * kScaleChunk + g * 64) * 4, off, 0);
+            }
         }
     };
     float sc[TM];
     float sc_up[ACT ? TM : 1];  // fused activation: column tiles TN/2 .. TN-1 are up columns, with their own weight block
-    auto read_scales = [&](auto ntm_tag, int kstep, const float* cS) {
+    // position of row tile_row(0) + li in a chunk buffer, without the step rotation (see above)
+    const int s_rbase = (wm * 2 + (li >> 3)) * 64 + (li & 7) * 8;
+    auto read_scales = [&](auto ntm_tag, int kstep) {
         constexpr int NTM = decltype(ntm_tag)::value;
         if constexpr (BLOCKSCALE && NTM > 0) {
+            const int kk = kstep - ks;
+            const float* cS = sTab + ((kk / kScaleChunk) & 1) * (BM * kScaleChunk) + s_rbase + (((kk % kScaleChunk) + li) & 7);
             const float bs = sBs[ACT ? 0 : (wn * WTN) / 128][kstep];
 #pragma unroll
             for (int tm = 0; tm < NTM; ++tm) {
-                const float as = cS[tile_row(tm) + li];
+                const float as = cS[tm * (WGM * 128)];
                 sc[tm] = as * bs;
                 if constexpr (ACT) sc_up[tm] = as * sBs[1][kstep];
             }
@@ -582,7 +594,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         }
     }
     issue_a(ks, sA0);  // (the weight slab of this step is in flight since the top of the kernel)
-    issue_s(ks, sS0);
+#pragma unroll
+    for (int ph = 0; ph < S_PHASES; ++ph) issue_s(0, ph);
     issue_a(min(ks + 1, last), sA1);
     __builtin_amdgcn_s_waitcnt(kWaitAllButA);  // a wave without loads in flight passes at once
     lds_barrier();
@@ -590,11 +603,11 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // waves of a workgroup can run different copies, every copy issues the same loads and barriers.
     auto k_loop = [&](auto ntm_tag) {
         constexpr int NTM = decltype(ntm_tag)::value;
-        auto step = [&](int k, uint8_t* cA, uint8_t* cB, float* cS, uint8_t* oB, float* oS) {
+        auto step = [&](int k, uint8_t* cA, uint8_t* cB, uint8_t* oB) {
             issue_b(min(k + 1, last), oB);
-            issue_s(min(k + 1, last), oS);
+            issue_s((k - ks) / kScaleChunk + 1, (k - ks) % kScaleChunk);
             read_a(ntm_tag, cA);
-            read_scales(ntm_tag, k, cS);
+            read_scales(ntm_tag, k);
             lds_barrier();
             issue_a(min(k + 2, last), cA);
             mma(ntm_tag, cB);
@@ -604,10 +617,10 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         };
         int i = 0;
         for (; i + 1 < nsteps; i += 2) {
-            step(ks + i, sA0, sB0, sS0, sB1, sS1);
-            step(ks + i + 1, sA1, sB1, sS1, sB0, sS0);
+            step(ks + i, sA0, sB0, sB1);
+            step(ks + i + 1, sA1, sB1, sB0);
         }
-        if (i < nsteps) step(ks + i, sA0, sB0, sS0, sB1, sS1);
+        if (i < nsteps) step(ks + i, sA0, sB0, sB1);
     };
     // Row groups of this wave that hold at least one valid row, counted up to the last such group (the
     // valid rows of a tile are a prefix wherever the row maps come from this library's own alignment;
@@ -644,7 +657,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // 8 bytes per lane and column-tile pair.
     if constexpr (ACT) {
         float actv[TM][TN / 4][8];
-        float* const amax_mine = wn == 0 ? sS0 : sS1;  // the scale stages are idle now
+        float* const amax_lo = sTab, * const amax_hi = sTab + BM * kScaleChunk;  // the scale table is idle now
+        float* const amax_mine = wn == 0 ? amax_lo : amax_hi;
         // (one branch on the type around all 64 elements of the lane, so that their chains interleave)
         auto activate = [&](auto type_tag) {
             using T = decltype(type_tag);
@@ -677,7 +691,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
             const int rt = tile_row(tm) + li;
-            const float amax = fmaxf(sS0[rt], sS1[rt]);
+            const float amax = fmaxf(amax_lo[rt], amax_hi[rt]);
             const float sc1 = amax == 0.f ? 1.0f : amax / 448.0f;
             const int dst = s_dst[rt];
             if (dst < 0) continue;
