@@ -625,11 +625,12 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // Row groups of this wave that hold at least one valid row, counted up to the last such group (the
     // valid rows of a tile are a prefix wherever the row maps come from this library's own alignment;
     // any other map only costs the skipped work).  Dense problems skip nothing: one copy of the loop.
+    int n_tm = TM;
     if constexpr (GROUP == GROUP_DENSE) {
         k_loop(std::integral_constant<int, TM>{});
     } else {
         static_assert(TM == 4, "dispatch below");
-        int n_tm = 0;
+        n_tm = 0;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
             if (__ballot(s_dst[tile_row(tm) + li] >= 0) != 0) n_tm = tm + 1;
@@ -663,14 +664,22 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         auto activate = [&](auto type_tag) {
             using T = decltype(type_tag);
 #pragma unroll
-            for (int tm = 0; tm < TM; ++tm)
+            for (int tm = 0; tm < TM; ++tm) {
+                if (tm < n_tm) {  // wave-uniform: row groups without a valid row were not computed and are not stored
 #pragma unroll
-                for (int tp = 0; tp < TN / 4; ++tp)
+                    for (int tp = 0; tp < TN / 4; ++tp)
 #pragma unroll
-                    for (int q = 0; q < 8; ++q) {
-                        const float ga = acc[2 * tp + (q >> 2)][tm][q & 3], ua = acc[TN / 2 + 2 * tp + (q >> 2)][tm][q & 3];
-                        actv[tm][tp][q] = silu_mul_round<T>((float)(T)ga, (float)(T)ua);
-                    }
+                        for (int q = 0; q < 8; ++q) {
+                            const float ga = acc[2 * tp + (q >> 2)][tm][q & 3], ua = acc[TN / 2 + 2 * tp + (q >> 2)][tm][q & 3];
+                            actv[tm][tp][q] = silu_mul_round<T>((float)(T)ga, (float)(T)ua);
+                        }
+                } else {
+#pragma unroll
+                    for (int tp = 0; tp < TN / 4; ++tp)
+#pragma unroll
+                        for (int q = 0; q < 8; ++q) actv[tm][tp][q] = 0.f;
+                }
+            }
         };
         if (p.act_is_bf16) activate(__bf16{});
         else activate(_Float16{});
