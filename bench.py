@@ -43,8 +43,8 @@ ROTATE_BYTES = 640 << 20
 # Decode entries are the average over M = 1, 8, 16 of one projection (same grid).
 KIB = 1024
 MEASURED_TRAFFIC = {
-    "c3_prefill_qkv_M8192": (147668.3 * 2 + 98800.2) * KIB,
-    "c3_prefill_gate_up_M8192": (688618.2 * 2 + 460672.2) * KIB,
+    "c3_prefill_qkv_M8192": (147830.5 * 2 + 98766.2) * KIB,
+    "c3_prefill_gate_up_M8192": (689064.4 * 2 + 460647.2) * KIB,
     "c2_decode_qkv": (12497.2 * 2 + 100.0) * KIB,
     "c2_decode_o": (8370.3 * 2 + 66.7) * KIB,
     "c2_decode_gate_up": (57522.9 * 2 + 467.1) * KIB,
