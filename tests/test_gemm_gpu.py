@@ -654,6 +654,53 @@ def test_fused_experts_fp8_small(device, in_dtype):
         fused_experts_impl(hidden.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device), use_fp8_w8a8=False)
 
 
+def test_launches_replay_from_a_hip_graph(device):
+    """Every entry point only enqueues on the caller's stream (no allocation, synchronisation or memset of its
+    own), so a caller may capture it: the MoE layer (align, quantizer, both grouped GEMMs with the fused
+    activation epilogue, top-k sum) and a split-K decode GEMM with its workspace are captured once and replayed
+    three times with eager work in between; every replay must reproduce the eager result bit for bit."""
+    from tilegym_amd.ops import fused_moe
+
+    g = _g(33)
+    T, E, k, H, I = 600, 4, 2, 256, 384
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16).to(device)
+    w1q, w1s = R.quantize_weight_128x128(torch.randn(E * 2 * I, H, generator=g) * 0.05)
+    w2q, w2s = R.quantize_weight_128x128(torch.randn(E * H, I, generator=g) * 0.05)
+    w1q, w1s = w1q.reshape(E, 2 * I, H).to(device), w1s.reshape(E, 2 * I // 128, H // 128).to(device)
+    w2q, w2s = w2q.reshape(E, H, I).to(device), w2s.reshape(E, H // 128, I // 128).to(device)
+    tw, ids = W.moe_routing(T, E, k, seed=6)
+    tw, ids = tw.to(device), ids.to(device)
+    a = fp8_randn((16, 14336), g).to(device)
+    b = fp8_randn((4096, 14336), g, 0.05).to(device)
+    one = torch.ones(1, device=device)
+
+    def work():
+        out = fused_moe(hidden, w1q, w2q, tw, ids, w1_scale=w1s, w2_scale=w2s)
+        return out, matmul(a, b, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+
+    eager_moe, eager_mm = work()
+    assert _lib.last_config()["SPLIT_K"] > 1  # the decode GEMM takes the split-K path (workspace + reduction)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()  # warm-up on the capture stream (workspace allocation happens here, not under capture)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_moe, g_mm = work()
+    for rep in range(3):
+        g_moe.zero_()
+        g_mm.zero_()
+        hidden.add_(0.0)  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_moe, eager_moe), f"MoE layer differs on replay {rep}"
+        assert torch.equal(g_mm, eager_mm), f"split-K GEMM differs on replay {rep}"
+
+
 def test_config5_fused_experts_full_size(device):
     """DeepSeek-V2-Lite MoE layer at full size (4096 tokens, 64 experts, top-6, H 2048, I 1408) through
     fused_moe; the oracle is evaluated on 24 sampled tokens (a token's output depends on its own row only)."""
