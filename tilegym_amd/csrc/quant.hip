@@ -38,36 +38,60 @@ __device__ __forceinline__ v8f_q load8<float>(const float* p) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// kGroupsPerLane groups per 16 lanes, all loads issued before the first use (one 16-byte load per lane
+// leaves too few bytes in flight per wave for an HBM-bound kernel).
+constexpr int kQuantGroupsPerLane = 4;
+
 template <typename T>
 __global__ void __launch_bounds__(256) act_quant_1x128_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
                                                              float* __restrict__ scales, int64_t groups, float eps,
                                                              int flashinfer_rule) {
-    const int64_t g = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-    if (g >= groups) return;  // whole 16-lane groups leave together: the shuffles below stay inside a group
+    constexpr int G = kQuantGroupsPerLane;
     const int sub = threadIdx.x & 15;
-    const int64_t base = g * 128 + sub * 8;
-    const v8f_q v = load8<T>(x + base);
-    float amax = 0.f;
+    const int64_t g0 = (int64_t)blockIdx.x * (16 * G) + (threadIdx.x >> 4);
+    v8f_q v[G];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    for (int j = 0; j < G; ++j) {
+        const int64_t g = g0 + j * 16;
+        // whole 16-lane groups are in or out together: the shuffles below stay inside a group
+        if (g < groups) v[j] = load8<T>(x + g * 128 + sub * 8);
+        else {
 #pragma unroll
-    for (int d = 1; d < 16; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
-    float s;
-    if (flashinfer_rule) s = fmaxf(amax, eps) / 448.0f;
-    else s = amax == 0.f ? 1.0f : amax / 448.0f;
-    int packed[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        float c[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) c[i] = fminf(fmaxf(v[4 * h + i] / s, -448.0f), 448.0f);
-        int w = 0;
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], w, false);
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
-        packed[h] = w;
+            for (int i = 0; i < 8; ++i) v[j][i] = 0.f;
+        }
     }
-    *reinterpret_cast<v2i*>(q + base) = v2i{packed[0], packed[1]};
-    if (sub == 0) scales[g] = s;
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        const int64_t g = g0 + j * 16;
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[j][i]));
+#pragma unroll
+        for (int d = 1; d < 16; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+        float s;
+        if (flashinfer_rule) s = fmaxf(amax, eps) / 448.0f;
+        else s = amax == 0.f ? 1.0f : amax / 448.0f;
+        if (g >= groups) continue;
+        const ScaleDivider div(s);
+        float c[8];
+        if (div.fast) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) c[i] = div.quotient(v[j][i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) c[i] = v[j][i] / s;
+        }
+        int packed[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            int w = 0;
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(fminf(fmaxf(c[4 * h], -448.0f), 448.0f), fminf(fmaxf(c[4 * h + 1], -448.0f), 448.0f), w, false);
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(fminf(fmaxf(c[4 * h + 2], -448.0f), 448.0f), fminf(fmaxf(c[4 * h + 3], -448.0f), 448.0f), w, true);
+            packed[h] = w;
+        }
+        *reinterpret_cast<v2i*>(q + g * 128 + sub * 8) = v2i{packed[0], packed[1]};
+        if (sub == 0) scales[g] = s;
+    }
 }
 
 // Between the two MoE GEMMs: act = silu(gate) * up of a (R, 2*I) bf16/f16 GEMM output (gate =
@@ -136,7 +160,8 @@ __global__ void __launch_bounds__(256) moe_sum_kernel(const T* __restrict__ x, T
 hipError_t run_act_quant_1x128(const void* x, int x_type, uint8_t* q, float* scales, int64_t groups, float eps,
                                int flashinfer_rule, hipStream_t s) {
     if (groups <= 0) return hipSuccess;
-    const dim3 grid((unsigned)((groups + 15) / 16)), block(256);
+    constexpr int per_wg = 16 * kQuantGroupsPerLane;
+    const dim3 grid((unsigned)((groups + per_wg - 1) / per_wg)), block(256);
     if (x_type == OUT_BF16)
         hipLaunchKernelGGL(act_quant_1x128_kernel<__bf16>, grid, block, 0, s, (const __bf16*)x, q, scales, groups, eps, flashinfer_rule);
     else if (x_type == OUT_F16)

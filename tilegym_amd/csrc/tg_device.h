@@ -172,15 +172,16 @@ __device__ __forceinline__ float silu_mul_round(float gate, float up) {
 // exponent range this is the compiler's own expansion of a float division without the operand
 // pre-scaling and the special-case fix-up, which only act on extreme exponents (reciprocal estimate,
 // one Newton step, then two residual corrections of the quotient; the reciprocal is shared by all
-// numerators).  Where the pre-scaling would act on a tiny quotient (|a / s| < 2^-90) the result may
-// differ in its last bits; every caller rounds the quotient to e4m3, where all such values are zero
-// of the same sign.  For other divisors (zero, subnormal, huge, inf, nan) `fast` is false and the caller
+// numerators).  The fast form is used for 2^-60 <= s <= 2^60: every numerator whose quotient is not
+// far below the smallest e4m3 step (|a / s| >= 2^-30) then has normal residuals, so the corrections
+// are exact; smaller quotients may differ in their last bits, and every caller rounds the quotient to
+// e4m3, where all such values are zero of the same sign.  For other divisors (zero, subnormal, huge, inf, nan) `fast` is false and the caller
 // divides plainly; the test is per divisor so that a caller branches once for all its numerators.
 struct ScaleDivider {
     float s, r;
     bool fast;
     __device__ __forceinline__ explicit ScaleDivider(float scale) : s(scale) {
-        fast = scale >= 0x1p-100f && scale <= 0x1p100f;
+        fast = scale >= 0x1p-60f && scale <= 0x1p60f;
         const float r0 = __builtin_amdgcn_rcpf(scale);
         r = __builtin_fmaf(__builtin_fmaf(-scale, r0, 1.0f), r0, r0);
     }
