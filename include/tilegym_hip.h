@@ -148,7 +148,8 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
  * Replaces the GEMM1 + SiLU-and-multiply steps of fused_experts_impl, src/tilegym/ops/moe_interface.py:252-277
  * (activation: src/tilegym/ops/ops.py:172-193).
  * b (E, 2*I, K) e4m3 with I % 128 == 0 and K % 128 == 0; q (num_valid, I) e4m3; scales (num_valid, I/128) f32;
- * act_dtype: TG_BF16 or TG_F16; block_m (the moe_align block size) must be a multiple of 256; the other
+ * act_dtype: TG_BF16 or TG_F16; block_m (the moe_align block size) must be a multiple of 128 (256-row tiles when
+ * it is a multiple of 256, else 128-row tiles); the other
  * arguments as for tg_fp8_moe_gemm.  Shapes outside these limits return TG_ERR_INVALID: call the two-step form.
  */
 int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* a, const tg_tensor* b,

@@ -136,7 +136,7 @@ def test_moe_gemm_silu_quant_argument_validation():
         ds = [_lib.make_tensor_desc(t) for t in (q, scales, a, b, a_s, b_s, sorted_ids, expert_ids, post)]
         return L.tg_fp8_moe_gemm_silu_quant(*[ctypes.byref(d) for d in ds], top_k, block_m, act, 0, 0)
 
-    assert call(block_m=128) == -6                                          # row tile of the fused form
+    assert call(block_m=64) == -6                                           # row tile of the fused form
     assert call(top_k=0) == -6
     assert call(act=_lib._DTYPE_CODES[torch.float32]) == -2                 # 16-bit intermediate type only
     assert call(q=torch.zeros(T * top_k, I, dtype=torch.bfloat16)) == -2
@@ -148,7 +148,8 @@ def test_moe_gemm_silu_quant_argument_validation():
     assert call(expert_ids=torch.zeros(1, dtype=torch.int32)) == -6
     assert call(sorted_ids=torch.zeros(512, dtype=torch.int64)) == -2
     assert call(q=torch.zeros(0, I).to(FP8), scales=torch.zeros(0, 1)) == 0  # nothing to do, no device needed
-    assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * I, K), 128)
+    assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * I, K), 64)
+    assert _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * I, K), 128)
     assert _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * I, K), 256)
     assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * 200, K), 256)
 

@@ -552,11 +552,12 @@ def test_silu_mul_quant_kernel(device, dtype, R_, I):
     assert same > 0.995, f"only {same:.4f} of the codes equal the oracle's"
 
 
+@pytest.mark.parametrize("block_m", [256, 128])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,E,top_k,H,I", [(64, 4, 2, 256, 128), (300, 8, 2, 512, 384), (700, 3, 1, 128, 1408)])
-def test_moe_gemm_silu_quant_equals_the_two_steps(device, dtype, T, E, top_k, H, I):
+def test_moe_gemm_silu_quant_equals_the_two_steps(device, dtype, T, E, top_k, H, I, block_m):
     """GEMM1 with the activation and the 1x128 re-quantization in its epilogue returns the very bits of
-    GEMM1 (256-row blocks) followed by the stand-alone activation kernel, and stays within that kernel's
+    GEMM1 (same row blocks) followed by the stand-alone activation kernel, and stays within that kernel's
     bar against the oracle (src/tilegym/ops/moe_interface.py:252-277, src/tilegym/ops/ops.py:172-193)."""
     g = _g(T + I)
     A = fp8_randn((T, H), g)
@@ -567,13 +568,13 @@ def test_moe_gemm_silu_quant_equals_the_two_steps(device, dtype, T, E, top_k, H,
     if E > 2:
         ids[ids == 1] = 2  # an expert without tokens
     Ad, Bd, asd, bsd = A.to(device), B.to(device), a_s.to(device), b_s.to(device)
-    sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids.to(device), 256, E)
+    sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids.to(device), block_m, E)
     C = torch.zeros(T, top_k, 2 * I, dtype=dtype, device=device)
     invoke_fused_moe_kernel(Ad, Bd, C, asd, bsd, w.to(device), ids.to(device), sorted_ids, expert_ids, post,
-                            False, top_k, {"BLOCK_SIZE_M": 256}, compute_type=dtype, use_fp8_w8a8=True)
+                            False, top_k, {"BLOCK_SIZE_M": block_m}, compute_type=dtype, use_fp8_w8a8=True)
     q2, s2 = _lib.silu_mul_quant_1x128(C.view(T * top_k, 2 * I))
-    assert _lib.moe_gemm_silu_quant_ok(Bd, 256)
-    q, s = _lib.fp8_moe_gemm_silu_quant(Ad, Bd, asd, bsd, sorted_ids, expert_ids, post, top_k, 256, T * top_k, dtype)
+    assert _lib.moe_gemm_silu_quant_ok(Bd, block_m)
+    q, s = _lib.fp8_moe_gemm_silu_quant(Ad, Bd, asd, bsd, sorted_ids, expert_ids, post, top_k, block_m, T * top_k, dtype)
     used("tiled")
     assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
     # against the oracle: its GEMM1 output rounded to the 16-bit type, then its activation + quantization

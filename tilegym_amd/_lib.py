@@ -252,7 +252,7 @@ def fp8_moe_gemm(c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids, expe
 def moe_gemm_silu_quant_ok(b, block_m) -> bool:
     """Shapes the fused GEMM1 + SiLU-multiply + 1x128 quantization entry point accepts."""
     two_i, k = b.shape[1], b.shape[2]
-    return two_i % 256 == 0 and k % 128 == 0 and 128 <= k <= 65536 and block_m % 256 == 0
+    return two_i % 256 == 0 and k % 128 == 0 and 128 <= k <= 65536 and block_m % 128 == 0
 
 
 def fp8_moe_gemm_silu_quant(a, b, a_scale, b_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,

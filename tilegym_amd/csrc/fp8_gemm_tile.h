@@ -247,7 +247,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     static_assert(!SPLIT || GROUP == GROUP_DENSE, "split-K is dense only");
     // fused activation epilogue (MoE gate/up GEMM): a tile is 128 gate columns + the 128 matching up columns
     constexpr bool ACT = GROUP == GROUP_GATHER_ACT;
-    static_assert(!ACT || (BLOCKSCALE && BM == 256 && BN == 256 && WGM == 4 && WGN == 2), "fused activation: block-scaled 256x256 only");
+    static_assert(!ACT || (BLOCKSCALE && BN == 256 && WTN % 64 == 0 && WGN * BM <= 2 * BM * kScaleChunk),
+                  "fused activation: block-scaled, 128 gate + 128 up columns per tile, each wave with as many gate as up column tiles");
 
     __shared__ __align__(1024) uint8_t sA0[BM * kKBlock];
     __shared__ __align__(1024) uint8_t sA1[BM * kKBlock];
@@ -339,8 +340,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     for (int i = 0; i < B_IT; ++i) {
         const int br = (i * NL + (wave % NL)) * 8 + lrow;  // slab row
         int n;
-        // fused activation: wave column wn owns slab rows 128*wn .. +127 = 64 gate rows, then the 64 up rows of the same columns
-        if constexpr (ACT) n = ((br >> 6) & 1) * p.inter + n0 + (br >> 7) * 64 + (br & 63);
+        // fused activation: wave column wn owns slab rows WTN*wn .. +WTN-1 = WTN/2 gate rows, then the WTN/2 up rows of the same columns
+        if constexpr (ACT) n = ((br % WTN) / (WTN / 2)) * p.inter + n0 + (br / WTN) * (WTN / 2) + br % (WTN / 2);
         else n = min(n0 + br, p.N - 1);
         b_off[i] = (uint32_t)n * (uint32_t)K + ljb * 16;
     }
@@ -648,18 +649,17 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     __syncthreads();
 
     // ---------------------------------------------------------------- fused activation epilogue
-    // Wave (wm, wn) holds, for its four 16-row groups, gate columns 64*wn .. +63 of the tile in column tiles
-    // 0..3 and the matching up columns in column tiles 4..7: a lane has gate and up of the same 16
-    // elements of each of its four rows in registers and computes, exactly as the stand-alone kernel
+    // Wave (wm, wn) holds, for its 16-row groups, gate columns (WTN/2)*wn .. of the tile in its first
+    // TN/2 column tiles and the matching up columns in the other TN/2: a lane has gate and up of the same
+    // elements of each of its rows in registers and computes, exactly as the stand-alone kernel
     // does on the stored GEMM output,
     //   g = T(acc_gate), u = T(acc_up), act = T(g * sigmoid(g) * u)          (T = the 16-bit type)
-    // The maximum of a row's 128 activations (4 lanes x 2 waves) goes through two shuffles and one LDS
+    // The maximum of a row's 128 activations (4 lanes x WGN waves) goes through two shuffles and one LDS
     // exchange; then scale = amax / 448 (1 for an all-zero group), codes = e4m3(act / scale), written
     // 8 bytes per lane and column-tile pair.
     if constexpr (ACT) {
         float actv[TM][TN / 4][8];
-        float* const amax_lo = sTab, * const amax_hi = sTab + BM * kScaleChunk;  // the scale table is idle now
-        float* const amax_mine = wn == 0 ? amax_lo : amax_hi;
+        float* const amax_mine = sTab + wn * BM;  // (the scale table is idle now) one row of maxima per wave column
         // (one branch on the type around all 64 elements of the lane, so that their chains interleave)
         auto activate = [&](auto type_tag) {
             using T = decltype(type_tag);
@@ -700,7 +700,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
             const int rt = tile_row(tm) + li;
-            const float amax = fmaxf(amax_lo[rt], amax_hi[rt]);
+            float amax = sTab[rt];
+#pragma unroll
+            for (int w = 1; w < WGN; ++w) amax = fmaxf(amax, sTab[w * BM + rt]);
             const float sc1 = amax == 0.f ? 1.0f : amax / 448.0f;
             const int dst = s_dst[rt];
             if (dst < 0) continue;
@@ -729,7 +731,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
                     w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
                     packed[h] = w;
                 }
-                *reinterpret_cast<v2i*>(qout + (int64_t)dst * p.inter + n0 + wn * 64 + tp * 32 + lg * 8) = v2i{packed[0], packed[1]};
+                *reinterpret_cast<v2i*>(qout + (int64_t)dst * p.inter + n0 + wn * (WTN / 2) + tp * 32 + lg * 8) = v2i{packed[0], packed[1]};
             }
             if (wn == 0 && lg == 0) p.act_scales[(int64_t)dst * groups_per_row + tile_n] = sc1;
         }

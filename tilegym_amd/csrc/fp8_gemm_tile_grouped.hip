@@ -20,9 +20,11 @@ hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p
     return hipErrorInvalidConfiguration;
 }
 
-// Gate/up MoE GEMM with the SiLU-multiply-quantize epilogue (256x256 tiles: 128 gate + 128 up columns).
-hipError_t run_tile_moe_act(const GemmParams& p, int gx, hipStream_t s) {
-    return launch_tile<256, 256, 4, 2, true, GROUP_GATHER_ACT, false>(p, gx, 1, s);
+// Gate/up MoE GEMM with the SiLU-multiply-quantize epilogue (a tile is 128 gate + 128 up columns; 256 or 128 rows).
+hipError_t run_tile_moe_act(int bm, const GemmParams& p, int gx, hipStream_t s) {
+    if (bm == 256) return launch_tile<256, 256, 4, 2, true, GROUP_GATHER_ACT, false>(p, gx, 1, s);
+    if (bm == 128) return launch_tile<128, 256, 2, 4, true, GROUP_GATHER_ACT, false>(p, gx, 1, s);
+    return hipErrorInvalidConfiguration;
 }
 
 }  // namespace tg

@@ -21,7 +21,7 @@ struct TileShape { int bm, bn; };
 // Launchers return hipErrorInvalidConfiguration when the combination is not instantiated.
 hipError_t run_tile_per_tensor(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
 hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
-hipError_t run_tile_moe_act(const GemmParams& p, int gx, hipStream_t s);
+hipError_t run_tile_moe_act(int bm, const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p, int gx, hipStream_t s);
 // up to kListMax per-tensor NT problems in one launch (tile 256x256, 128x128 or 64x128)
 hipError_t run_tile_list(int bm, int bn, const GemmList& gl, int gx, hipStream_t s);

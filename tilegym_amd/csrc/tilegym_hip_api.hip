@@ -565,11 +565,11 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
     }
     int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
     if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, true))) {
-        // measured on the 64-expert workload (384 rows per expert): 256x256 is 7-12 % faster than
-        // 128x128 although a quarter of its row tiles is padding; below ~192 rows per expert the
-        // padding wins
-        if (total_m / E >= 192 && N >= 256) { bm = 256; bn = 256; }
-        else { bm = (total_m / E >= 96) ? 128 : 64; bn = 128; }
+        // measured on 64 experts of (2816, 2048) weights: padding rows cost no MFMA work (the kernel skips
+        // row groups without valid rows), so 256x256 wins from ~96 rows per expert up (101 vs 106-109 us
+        // at 96, 172 vs 184-209 at 300), 128x128 down to ~40 (88 vs 102 us at 64), 64x128 below (69 vs 80 at 24)
+        if (total_m / E >= 96 && N >= 256) { bm = 256; bn = 256; }
+        else { bm = (total_m / E >= 40) ? 128 : 64; bn = 128; }
     }
     s.kernel = 1; s.bm = bm; s.bn = bn;
     remember(s);
@@ -681,7 +681,7 @@ int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, 
     if (N % 2 || I % 128 || I == 0) return fail(TG_ERR_INVALID, "b must hold 2*I rows per expert with I a positive multiple of 128 (got %lld)", (long long)N);
     if (K % 128 || K == 0 || K > 65536) return fail(TG_ERR_INVALID, "K must be a multiple of 128 in [128, 65536]");
     if (top_k <= 0) return fail(TG_ERR_INVALID, "top_k must be positive");
-    if (block_m <= 0 || block_m % 256) return fail(TG_ERR_INVALID, "block_m must be a positive multiple of 256 for the fused form");
+    if (block_m <= 0 || block_m % 128) return fail(TG_ERR_INVALID, "block_m must be a positive multiple of 128 for the fused form");
     const int64_t num_valid = q->shape[0];
     if (q->shape[1] != I) return fail(TG_ERR_INVALID, "q must have %lld columns", (long long)I);
     if (num_valid > T * top_k) return fail(TG_ERR_INVALID, "q has %lld rows but a provides only %lld slots", (long long)num_valid, (long long)(T * top_k));
@@ -729,11 +729,12 @@ int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, 
     p.act_scales = reinterpret_cast<float*>(scales->ptr);
     p.act_is_bf16 = act_dtype == TG_BF16 ? 1 : 0;
 
-    Schedule s{1, 256, 256, 1, -1, -1, -1};
+    const int bm = block_m % 256 == 0 ? 256 : 128;  // a row tile must not span two alignment blocks (experts)
+    Schedule s{1, bm, 256, 1, -1, -1, -1};
     remember(s);
-    const int64_t gx = cdiv(EM, 256) * (I / 128);
+    const int64_t gx = cdiv(EM, bm) * (I / 128);
     if (gx > INT32_MAX) return fail(TG_ERR_INVALID, "too many tiles");
-    hipError_t e = tg::run_tile_moe_act(p, (int)gx, stream);
+    hipError_t e = tg::run_tile_moe_act(bm, p, (int)gx, stream);
     if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "fused MoE kernel launch failed: %s", hipGetErrorString(e));
     return TG_OK;
 }
