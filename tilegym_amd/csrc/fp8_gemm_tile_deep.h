@@ -1,0 +1,156 @@
+// Deep-pipelined form of the 64x128 per-tensor tile (16 < M <= 64, usually with split-K): three LDS
+// stages of one K step each (3 x 24 KiB, two workgroups per compute unit), loads requested two steps
+// ahead, one barrier per step (four stages measured the same).
+// These launches are weight-streaming: a workgroup runs 8-16 K steps of 8 MFMAs per wave, and with the
+// two stages of fp8_gemm_tile.h (weights one step ahead) every step waited for a full trip to HBM
+// (1.3-2.2 k clocks per step measured, against 0.8 k of load issue and 0.26 k of MFMA).
+//
+// Same slab layout, swizzles, fragment addressing, MFMA order per accumulator and epilogue arithmetic
+// as fp8_gemm_tile_kernel<64, 128, 1, 4, false, GROUP_DENSE, SPLIT>: identical results.
+//
+// Step k of a workgroup:   wait until the loads of step k have landed (all but the newest step's worth)
+//                          barrier            (every wave's share of step k is in LDS; everyone is done with step k-1)
+//                          request step k+2 into the stage step k-1 used
+//                          fragments of step k -> MFMAs
+// Steps past the end re-fetch the last one, which keeps the wait counts uniform.
+#pragma once
+
+#include "fp8_gemm_tile.h"
+
+namespace tg {
+
+template <bool SPLIT>
+__global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int BM = 64, BN = 128, WGN = 4, NW = 4, NL = 4, STAGES = 3, AHEAD = STAGES - 1;
+    constexpr int WTN = BN / WGN;            // 32 columns per wave, all 64 rows
+    constexpr int TM = BM / 16, TN = WTN / 16;
+    constexpr int RPP = 8 * NL;
+    constexpr int A_IT = BM / RPP, B_IT = BN / RPP;
+    constexpr int STAGE_BYTES = (BM + BN) * kKBlock;
+    static_assert(TN == 2 && A_IT == 2 && B_IT == 4 && NW == WGN, "shape");
+
+    __shared__ __align__(1024) uint8_t lds[STAGES * STAGE_BYTES];  // stage s: A slab (8 KiB), then B slab (16 KiB)
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave;
+    const int K = p.K;
+    const int tiles_n = (p.N + BN - 1) / BN, tiles_m = (p.M + BM - 1) / BM;
+    const int pid = xcd_remap((int)blockIdx.x, tiles_m * tiles_n);
+    constexpr int GM = 8;
+    const int width = GM * tiles_n;
+    const int group = pid / width, first_m = group * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    const int tile_m = first_m + (pid % width) % gsz, tile_n = (pid % width) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int rows_valid = min(BM, p.M - m0);
+
+    int ks = 0, ks_end = p.kblocks;
+    if constexpr (SPLIT) {
+        ks = blockIdx.y * p.ksteps_per_split;
+        ks_end = min(ks + p.ksteps_per_split, p.kblocks);
+    }
+    const int nsteps = ks_end - ks, last = ks_end - 1;
+    if (nsteps <= 0) return;
+
+    const int lrow = lane >> 3;
+    const int lj = (lane & 7) ^ swz16(lrow);
+    const int ljb = (lane & 7) ^ swz_w(((wave & 1) << 3) | lrow);
+    uint32_t a_off[A_IT], b_off[B_IT];
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+        const int r = (i * NL + wave) * 8 + lrow;
+        a_off[i] = (uint32_t)(m0 + min(r, rows_valid - 1)) * (uint32_t)K + lj * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) {
+        const int br = (i * NL + wave) * 8 + lrow;
+        b_off[i] = (uint32_t)min(n0 + br, p.N - 1) * (uint32_t)K + ljb * 16;
+    }
+    const v4i rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(p.B);
+    const uint32_t lds0 = lds_address(lds) + wave * 1024;
+    auto issue = [&](int kstep, int stage) {  // this wave's share of one K step: 2 + 4 direct loads
+        const int k0 = min(kstep, last) * kKBlock;
+        const uint32_t dst = lds0 + stage * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) direct_load_b128(rsrc_a, dst + i * NL * 1024, a_off[i], k0);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) direct_load_b128_nt(rsrc_b, dst + BM * kKBlock + i * NL * 1024, b_off[i], k0);
+    };
+
+    const int li = lane & 15, lg = lane >> 4;
+    const uint32_t frag0 = li * kKBlock + ((lg ^ swz16(li)) << 4), frag1 = frag0 ^ 64;
+    const int wrow = ((li >> 2) << 3) | (li & 3);
+    const uint32_t wfrag0 = BM * kKBlock + wn * WTN * kKBlock + wrow * kKBlock + ((lg ^ swz_w(wrow)) << 4), wfrag1 = wfrag0 ^ 64;
+
+    v4f acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    // vmcnt(n): all of this wave's direct loads except the n most recent have landed
+    constexpr int PER_STEP = A_IT + B_IT;
+    constexpr int kKeep = (AHEAD - 1) * PER_STEP;  // the steps after the one about to be used may still be in flight
+    constexpr int kWaitStep = 0x0F70 | (kKeep & 15) | ((kKeep >> 4) << 14);
+    constexpr int kWaitAll = 0x0F70;
+    constexpr int kWaitLds = 0xC07F;
+
+#pragma unroll
+    for (int s = 0; s < AHEAD; ++s) issue(ks + s, s);
+    for (int i = 0; i < nsteps; ++i) {
+        const int stage = i % STAGES;
+        __builtin_amdgcn_s_waitcnt(kWaitStep);
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        __builtin_amdgcn_s_barrier();
+        issue(ks + i + AHEAD, (i + AHEAD) % STAGES);
+        const uint8_t* base = lds + stage * STAGE_BYTES;
+        v8i af[TM];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const uint8_t* a = base + tm * 16 * kKBlock;
+            af[tm] = join(*reinterpret_cast<const v4i*>(a + frag0), *reinterpret_cast<const v4i*>(a + frag1));
+        }
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            const uint8_t* b = base + ((tn >> 1) * 32 + (tn & 1) * 4) * kKBlock;
+            const v8i wf = join(*reinterpret_cast<const v4i*>(b + wfrag0), *reinterpret_cast<const v4i*>(b + wfrag1));
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitAll);  // the re-fetches past the end must land before the workgroup's LDS is released
+
+    // epilogue, straight from the accumulators (row 16*tm + li, eight consecutive columns per lane)
+    float scale = p.alpha;
+    if (p.As) scale *= p.As[0];
+    if (p.Bs) scale *= p.Bs[0];
+    const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;
+    const int64_t MN = (int64_t)p.M * p.N;
+    const int col = n0 + wn * WTN + lg * 8;
+    auto emit = [&](auto type_tag) {
+        constexpr int OT = decltype(type_tag)::value;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            const int rt = tm * 16 + li;
+            if (rt >= rows_valid || col >= p.N) continue;
+            if constexpr (SPLIT)
+                store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, m0 + rt, col, p.N, acc[0][tm], acc[1][tm], 0.f, vec_ok);
+            else
+                store8(p.C, OT, m0 + rt, col, p.N, acc[0][tm] * scale, acc[1][tm] * scale, p.beta, vec_ok);
+        }
+    };
+    if (SPLIT || p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
+    else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
+    else emit(std::integral_constant<int, OUT_F16>{});
+#endif
+}
+
+template <bool SPLIT>
+inline hipError_t launch_tile_deep(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
+    hipLaunchKernelGGL(fp8_gemm_tile_deep_kernel<SPLIT>, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace tg

@@ -1,5 +1,6 @@
 // Instantiations of the LDS-tiled kernel: per-tensor scales, dense rows.
 #include "fp8_gemm_tile.h"
+#include "fp8_gemm_tile_deep.h"
 #include "tg_host.h"
 
 namespace tg {
@@ -16,6 +17,10 @@ hipError_t run_tile_per_tensor(int bm, int bn, bool split, const GemmParams& p, 
     TG_CASE(64, 128, 1, 4)
 #undef TG_CASE
     return hipErrorInvalidConfiguration;
+}
+
+hipError_t run_tile_deep(bool split, const GemmParams& p, int gx, int gy, hipStream_t s) {
+    return split ? launch_tile_deep<true>(p, gx, gy, s) : launch_tile_deep<false>(p, gx, gy, s);
 }
 
 }  // namespace tg

@@ -20,6 +20,8 @@ struct TileShape { int bm, bn; };
 
 // Launchers return hipErrorInvalidConfiguration when the combination is not instantiated.
 hipError_t run_tile_per_tensor(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
+// 64x128 per-tensor tile with four LDS stages (loads three K steps ahead): the 16 < M <= 64 form
+hipError_t run_tile_deep(bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
 hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
 hipError_t run_tile_moe_act(int bm, const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p, int gx, hipStream_t s);

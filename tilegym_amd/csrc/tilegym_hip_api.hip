@@ -239,6 +239,13 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     }
     if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
+    } else if (want_split < 0 && M <= 64 && !block_scaled) {
+        // weight-streaming regime, four-stage 64x128 kernel (one workgroup per compute unit): the largest
+        // power-of-two split that keeps the grid within one round of the chip and >= 8 K steps per split
+        // (measured at M = 32 and 64 on the four Llama shapes: 4 / 4 / 1 / 8 for qkv / o / gate+up / down)
+        int want = 1;
+        while (want < 16 && want * 2 * wgs <= 256 && kblocks / (want * 2) >= 8) want *= 2;
+        if (want > 1) s.split_k = pick_split(wgs, want * wgs, kblocks, 4, M, N, partial_bytes_avail, want);
     } else if (want_split < 0 && M <= 64) {
         // weight-streaming regime: at least 128 workgroups and at most 16 K steps per split
         int64_t units = 128;
@@ -463,7 +470,9 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
             if (gx > cus) gx = cus;
         }
         const bool split = pc.split_k > 1;
+        const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128;
         hipError_t e = s.kernel == 4 ? tg::run_pipe(8, s.waves, pc, gx, stream)
+                     : deep ? tg::run_tile_deep(split, pc, gx, pc.split_k, stream)
                      : block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
                                     : tg::run_tile_per_tensor(s.bm, s.bn, split, pc, gx, pc.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "tiled kernel launch failed: %s", hipGetErrorString(e));
