@@ -221,7 +221,10 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // that, so compare the two by (fraction of the rounds' slots that hold a tile) x (tile rate).
         auto fill = [&](int64_t n, int64_t slots) { return (double)n / (double)(cdiv(n, slots) * slots); };
         const double s256 = fill(tiles(256, 256), 256) * 1.0, s128 = fill(tiles(128, 128), 512) * 0.83;
-        if (M <= 64) { bm = 64; bn = 128; }
+        // the three-stage 64x128 kernel (per-tensor) also wins above 64 rows while its tiles fit one round of the
+        // chip: 13.3 / 14.5 / 17.8 / 18.1 us against 17.1 / 18.8 / 18.7 / 21.6 for M = 96 / 128 / 256 / 512 at
+        // N = K = 4096; with more tiles the larger tiles' operand reuse wins (M = 1024: 32 vs 23 us)
+        if (M <= 64 || (!block_scaled && tiles(64, 128) <= 256)) { bm = 64; bn = 128; }
         else if (tiles(256, 256) >= 200 && s256 >= s128) { bm = 256; bn = 256; }
         else if (!block_scaled && tiles(128, 256) >= 200 && tiles(256, 256) < 200) { bm = 128; bn = 256; }
         else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
@@ -239,7 +242,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     }
     if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
-    } else if (want_split < 0 && M <= 64 && !block_scaled) {
+    } else if (want_split < 0 && bm == 64 && bn == 128 && !block_scaled) {
         // weight-streaming regime, four-stage 64x128 kernel (one workgroup per compute unit): the largest
         // power-of-two split that keeps the grid within one round of the chip and >= 8 K steps per split
         // (measured at M = 32 and 64 on the four Llama shapes: 4 / 4 / 1 / 8 for qkv / o / gate+up / down)
