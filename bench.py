@@ -43,8 +43,8 @@ ROTATE_BYTES = 640 << 20
 # Decode entries are the average over M = 1, 8, 16 of one projection (same grid).
 KIB = 1024
 MEASURED_TRAFFIC = {
-    "c3_prefill_qkv_M8192": (147830.5 * 2 + 98766.2) * KIB,
-    "c3_prefill_gate_up_M8192": (689064.4 * 2 + 460647.2) * KIB,
+    "c3_prefill_qkv_M8192": (147821.3 * 2 + 98752.3) * KIB,
+    "c3_prefill_gate_up_M8192": (689130.5 * 2 + 460665.8) * KIB,
     "c2_decode_qkv": (12497.2 * 2 + 100.0) * KIB,
     "c2_decode_o": (8370.3 * 2 + 66.7) * KIB,
     "c2_decode_gate_up": (57522.9 * 2 + 467.1) * KIB,
@@ -53,9 +53,12 @@ MEASURED_TRAFFIC = {
 
 
 def kernel_symbol(shape):
-    """Device function a measured shape ran (the stream kernel's 64-row form is a kernel of its own)."""
+    """Device function a measured shape ran (the stream kernel's 64-row form and the three-stage 64x128
+    per-tensor tile are kernels of their own)."""
     if shape["kernel"] == "stream" and shape["row_groups"] == 4:
         return "fp8_gemm_stream_wide_kernel"
+    if shape["kernel"] == "tiled" and shape["block_m"] == 64 and shape["block_n"] == 128 and not shape.get("block_scaled", False):
+        return "fp8_gemm_tile_deep_kernel"
     return KERNEL_SYMBOLS[shape["kernel"]]
 
 
