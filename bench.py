@@ -294,6 +294,14 @@ def main():
         del runners
         torch.cuda.empty_cache()
 
+    # ------------------------------------------------------------------ config 1 (the reference's CPU-runnable case; a parity case, timed for completeness)
+    if args.workload in ("prefill", "all"):
+        case = W.config1()
+        r = DenseRunner(case, device, copies=_copies_for(case.algorithmic_bytes()))
+        detail["config1"] = [measure_shape(r, max(args.steps, 64), args.warmup, stream, use_graph=not args.no_graph)]
+        del r
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ decode
     if args.workload in ("decode", "all"):
         shapes = []
