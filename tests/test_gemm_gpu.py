@@ -445,6 +445,49 @@ def test_moe_gather_gemm(device, block_m, mul_w):
     check(C, ref, what=f"moe gather block_m={block_m} mul={mul_w}")
 
 
+@pytest.mark.parametrize("block_m", [256, 128, 64])
+def test_moe_gather_with_holes_in_the_slot_sequence(device, block_m):
+    """Slots masked out in the middle of an expert's group (sentinel ids) and ids beyond the output's rows: the row
+    groups a wave skips are decided from the row map itself, not from a "valid rows are a prefix" assumption.  Rows
+    that stay valid match the oracle, every other output row is left untouched."""
+    g = _g(block_m + 1)
+    T, E, N, K, top_k = 300, 3, 256, 256, 2
+    A = fp8_randn((T, K), g)
+    B = fp8_randn((E, N, K), g, 0.5)
+    a_s = torch.rand(T, K // 128, generator=g) + 0.1
+    b_s = torch.rand(E, N // 128, K // 128, generator=g) + 0.1
+    w, ids = W.moe_routing(T, E, top_k, seed=7)
+    ref = R.ref_fused_moe_gemm(A, B, a_s, b_s, w, ids, False, top_k).reshape(T * top_k, N)
+    sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids.to(device), block_m, E)
+    sorted_ids = sorted_ids.clone()
+    hole = torch.rand(sorted_ids.numel(), generator=g) < 0.3
+    hole[:40] = True                                  # a whole leading stretch of the first tile as well
+    sorted_ids[hole.to(device)] = T * top_k           # the sentinel
+    num_valid = T * top_k - 37                        # ids >= num_valid have no output row
+    C = torch.zeros(num_valid, N, dtype=torch.bfloat16, device=device)
+    _lib.fp8_moe_gemm(C, A.to(device), B.to(device), a_s.to(device), b_s.to(device), w.to(device), sorted_ids, expert_ids, post,
+                      False, top_k, block_m)
+    used("tiled")
+    kept = torch.zeros(T * top_k, dtype=torch.bool)
+    live = sorted_ids.cpu()
+    live = live[(live >= 0) & (live < num_valid)].long()
+    kept[live] = True
+    kept = kept[:num_valid]
+    check(C[kept.to(device)], ref[:num_valid][kept], what=f"gather with holes, block_m={block_m}")
+    assert (C[(~kept).to(device)] == 0).all()
+    if block_m >= 128:
+        B2 = fp8_randn((E, 2 * 128, K), g, 0.5)
+        b2_s = torch.rand(E, 2, K // 128, generator=g) + 0.1
+        C1 = torch.zeros(T, top_k, 256, dtype=torch.bfloat16, device=device)
+        invoke_fused_moe_kernel(A.to(device), B2.to(device), C1, a_s.to(device), b2_s.to(device), w.to(device), ids.to(device),
+                                sorted_ids, expert_ids, post, False, top_k, {"BLOCK_SIZE_M": block_m}, use_fp8_w8a8=True)
+        q2, s2 = _lib.silu_mul_quant_1x128(C1.view(T * top_k, 256)[:num_valid].contiguous())
+        q, s_ = _lib.fp8_moe_gemm_silu_quant(A.to(device), B2.to(device), a_s.to(device), b2_s.to(device), sorted_ids, expert_ids, post,
+                                             top_k, block_m, num_valid, torch.bfloat16)
+        kd = kept.to(device)
+        assert torch.equal(q.view(torch.uint8)[kd], q2.view(torch.uint8)[kd]) and torch.equal(s_[kd], s2[kd])
+
+
 def test_moe_fc2_shape_top_k_1(device):
     """Second MoE GEMM: activations already expanded per slot (top_k = 1), routed weight applied
     (src/tilegym/ops/moe_interface.py:290-307)."""
