@@ -11,11 +11,15 @@
 //
 // The MFMA "row" operand is fed from B (weights) and the "column" operand from A
 // (activations): a lane then owns, for one activation row m, four consecutive n, so a
-// per-token scale is one register per lane.
+// per-token scale is one register per lane.  The weight rows of a column-tile pair are
+// permuted so that those four-column runs of the two tiles join into eight consecutive columns.
 //
-// Epilogue: each wave passes its accumulators through the (now idle) LDS in 64-column slices
-// and writes C with one 16-byte store per lane, rows contiguous; scaling, beta, routed weights
-// and the output cast happen in that short rolled loop.
+// Epilogue: straight from the accumulators, one 16-byte store (8 bf16/f16 outputs) per lane and
+// column-tile pair; scaling, beta, routed weights and the output cast happen there.  The gate/up
+// form of the MoE layer computes SiLU(gate) * up and its 1 x 128 e4m3 quantization instead.
+//
+// Rows are dealt to the wave rows in interleaved 16-row groups, and the grouped forms run the K
+// loop specialised on how many of a wave's row groups hold valid rows: padding rows cost no MFMAs.
 //
 // Scale modes:  per-tensor (one multiply in the epilogue) or block-scaled (every K step's
 // 16x16 product is multiplied by As[m,kb] * Bs[n/128,kb] while it is added to the
@@ -254,7 +258,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     __shared__ __align__(1024) uint8_t sA1[BM * kKBlock];
     __shared__ __align__(1024) uint8_t sB0[BN * kKBlock];
     __shared__ __align__(1024) uint8_t sB1[BN * kKBlock];
-    // per-stage activation scales of the slab rows (block-scaled kernels only)
+    // activation scales of the tile rows, two chunks of kScaleChunk K steps (block-scaled kernels only)
     __shared__ __align__(256) float sTab[BLOCKSCALE ? 2 * BM * kScaleChunk : 1];
     // weight block scales of this tile's column blocks for every K step (fetched once)
     __shared__ float sBs[BLOCKSCALE ? (BN + 127) / 128 : 1][BLOCKSCALE ? kMaxKBlocks : 1];
@@ -577,8 +581,8 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // Stage buffers (sA0,sB0) and (sA1,sB1); step k computes from stage k%2.  The B slab of a stage
     // is read throughout the step, the A slab only at its start (the A fragments stay in
     // registers), so A is prefetched two steps ahead and B one:
-    //   top of step k : issue B(k+1) (and its activation scales) -> other stage;  read A fragments
-    //                   (and scales) of stage k%2;  barrier
+    //   top of step k : issue B(k+1) -> other stage (and one row group of the next chunk of activation
+    //                   scales);  read A fragments (and scales) of stage k%2;  barrier
     //                   (every wave holds its A fragments: that A slab is free)
     //   then          : issue A(k+2) -> this stage's A slab;  MFMAs with B fragments streamed from LDS
     //   end of step k : wait for all direct loads except A(k+2);  barrier
