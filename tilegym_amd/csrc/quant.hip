@@ -9,11 +9,12 @@
 //   q     = rne_e4m3(clamp(x / scale, -448, 448))
 // Arithmetic of src/tilegym/suites/unsloth/cutile/fp8.py:92-120 and
 // src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:22-66; both divisions are
-// IEEE divisions (a reciprocal multiply moves values across rounding boundaries).
+// correctly rounded (IEEE) divisions (a plain reciprocal multiply moves values across rounding boundaries).
 //
-// HBM-bound: 16 lanes own one group (8 elements = one 16-byte load of bf16/f16 per lane, two for
-// fp32), the maximum is reduced over the 16 lanes with cross-lane shuffles, every lane writes 8
-// bytes of codes and lane 0 of the group the scale.
+// HBM-bound: 16 lanes own one group at a time (8 elements = one 16-byte load of bf16/f16 per lane,
+// two for fp32) and four groups in all, whose loads are issued together; the maximum is reduced over
+// the 16 lanes with cross-lane shuffles, every lane writes 8 bytes of codes and lane 0 of the group
+// the scale.  The divisions go through ScaleDivider (bit-equal to the IEEE division).
 #include "tg_host.h"
 
 typedef float v8f_q __attribute__((ext_vector_type(8)));
