@@ -745,6 +745,28 @@ def test_launches_replay_from_a_hip_graph(device):
         assert torch.equal(g_mm, eager_mm), f"split-K GEMM differs on replay {rep}"
 
 
+def test_fused_moe_more_tokens_than_one_chunk(device):
+    """33000 tokens: fused_experts_impl works in chunks of 32768 tokens (src/tilegym/ops/moe_interface.py:216-233);
+    rows around the chunk boundary and at both ends against the oracle."""
+    from tilegym_amd.ops import fused_moe
+
+    g = _g(3)
+    T, E, k, H, I = 33000, 4, 2, 256, 128
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w1q, w1s = R.quantize_weight_128x128(torch.randn(E * 2 * I, H, generator=g) * 0.05)
+    w2q, w2s = R.quantize_weight_128x128(torch.randn(E * H, I, generator=g) * 0.05)
+    w1q, w1s = w1q.reshape(E, 2 * I, H), w1s.reshape(E, 2 * I // 128, H // 128)
+    w2q, w2s = w2q.reshape(E, H, I), w2s.reshape(E, H // 128, I // 128)
+    tw, ids = W.moe_routing(T, E, k, seed=5)
+    out = fused_moe(hidden.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device),
+                    w1_scale=w1s.to(device), w2_scale=w2s.to(device))
+    rows = torch.cat([torch.arange(0, 40), torch.arange(32748, 32808), torch.arange(T - 40, T)])
+    ref = R.ref_fused_experts_fp8(hidden[rows], w1q, w2q, w1s, w2s, tw[rows], ids[rows])
+    ok, rep = R.compare_to_oracle(out[rows.to(device)], ref, RTOL, ATOL)
+    # one flipped activation code moves the 256 outputs of its token (I = 128: one of 128 inputs of the second GEMM)
+    assert rep["matched"] >= 0.99 and rep["max_rel_to_sigma"] <= 0.1, rep
+
+
 def test_config5_fused_experts_full_size(device):
     """DeepSeek-V2-Lite MoE layer at full size (4096 tokens, 64 experts, top-6, H 2048, I 1408) through
     fused_moe; the oracle is evaluated on 24 sampled tokens (a token's output depends on its own row only)."""
