@@ -383,10 +383,25 @@ def main():
             n = max(args.steps, 32)
             us = _events_ms(fn, n, stream) * 1e3 / n
             nbytes = M * K * 3 + M * (K // 128) * 4
-            shapes.append({"name": f"act_quant_1x128_bf16_{M}x{K}", "kernel": "act_quant_1x128_kernel", "us": round(us, 2),
+            shapes.append({"name": f"act_quant_1x128_bf16_{M}x{K}", "kernel": "act_quant_group_kernel", "us": round(us, 2),
                            "gbs": round(nbytes / us * 1e-3, 1), "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
                            "note": "includes the torch allocation of the two outputs"})
             del xs
+            torch.cuda.empty_cache()
+        for (N, K) in ((28672, 4096), (12288, 5120)):
+            ws = [torch.randint(0, 120, (N, K), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+                  for _ in range(_copies_for(N * K * 3))]
+            sc = torch.rand(N // 128, K // 128, device=device) + 0.5
+            fn = lambda i: _lib.fp8_weight_dequant(ws[i % len(ws)], sc, 128, torch.bfloat16)  # noqa: E731
+            for w in range(max(1, args.warmup)):
+                fn(w)
+            n = max(args.steps, 32)
+            us = _events_ms(fn, n, stream) * 1e3 / n
+            nbytes = N * K * 3 + sc.numel() * 4
+            shapes.append({"name": f"weight_dequant_bf16_{N}x{K}", "kernel": "weight_dequant_kernel", "us": round(us, 2),
+                           "gbs": round(nbytes / us * 1e-3, 1), "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
+                           "note": "includes the torch allocation of the output"})
+            del ws
             torch.cuda.empty_cache()
         ids = W.moe_routing(4096, 64, 6, seed=0)[1].to(device)
         fn = lambda i: _lib.moe_align_block_size(ids, 128, 64)  # noqa: E731

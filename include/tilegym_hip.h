@@ -202,6 +202,29 @@ int32_t tg_fp8_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg
                            int32_t rule, int32_t device_id, uint64_t hip_stream);
 
 /*
+ * Per-token group FP8 quantizer, the general form of tg_fp8_quant_1x128: groups of group_size = 16, 32, 64 or 128
+ * consecutive elements of a row, and a third scale rule,
+ *   rule 2: as rule 1, then scale = 2^ceil(log2(max(|scale|, 1e-10)))   (power-of-two "UE8M0" scales).
+ * scales is either contiguous with numel(x) / group_size elements (row-major), or a 2-D (rows, K / group_size)
+ * descriptor with any element strides - (1, rows) is the column-major layout and (1, ceil4(rows)) the 16-byte
+ * aligned one of the reference.  rows = numel(x) / K.
+ * Replaces src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:22-145 (both kernels) and the host
+ * function at :152-272 for dst_dtype float8_e4m3fn.
+ * x (..., K) bf16 / f16 / f32 contiguous, K % group_size == 0, 16-byte aligned; q same shape e4m3fn, 8-byte aligned.
+ */
+int32_t tg_fp8_quant_group(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x, int32_t group_size,
+                           float eps, int32_t rule, int32_t device_id, uint64_t hip_stream);
+
+/*
+ * Block dequantization of a weight: y[i, j] = float(x[i, j]) * s[i / block_size, j / block_size], fp32 product
+ * rounded once to y's type.  Replaces src/tilegym/suites/unsloth/cutile/fp8.py:36-71 (kernel) and :348-367 (host).
+ * x (M, N) e4m3fn contiguous; s (ceil(M / block_size), ceil(N / block_size)) f32 contiguous; y (M, N) bf16 / f16 / f32
+ * contiguous; block_size >= 1.
+ */
+int32_t tg_fp8_weight_dequant(const tg_tensor* y, const tg_tensor* x, const tg_tensor* s, int32_t block_size,
+                              int32_t device_id, uint64_t hip_stream);
+
+/*
  * Between the two MoE GEMMs, one launch: act = silu(x[:, :I]) * x[:, I:], rounded to x's 16-bit type
  * (the reference's intermediate cache, src/tilegym/ops/moe_interface.py:206-210,272-277; silu_and_mul:
  * src/tilegym/ops/ops.py:172-193), then quantized 1 x 128 (all-zero group -> scale 1.0).  The reference

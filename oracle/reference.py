@@ -16,7 +16,10 @@ e4m3fn_decode_table            closed form of OCP FP8 E4M3 checked code by code
 e4m3fn_encode_rne              brute force over a dense grid of floats against
                                torch's ``.to(float8_e4m3fn)`` after clamping
 quantize_*                     scale*q round trip error bound, amax hits +-448,
-                               all-zero block -> scale 1.0 (unsloth) / eps (flashinfer)
+                               all-zero block -> scale 1.0 (unsloth) / eps (flashinfer);
+                               power-of-two scales against exponent-bit arithmetic;
+                               groups of 16/32/64 against a per-group loop
+weight_dequant                 element loop with ragged edge blocks
 ref_gemm_per_tensor            integer-valued inputs whose product is exact in fp32
                                (compared with an int64 matmul), power-of-two scale
                                linearity, transposed-operand shapes (M != N != K)
@@ -120,21 +123,25 @@ def quantize_per_tensor(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q, scale.reshape(1)
 
 
-def quantize_act_1x128(x: torch.Tensor, block: int = 128, eps: Optional[float] = None):
+def quantize_act_1x128(x: torch.Tensor, block: int = 128, eps: Optional[float] = None, ue8m0: bool = False):
     """Per-token 1 x ``block`` quantization; returns (q, scales[..., K/block]).
 
     ``eps=None``: the unsloth rule, all-zero block -> scale 1.0
     (tests/suites/unsloth/test_fp8.py:80-97, src/.../unsloth/cutile/fp8.py:105-116).
     ``eps=1e-10``: the flashinfer rule, amax clamped below by eps
-    (tests/suites/flashinfer/test_per_token_group_quant_8bit.py:41-68)."""
+    (tests/suites/flashinfer/test_per_token_group_quant_8bit.py:41-68); with ``ue8m0`` the scale is then
+    rounded up to a power of two, ``2^ceil(log2(max(|s|, 1e-10)))`` (same file, :61-63)."""
     assert x.shape[-1] % block == 0
     xb = x.float().reshape(-1, block)
     amax = xb.abs().amax(dim=-1, keepdim=True)
     if eps is None:
+        assert not ue8m0
         s = amax / FP8_MAX
         s = torch.where(s == 0, torch.ones_like(s), s)
     else:
         s = amax.clamp(min=eps) / FP8_MAX
+        if ue8m0:
+            s = torch.exp2(torch.ceil(torch.log2(torch.maximum(s.abs(), torch.tensor(1e-10)))))
     q = (xb / s).clamp(-FP8_MAX, FP8_MAX).to(FP8).reshape(x.shape)
     return q, s.reshape(*x.shape[:-1], x.shape[-1] // block)
 

@@ -194,6 +194,40 @@ def test_quantizer_argument_validation():
     assert quant(torch.zeros(0, 256, dtype=torch.bfloat16)) == 0       # nothing to do, no device needed
 
 
+def test_group_quantizer_and_weight_dequant_argument_validation():
+    L = _lib.load()
+
+    def quant(x, group, q=None, s=None, rule=1):
+        q = torch.zeros(x.shape, dtype=FP8) if q is None else q
+        s = torch.zeros(x.shape[:-1] + (max(x.shape[-1] // max(group, 1), 1),)) if s is None else s
+        ds = [_lib.make_tensor_desc(t) for t in (q, s, x)]
+        return L.tg_fp8_quant_group(*[ctypes.byref(d) for d in ds], group, 1e-10, rule, 0, 0)
+
+    x = torch.zeros(6, 256, dtype=torch.float16)
+    assert quant(x, 48) == -6 and quant(x, 256) == -6 and quant(x, 0) == -6     # group size
+    assert quant(torch.zeros(6, 200, dtype=torch.float16), 64) == -6            # K % group
+    assert quant(x, 64, rule=3) == -6
+    assert quant(x, 64, s=torch.zeros(6, 3)) == -6
+    assert quant(x, 64, s=torch.zeros(6, 4, dtype=torch.int32)) == -2
+    assert quant(x, 64, s=torch.zeros(6, 4).t()) == -6                          # strided, but not (rows, groups)
+    assert quant(x, 64, s=torch.zeros(4).expand(6, 4)) == -6                    # overlapping elements
+    assert quant(torch.zeros(0, 256, dtype=torch.float16), 64, s=torch.zeros(0, 4)) == 0
+
+    def dequant(x, s, y=None, bs=128):
+        y = torch.zeros(x.shape, dtype=torch.bfloat16) if y is None else y
+        ds = [_lib.make_tensor_desc(t) for t in (y, x, s)]
+        return L.tg_fp8_weight_dequant(*[ctypes.byref(d) for d in ds], bs, 0, 0)
+
+    w = torch.zeros(200, 300).to(FP8)
+    assert dequant(w, torch.ones(2, 2)) == -6                                   # s must be (2, 3)
+    assert dequant(w, torch.ones(2, 3), bs=0) == -6
+    assert dequant(w.view(torch.uint8), torch.ones(2, 3)) == -2
+    assert dequant(w, torch.ones(2, 3, dtype=torch.int32)) == -2
+    assert dequant(w, torch.ones(2, 3), y=torch.zeros(200, 300, dtype=torch.int32)) == -2
+    assert dequant(w, torch.ones(2, 3), y=torch.zeros(200, 301, dtype=torch.bfloat16)) == -6
+    assert dequant(torch.zeros(0, 300).to(FP8), torch.ones(0, 3)) == 0          # nothing to do, no device needed
+
+
 def test_workspace_bytes_and_cfg():
     L = _lib.load()
     cfg, n = _lib.make_cfg(None)

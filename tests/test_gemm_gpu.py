@@ -560,6 +560,78 @@ def test_act_quant_kernels_bit_exact(device, dtype, shape):
         assert not bad.any(), f"{rule}: {int(bad.sum())} of {bad.numel()} codes differ"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("group", [16, 32, 64, 128])
+@pytest.mark.parametrize("tokens,hidden", [(1, 128), (513, 2048), (37, 384)])
+def test_group_quantizer_forms_bit_exact(device, dtype, group, tokens, hidden):
+    """Group sizes and scale layouts of per_token_group_quant_8bit
+    (tests/suites/flashinfer/test_per_token_group_quant_8bit.py:70-110 sweeps the same group sizes and
+    513 tokens): row-major, column-major, the aligned column-major form (returned row-major, as the
+    reference returns it), power-of-two scales; and act_quant with the same group sizes.  Codes and
+    scales bit for bit against the oracle."""
+    from tilegym_amd.suites.flashinfer.ops import per_token_group_quant_8bit
+    from tilegym_amd.suites.unsloth.ops import act_quant
+
+    g = _g(tokens + hidden + group)
+    x = torch.randn(tokens, hidden, generator=g) * torch.exp(torch.randn(tokens, 1, generator=g) * 2)
+    flat = x.reshape(-1, group)
+    flat[0] = 0.0
+    if flat.shape[0] > 3:
+        flat[1] *= 1e-12
+        flat[2] = 448.0 * 2.0 ** -5 * torch.sign(flat[2] + 1e-30)   # plain scale exactly 2^-5
+        flat[3, 0] = 448.0 * 2.0 ** -5 * 1.5                        # plain scale 1.5 * 2^-5 at least
+    x = x.clamp(-6e4, 6e4).to(dtype)
+    xd = x.to(device)
+    G = hidden // group
+
+    def same(q, s, q_ref, s_ref, what):
+        assert q.dtype == FP8 and s.dtype == torch.float32 and q.shape == x.shape and s.shape == s_ref.shape, what
+        assert torch.equal(s.cpu().view(torch.int32), s_ref.view(torch.int32)), f"{what}: scales differ"
+        bad = q.cpu().view(torch.uint8) != q_ref.view(torch.uint8)
+        assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} codes differ"
+
+    q_ref, s_ref = R.quantize_act_1x128(x, group, 1e-10)
+    q, s = per_token_group_quant_8bit(xd, group)
+    assert s.is_contiguous()
+    same(q, s, q_ref, s_ref, "row-major")
+    q, s = per_token_group_quant_8bit(xd, group, column_major_scales=True)
+    assert s.shape == (tokens, G) and (G == 1 or tokens == 1 or s.stride() == (1, tokens))
+    same(q, s, q_ref, s_ref, "column-major")
+    q, s = per_token_group_quant_8bit(xd, group, column_major_scales=True, scale_tma_aligned=True)
+    assert s.is_contiguous()
+    same(q, s, q_ref, s_ref, "aligned column-major")
+    q_ref2, s_ref2 = R.quantize_act_1x128(x, group, 1e-10, ue8m0=True)
+    q, s = per_token_group_quant_8bit(xd, group, column_major_scales=True, scale_ue8m0=True)
+    same(q, s, q_ref2, s_ref2, "power-of-two scales")
+    q, s = per_token_group_quant_8bit(xd, group, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    same(q, s, q_ref2, s_ref2, "power-of-two scales, aligned")
+    q_ref3, s_ref3 = R.quantize_act_1x128(x, group, None)
+    q, s = act_quant(xd, group)
+    same(q, s, q_ref3, s_ref3, "act_quant")
+    with pytest.raises(AssertionError):
+        per_token_group_quant_8bit(xd, group, scale_ue8m0=True)     # needs column_major_scales, as in the reference
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N,bs", [(256, 384, 128), (200, 300, 128), (70, 150, 32), (2816, 2048, 128), (33, 48, 16), (5, 7, 3)])
+def test_weight_dequant_bit_exact(device, dtype, M, N, bs):
+    """Every e4m3 code (NaN codes included) times a block scale, rounded once to the output type,
+    against the oracle; ragged edge blocks, vector and element forms of the kernel."""
+    from tilegym_amd.suites.unsloth.ops import weight_dequant
+
+    g = _g(M + N + bs)
+    codes = torch.randint(0, 256, (M, N), generator=g, dtype=torch.int32).to(torch.uint8)
+    w = codes.view(FP8)
+    sc = torch.exp(torch.randn(-(-M // bs), -(-N // bs), generator=g) * 2)
+    y_ref = R.weight_dequant(w, sc, bs, dtype)
+    y = weight_dequant(w.to(device), sc.to(device), bs, dtype)
+    assert y.dtype == dtype and y.shape == (M, N)
+    nan = torch.isnan(y_ref.float())
+    assert torch.equal(torch.isnan(y.cpu().float()), nan)
+    bits = torch.int32 if dtype == torch.float32 else torch.int16
+    assert torch.equal(y.cpu().view(bits)[~nan], y_ref.view(bits)[~nan])
+
+
 def test_quantize_then_gemm_end_to_end(device):
     """bf16 activations -> HIP quantizer -> block-scaled GEMM, against the oracle on the same bf16 input."""
     from tilegym_amd.suites.unsloth.ops import act_quant

@@ -1,6 +1,8 @@
 """Pins of the CPU oracle (oracle/reference.py, oracle/fp8_oracle.c): closed forms, exact integer
 cases, brute force on tiny inputs, invariants, and the reference's one known-answer vector."""
 
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -69,6 +71,40 @@ def test_quantizers_scale_rule_and_zero_blocks():
     assert (back - w).abs().max() <= w.abs().max() * 2 ** -4
     qt, st = R.quantize_per_tensor(w)
     assert st.shape == (1,) and torch.equal(st[0], w.abs().max() / 448.0)
+
+
+def test_quantizer_power_of_two_scales_and_small_groups():
+    """Pins of the remaining quantizer forms: (a) with ue8m0 every scale is the smallest power of two that is
+    not below the plain scale (exponent arithmetic on the fp32 bits, no logarithm), (b) groups of 16 / 32 / 64
+    against a per-group Python loop, (c) weight_dequant against an element loop with ragged edge blocks."""
+    x = torch.randn(9, 256, generator=_g(11)) * 3.0
+    x[4, 128:] = 0
+    x[5, :128] = 448.0 * 2.0 ** -7                                   # plain scale exactly 2^-7: must stay 2^-7
+    for block in (16, 32, 64, 128):
+        q, s = R.quantize_act_1x128(x, block, eps=1e-10)
+        qp, sp = R.quantize_act_1x128(x, block, eps=1e-10, ue8m0=True)
+        bits = sp.view(torch.int32)
+        assert torch.all((bits & 0x7FFFFF) == 0) and torch.all(sp > 0)   # powers of two
+        floor_pow2 = torch.maximum(s, torch.tensor(1e-10)).view(torch.int32).bitwise_and(0x7F800000).view(torch.float32)
+        want = torch.where(floor_pow2 == torch.maximum(s, torch.tensor(1e-10)), floor_pow2, floor_pow2 * 2)
+        assert torch.equal(sp, want)
+        xb = x.reshape(-1, block)
+        for gi in (0, 3, xb.shape[0] - 1):                           # per-group loop
+            amax = max(abs(v) for v in xb[gi].tolist())
+            sc = np.float32(max(amax, 1e-10)) / np.float32(448.0)
+            assert np.float32(s.reshape(-1)[gi].item()) == sc
+            codes = (xb[gi] / torch.tensor(sc)).clamp(-448, 448).to(FP8)
+            assert torch.equal(codes.view(torch.uint8), q.reshape(-1, block)[gi].view(torch.uint8))
+            codes2 = (xb[gi] / sp.reshape(-1)[gi]).clamp(-448, 448).to(FP8)
+            assert torch.equal(codes2.view(torch.uint8), qp.reshape(-1, block)[gi].view(torch.uint8))
+    assert sp.reshape(9, 2)[5, 0] == 2.0 ** -7 and sp.reshape(9, 2)[4, 1] == 2.0 ** math.ceil(math.log2(1e-10))
+    w = (torch.randn(70, 150, generator=_g(12)) * 50).to(FP8)
+    sc = torch.rand(3, 5, generator=_g(13)) + 0.5
+    y = R.weight_dequant(w, sc, 32, torch.float32)
+    wf = R.fp8_to_f32(w)
+    for i, j in ((0, 0), (31, 32), (69, 149), (64, 127), (33, 96)):
+        assert y[i, j] == wf[i, j] * sc[i // 32, j // 32]
+    assert torch.equal(R.weight_dequant(w, sc, 32, torch.bfloat16), y.to(torch.bfloat16))
 
 
 # ---------------------------------------------------------------- GEMMs

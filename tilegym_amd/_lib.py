@@ -107,6 +107,10 @@ def load():
     L.tg_moe_align_block_size.argtypes = [P, ctypes.c_int32, ctypes.c_int32, P, P, P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_fp8_quant_1x128.restype = ctypes.c_int32
     L.tg_fp8_quant_1x128.argtypes = [P, P, P, ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_quant_group.restype = ctypes.c_int32
+    L.tg_fp8_quant_group.argtypes = [P, P, P, ctypes.c_int32, ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_weight_dequant.restype = ctypes.c_int32
+    L.tg_fp8_weight_dequant.argtypes = [P, P, P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     L.tg_silu_mul_quant_1x128.restype = ctypes.c_int32
     L.tg_silu_mul_quant_1x128.argtypes = [P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_moe_sum.restype = ctypes.c_int32
@@ -307,6 +311,32 @@ def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = F
                               float(eps), 1 if flashinfer_rule else 0, _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_fp8_quant_1x128")
     return q, scales
+
+
+def fp8_quant_group(x: torch.Tensor, group_size: int, eps: float, rule: int, scales: Optional[torch.Tensor] = None):
+    """(q e4m3fn like x, scales) through tg_fp8_quant_group; rule 0 zero-group -> 1, 1 eps clamp, 2 eps clamp and
+    power-of-two scales.  ``scales`` may be a 2-D (rows, K/group_size) f32 tensor with any strides (column-major
+    layouts); by default it is allocated row-major with x's leading shape."""
+    L = load()
+    x = x.contiguous()
+    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    if scales is None:
+        scales = torch.empty(x.shape[:-1] + (x.shape[-1] // group_size,), dtype=torch.float32, device=x.device)
+    rc = L.tg_fp8_quant_group(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+                              int(group_size), float(eps), int(rule), _device_index(x), _stream_handle(x))
+    check_rc(rc, "tg_fp8_quant_group")
+    return q, scales
+
+
+def fp8_weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, dtype: torch.dtype) -> torch.Tensor:
+    """y (M, N) of ``dtype`` = float(x) * s[i // block_size, j // block_size] through tg_fp8_weight_dequant."""
+    L = load()
+    x, s = x.contiguous(), s.contiguous()
+    y = torch.empty(x.shape, dtype=dtype, device=x.device)
+    rc = L.tg_fp8_weight_dequant(_ref(make_tensor_desc(y)), _ref(make_tensor_desc(x)), _ref(make_tensor_desc(s)),
+                                 int(block_size), _device_index(x), _stream_handle(x))
+    check_rc(rc, "tg_fp8_weight_dequant")
+    return y
 
 
 def silu_mul_quant_1x128(x: torch.Tensor):

@@ -1,19 +1,23 @@
-// Elementwise producers around the FP8 GEMMs: the per-token 1 x 128 activation quantizer, the
-// SiLU-and-multiply + requantization between the two MoE GEMMs, and the top-k combine.
+// Elementwise producers and consumers around the FP8 GEMMs: the per-token group quantizer, the block
+// dequantizer of a weight, the SiLU-and-multiply + requantization between the two MoE GEMMs, and the
+// top-k combine.
 //
-// Per-token 1 x 128 FP8 (e4m3fn) activation quantizer: the producer of the (M, K/128) scale
-// layout the block-scaled GEMMs consume.
-//   amax over each group of 128 consecutive elements of a row
-//   scale = amax / 448                      (all-zero group -> 1.0)        unsloth rule
-//           max(amax, eps) / 448                                           flashinfer rule
+// Per-token group FP8 (e4m3fn) activation quantizer (groups of 16, 32, 64 or 128 consecutive elements
+// of a row; 128 gives the (M, K/128) scale layout the block-scaled GEMMs consume):
+//   amax over the group
+//   scale = amax / 448                      (all-zero group -> 1.0)        rule 0, unsloth
+//           max(amax, eps) / 448                                           rule 1, flashinfer
+//           2^ceil(log2(max(that, 1e-10)))                                 rule 2, flashinfer with power-of-two scales
 //   q     = rne_e4m3(clamp(x / scale, -448, 448))
 // Arithmetic of src/tilegym/suites/unsloth/cutile/fp8.py:92-120 and
-// src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:22-66; both divisions are
+// src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:22-145; both divisions are
 // correctly rounded (IEEE) divisions (a plain reciprocal multiply moves values across rounding boundaries).
+// The scale of group j of row r is written to scales[r * row_stride + j * col_stride], which covers the
+// row-major layout and the column-major ones of per_token_group_quant_8bit.py:185-204.
 //
-// HBM-bound: 16 lanes own one group at a time (8 elements = one 16-byte load of bf16/f16 per lane,
-// two for fp32) and four groups in all, whose loads are issued together; the maximum is reduced over
-// the 16 lanes with cross-lane shuffles, every lane writes 8 bytes of codes and lane 0 of the group
+// HBM-bound: group_size / 8 lanes own one group at a time (8 elements = one 16-byte load of bf16/f16 per
+// lane, two for fp32) and four groups in all, whose loads are issued together; the maximum is reduced over
+// those lanes with cross-lane shuffles, every lane writes 8 bytes of codes and the first lane of the group
 // the scale.  The divisions go through ScaleDivider (bit-equal to the IEEE division).
 #include "tg_host.h"
 
@@ -39,23 +43,27 @@ __device__ __forceinline__ v8f_q load8<float>(const float* p) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// kGroupsPerLane groups per 16 lanes, all loads issued before the first use (one 16-byte load per lane
+// kQuantGroupsPerLane groups per lane, all loads issued before the first use (one 16-byte load per lane
 // leaves too few bytes in flight per wave for an HBM-bound kernel).
 constexpr int kQuantGroupsPerLane = 4;
 
-template <typename T>
-__global__ void __launch_bounds__(256) act_quant_1x128_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
+enum QuantRule { QUANT_ZERO_TO_ONE = 0, QUANT_EPS = 1, QUANT_EPS_POW2 = 2 };
+
+// LPG lanes per group (group size 8 * LPG).  STRIDED: the scale of group j of row r goes to
+// scales[r * s_row + j * s_col] (groups < 2^31); otherwise to scales[g].
+template <typename T, int LPG, bool STRIDED>
+__global__ void __launch_bounds__(256) act_quant_group_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
                                                              float* __restrict__ scales, int64_t groups, float eps,
-                                                             int flashinfer_rule) {
-    constexpr int G = kQuantGroupsPerLane;
-    const int sub = threadIdx.x & 15;
-    const int64_t g0 = (int64_t)blockIdx.x * (16 * G) + (threadIdx.x >> 4);
+                                                             int rule, uint32_t groups_per_row, int64_t s_row, int64_t s_col) {
+    constexpr int G = kQuantGroupsPerLane, GS = 8 * LPG, PASS = 256 / LPG;
+    const int sub = threadIdx.x & (LPG - 1);
+    const int64_t g0 = (int64_t)blockIdx.x * (PASS * G) + (threadIdx.x / LPG);
     v8f_q v[G];
 #pragma unroll
     for (int j = 0; j < G; ++j) {
-        const int64_t g = g0 + j * 16;
-        // whole 16-lane groups are in or out together: the shuffles below stay inside a group
-        if (g < groups) v[j] = load8<T>(x + g * 128 + sub * 8);
+        const int64_t g = g0 + j * PASS;
+        // the LPG lanes of a group are in or out together: the shuffles below stay inside a group
+        if (g < groups) v[j] = load8<T>(x + g * GS + sub * 8);
         else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[j][i] = 0.f;
@@ -63,15 +71,16 @@ __global__ void __launch_bounds__(256) act_quant_1x128_kernel(const T* __restric
     }
 #pragma unroll
     for (int j = 0; j < G; ++j) {
-        const int64_t g = g0 + j * 16;
+        const int64_t g = g0 + j * PASS;
         float amax = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[j][i]));
 #pragma unroll
-        for (int d = 1; d < 16; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+        for (int d = 1; d < LPG; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
         float s;
-        if (flashinfer_rule) s = fmaxf(amax, eps) / 448.0f;
-        else s = amax == 0.f ? 1.0f : amax / 448.0f;
+        if (rule == QUANT_ZERO_TO_ONE) s = amax == 0.f ? 1.0f : amax / 448.0f;
+        else s = fmaxf(amax, eps) / 448.0f;
+        if (rule == QUANT_EPS_POW2) s = exp2f(ceilf(log2f(fmaxf(fabsf(s), 1e-10f))));
         if (g >= groups) continue;
         const ScaleDivider div(s);
         float c[8];
@@ -90,8 +99,58 @@ __global__ void __launch_bounds__(256) act_quant_1x128_kernel(const T* __restric
             w = __builtin_amdgcn_cvt_pk_fp8_f32(fminf(fmaxf(c[4 * h + 2], -448.0f), 448.0f), fminf(fmaxf(c[4 * h + 3], -448.0f), 448.0f), w, true);
             packed[h] = w;
         }
-        *reinterpret_cast<v2i*>(q + g * 128 + sub * 8) = v2i{packed[0], packed[1]};
-        if (sub == 0) scales[g] = s;
+        *reinterpret_cast<v2i*>(q + g * GS + sub * 8) = v2i{packed[0], packed[1]};
+        if (sub == 0) {
+            if constexpr (STRIDED) {
+                const uint32_t row = (uint32_t)g / groups_per_row, col = (uint32_t)g - row * groups_per_row;
+                scales[row * s_row + col * s_col] = s;
+            } else {
+                scales[g] = s;
+            }
+        }
+    }
+}
+
+// y = float(x) * s[i / bs][j / bs] for an (M, N) e4m3 weight with one fp32 scale per bs x bs block
+// (src/tilegym/suites/unsloth/cutile/fp8.py:36-71,348-367): fp32 product, rounded once to the output
+// type.  HBM-bound (1 byte in, 2 or 4 out per element).  VEC: a lane converts 16 consecutive
+// elements of one row (N % 16 == 0, bs % 16 == 0, 16-byte aligned rows); otherwise one element.
+template <typename OT, bool VEC>
+__global__ void __launch_bounds__(256) weight_dequant_kernel(const uint8_t* __restrict__ x, const float* __restrict__ s,
+                                                            OT* __restrict__ y, int64_t M, int64_t N, int bs, int64_t s_cols) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if constexpr (VEC) {
+        const int64_t chunks = N / 16;
+        if (idx >= M * chunks) return;
+        const int64_t row = idx / chunks, col = (idx - row * chunks) * 16;
+        const float scale = s[(row / bs) * s_cols + col / bs];
+        const v4i raw = *reinterpret_cast<const v4i*>(x + row * N + col);
+        typedef OT vecT __attribute__((ext_vector_type(8)));
+        typedef float v2f_q __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            v8f_q f;
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+                const v2f_q lo = __builtin_amdgcn_cvt_pk_f32_fp8(raw[2 * h + w], false);
+                const v2f_q hi = __builtin_amdgcn_cvt_pk_f32_fp8(raw[2 * h + w], true);
+                f[4 * w] = lo[0] * scale, f[4 * w + 1] = lo[1] * scale, f[4 * w + 2] = hi[0] * scale, f[4 * w + 3] = hi[1] * scale;
+            }
+            // the fp32 products are rounded on their own before the conversion (no single-rounding mixed-precision FMA)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float t = f[i];
+                asm("" : "+v"(t));
+                f[i] = t;
+            }
+            *reinterpret_cast<vecT*>(y + row * N + col + 8 * h) = __builtin_convertvector(f, vecT);
+        }
+    } else {
+        if (idx >= M * N) return;
+        const int64_t row = idx / N, col = idx - row * N;
+        float t = e4m3_to_f32(x[idx]) * s[(row / bs) * s_cols + col / bs];
+        asm("" : "+v"(t));
+        y[idx] = (OT)t;
     }
 }
 
@@ -158,20 +217,60 @@ __global__ void __launch_bounds__(256) moe_sum_kernel(const T* __restrict__ x, T
     *reinterpret_cast<vecT*>(out + idx) = __builtin_convertvector(acc, vecT);
 }
 
-hipError_t run_act_quant_1x128(const void* x, int x_type, uint8_t* q, float* scales, int64_t groups, float eps,
-                               int flashinfer_rule, hipStream_t s) {
-    if (groups <= 0) return hipSuccess;
-    constexpr int per_wg = 16 * kQuantGroupsPerLane;
+template <typename T, int LPG>
+static void launch_act_quant(const T* x, uint8_t* q, float* scales, int64_t groups, float eps, int rule, bool strided,
+                             uint32_t groups_per_row, int64_t s_row, int64_t s_col, hipStream_t s) {
+    constexpr int per_wg = (256 / LPG) * kQuantGroupsPerLane;
     const dim3 grid((unsigned)((groups + per_wg - 1) / per_wg)), block(256);
-    if (x_type == OUT_BF16)
-        hipLaunchKernelGGL(act_quant_1x128_kernel<__bf16>, grid, block, 0, s, (const __bf16*)x, q, scales, groups, eps, flashinfer_rule);
-    else if (x_type == OUT_F16)
-        hipLaunchKernelGGL(act_quant_1x128_kernel<_Float16>, grid, block, 0, s, (const _Float16*)x, q, scales, groups, eps, flashinfer_rule);
-    else if (x_type == OUT_F32)
-        hipLaunchKernelGGL(act_quant_1x128_kernel<float>, grid, block, 0, s, (const float*)x, q, scales, groups, eps, flashinfer_rule);
+    if (strided)
+        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, true>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
     else
-        return hipErrorInvalidValue;
+        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, false>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
+}
+
+template <typename T>
+static hipError_t dispatch_act_quant(const T* x, uint8_t* q, float* scales, int64_t groups, int group_size, float eps, int rule,
+                                     bool strided, uint32_t groups_per_row, int64_t s_row, int64_t s_col, hipStream_t s) {
+    switch (group_size) {
+        case 128: launch_act_quant<T, 16>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        case 64: launch_act_quant<T, 8>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        case 32: launch_act_quant<T, 4>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        case 16: launch_act_quant<T, 2>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
+}
+
+// groups of group_size (16, 32, 64, 128) elements; with `strided` the scale of group j of row r (groups_per_row
+// groups in a row) is written to scales[r * s_row + j * s_col], otherwise to scales[r * groups_per_row + j]
+hipError_t run_act_quant_group(const void* x, int x_type, uint8_t* q, float* scales, int64_t groups, int group_size, float eps,
+                               int rule, bool strided, int64_t groups_per_row, int64_t s_row, int64_t s_col, hipStream_t s) {
+    if (groups <= 0) return hipSuccess;
+    if (strided && (groups > INT32_MAX || groups_per_row <= 0)) return hipErrorInvalidValue;
+    const uint32_t gpr = (uint32_t)groups_per_row;
+    if (x_type == OUT_BF16) return dispatch_act_quant((const __bf16*)x, q, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
+    if (x_type == OUT_F16) return dispatch_act_quant((const _Float16*)x, q, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
+    if (x_type == OUT_F32) return dispatch_act_quant((const float*)x, q, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
+    return hipErrorInvalidValue;
+}
+
+template <typename OT>
+static hipError_t launch_weight_dequant(const uint8_t* x, const float* sc, OT* y, int64_t M, int64_t N, int bs, int64_t s_cols,
+                                        bool vec, hipStream_t s) {
+    const int64_t work = vec ? M * (N / 16) : M * N;
+    const dim3 grid((unsigned)((work + 255) / 256)), block(256);
+    if (vec) hipLaunchKernelGGL((weight_dequant_kernel<OT, true>), grid, block, 0, s, x, sc, y, M, N, bs, s_cols);
+    else hipLaunchKernelGGL((weight_dequant_kernel<OT, false>), grid, block, 0, s, x, sc, y, M, N, bs, s_cols);
+    return hipGetLastError();
+}
+
+hipError_t run_weight_dequant(const uint8_t* x, const float* sc, void* y, int y_type, int64_t M, int64_t N, int bs, int64_t s_cols,
+                              bool vec, hipStream_t s) {
+    if (M <= 0 || N <= 0) return hipSuccess;
+    if (y_type == OUT_BF16) return launch_weight_dequant(x, sc, (__bf16*)y, M, N, bs, s_cols, vec, s);
+    if (y_type == OUT_F16) return launch_weight_dequant(x, sc, (_Float16*)y, M, N, bs, s_cols, vec, s);
+    if (y_type == OUT_F32) return launch_weight_dequant(x, sc, (float*)y, M, N, bs, s_cols, vec, s);
+    return hipErrorInvalidValue;
 }
 
 hipError_t run_silu_mul_quant(const void* x, int x_type, uint8_t* q, float* scales, int64_t rows, int I, hipStream_t s) {

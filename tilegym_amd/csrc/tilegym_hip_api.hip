@@ -787,29 +787,84 @@ int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, i
 }
 
 
+int32_t tg_fp8_quant_group(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x, int32_t group_size,
+                           float eps, int32_t rule, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(x, "x", -1)) || (rc = check_tensor(q, "q", -1))) return rc;
+    if (!scales) return fail(TG_ERR_NULL, "scales: null tensor descriptor");
+    if (scales->ndim < 0 || scales->ndim > TG_MAX_DIMS) return fail(TG_ERR_INVALID, "scales: ndim %d out of range", scales->ndim);
+    const int x_type = out_type_of(x->dtype);
+    if (x_type < 0) return fail(TG_ERR_DTYPE, "x must be bf16, f16 or f32");
+    if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
+    if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
+    if (rule < 0 || rule > 2) return fail(TG_ERR_INVALID, "rule must be 0, 1 or 2");
+    if (group_size != 16 && group_size != 32 && group_size != 64 && group_size != 128)
+        return fail(TG_ERR_INVALID, "group_size must be 16, 32, 64 or 128, got %d", group_size);
+    if (x->ndim < 1) return fail(TG_ERR_INVALID, "x needs at least one dimension");
+    const int64_t K = x->shape[x->ndim - 1], n = numel(x);
+    if (K % group_size != 0) return fail(TG_ERR_INVALID, "the last dimension (%lld) must be a multiple of %d", (long long)K, group_size);
+    if (numel(q) != n) return fail(TG_ERR_INVALID, "q must have the shape of x");
+    const int64_t groups = n / group_size, gpr = K / group_size, rows = K > 0 ? n / K : 0;
+    if (numel(scales) != groups) return fail(TG_ERR_INVALID, "scales must have %lld elements", (long long)groups);
+    bool strided = false;
+    int64_t s_row = gpr, s_col = 1;
+    if (!contiguous(scales)) {
+        if (scales->ndim != 2 || scales->shape[0] != rows || scales->shape[1] != gpr)
+            return fail(TG_ERR_INVALID, "strided scales must be 2-D (%lld, %lld)", (long long)rows, (long long)gpr);
+        s_row = scales->strides[0], s_col = scales->strides[1];
+        if (s_row < 0 || s_col < 0) return fail(TG_ERR_INVALID, "scales: negative stride");
+        // two (row, group) pairs must not share an element: one stride has to step over the other dimension
+        const bool col_major = s_row >= 1 && s_col >= s_row * rows, row_major = s_col >= 1 && s_row >= s_col * gpr;
+        if (groups > 1 && !col_major && !row_major) return fail(TG_ERR_INVALID, "scales: overlapping strides");
+        if (groups > INT32_MAX) return fail(TG_ERR_INVALID, "too many groups for strided scales");
+        strided = true;
+    }
+    if (groups > 0 && scales->ptr == 0) return fail(TG_ERR_NULL, "scales: null data pointer");
+    if (!aligned16(x->ptr) || (q->ptr & 7) != 0) return fail(TG_ERR_INVALID, "x must be 16-byte and q 8-byte aligned");
+    if (n == 0) return TG_OK;
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipError_t e = tg::run_act_quant_group(reinterpret_cast<const void*>(x->ptr), x_type, reinterpret_cast<uint8_t*>(q->ptr),
+                                           reinterpret_cast<float*>(scales->ptr), groups, group_size, eps, rule, strided, gpr,
+                                           s_row, s_col, reinterpret_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "quantizer launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
 int32_t tg_fp8_quant_1x128(const tg_tensor* q, const tg_tensor* scales, const tg_tensor* x, float eps,
                            int32_t rule, int32_t device_id, uint64_t hip_stream) {
     g_err[0] = 0;
     int32_t rc;
     if ((rc = check_tensor(x, "x", -1)) || (rc = check_tensor(q, "q", -1)) || (rc = check_tensor(scales, "scales", -1))) return rc;
-    const int x_type = out_type_of(x->dtype);
-    if (x_type < 0) return fail(TG_ERR_DTYPE, "x must be bf16, f16 or f32");
-    if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
-    if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
     if (rule != 0 && rule != 1) return fail(TG_ERR_INVALID, "rule must be 0 or 1");
-    if (x->ndim < 1) return fail(TG_ERR_INVALID, "x needs at least one dimension");
-    const int64_t K = x->shape[x->ndim - 1], n = numel(x);
-    if (K % 128 != 0) return fail(TG_ERR_INVALID, "the last dimension (%lld) must be a multiple of 128", (long long)K);
-    if (numel(q) != n) return fail(TG_ERR_INVALID, "q must have the shape of x");
-    if (numel(scales) != n / 128) return fail(TG_ERR_INVALID, "scales must have %lld elements", (long long)(n / 128));
-    if (!aligned16(x->ptr) || (q->ptr & 7) != 0) return fail(TG_ERR_INVALID, "x must be 16-byte and q 8-byte aligned");
-    if (n == 0) return TG_OK;
+    return tg_fp8_quant_group(q, scales, x, 128, eps, rule, device_id, hip_stream);
+}
+
+int32_t tg_fp8_weight_dequant(const tg_tensor* y, const tg_tensor* x, const tg_tensor* s, int32_t block_size,
+                              int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(x, "x", 2)) || (rc = check_tensor(y, "y", 2)) || (rc = check_tensor(s, "s", 2))) return rc;
+    if (x->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "x must be float8_e4m3fn (dtype code 7)");
+    if (s->dtype != TG_F32) return fail(TG_ERR_DTYPE, "s must be f32");
+    const int y_type = out_type_of(y->dtype);
+    if (y_type < 0) return fail(TG_ERR_DTYPE, "y must be bf16, f16 or f32");
+    if (block_size < 1) return fail(TG_ERR_INVALID, "block_size must be positive");
+    const int64_t M = x->shape[0], N = x->shape[1];
+    if (y->shape[0] != M || y->shape[1] != N) return fail(TG_ERR_INVALID, "y must be (%lld, %lld)", (long long)M, (long long)N);
+    if (s->shape[0] != cdiv(M, block_size) || s->shape[1] != cdiv(N, block_size))
+        return fail(TG_ERR_INVALID, "s must be (%lld, %lld)", (long long)cdiv(M, block_size), (long long)cdiv(N, block_size));
+    if (M == 0 || N == 0) return TG_OK;
+    const bool vec = N % 16 == 0 && block_size % 16 == 0 && aligned16(x->ptr) && aligned16(y->ptr);
+    const int64_t work = vec ? M * (N / 16) : M * N;
+    if (cdiv(work, 256) > INT32_MAX) return fail(TG_ERR_INVALID, "weight too large");
     DeviceGuard guard(device_id);
     if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
-    hipError_t e = tg::run_act_quant_1x128(reinterpret_cast<const void*>(x->ptr), x_type, reinterpret_cast<uint8_t*>(q->ptr),
-                                           reinterpret_cast<float*>(scales->ptr), n / 128, eps, rule,
-                                           reinterpret_cast<hipStream_t>(hip_stream));
-    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "quantizer launch failed: %s", hipGetErrorString(e));
+    hipError_t e = tg::run_weight_dequant(reinterpret_cast<const uint8_t*>(x->ptr), reinterpret_cast<const float*>(s->ptr),
+                                          reinterpret_cast<void*>(y->ptr), y_type, M, N, block_size, s->shape[1], vec,
+                                          reinterpret_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "dequantizer launch failed: %s", hipGetErrorString(e));
     return TG_OK;
 }
 

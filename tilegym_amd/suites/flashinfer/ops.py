@@ -42,6 +42,4 @@ def _per_token_group_quant_8bit(x, group_size, eps=1e-10, dst_dtype=torch.float8
                                 column_major_scales=False, scale_tma_aligned=False, scale_ue8m0=False):
     if dst_dtype != torch.float8_e4m3fn:
         raise NotImplementedError("only float8_e4m3fn is implemented")
-    if column_major_scales or scale_tma_aligned:
-        raise NotImplementedError("only row-major scales are implemented")
-    return _quant.per_token_group_quant_fp8(x, group_size, eps, scale_ue8m0)
+    return _quant.per_token_group_quant_fp8(x, group_size, eps, scale_ue8m0, column_major_scales, scale_tma_aligned)
