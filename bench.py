@@ -43,10 +43,10 @@ ROTATE_BYTES = 640 << 20
 # Decode entries are the average over M = 1, 8, 16 of one projection (same grid).
 KIB = 1024
 MEASURED_TRAFFIC = {
-    "c3_prefill_qkv_M8192": (147821.3 * 2 + 98752.3) * KIB,
-    "c3_prefill_gate_up_M8192": (689130.5 * 2 + 460665.8) * KIB,
-    "c2_decode_qkv": (12497.2 * 2 + 100.0) * KIB,
-    "c2_decode_o": (8370.3 * 2 + 66.7) * KIB,
+    "c3_prefill_qkv_M8192": (147790.8 * 2 + 98759.7) * KIB,
+    "c3_prefill_gate_up_M8192": (689180.8 * 2 + 460607.7) * KIB,
+    "c2_decode_qkv": (12471.9 * 2 + 100.0) * KIB,
+    "c2_decode_o": (8375.9 * 2 + 66.7) * KIB,
     "c2_decode_gate_up": (57522.9 * 2 + 467.1) * KIB,
     "c2_decode_down": (29179.7 * 2 + 933.6) * KIB,
 }
