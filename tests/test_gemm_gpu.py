@@ -632,6 +632,35 @@ def test_weight_dequant_bit_exact(device, dtype, M, N, bs):
     assert torch.equal(y.cpu().view(bits)[~nan], y_ref.view(bits)[~nan])
 
 
+def test_quantizers_at_the_reference_tests_shapes(device):
+    """The shapes the reference's own tests sweep: weight_dequant (tests/suites/unsloth/test_fp8.py:41-50),
+    act_quant (:99-108,129-135), per_token_group_quant_8bit with 512 and 513 tokens of 2048
+    (tests/suites/flashinfer/test_per_token_group_quant_8bit.py:71-73), bf16 inputs as there."""
+    from tilegym_amd.suites.flashinfer.ops import per_token_group_quant_8bit
+    from tilegym_amd.suites.unsloth.ops import act_quant, weight_dequant
+
+    for (M, N) in ((256, 256), (512, 1024), (384, 768), (2048, 4096), (4096, 8192)):
+        g = _g(M + N)
+        w = torch.randn(M, N, generator=g)
+        wq, ws = R.quantize_weight_128x128(w)
+        y = weight_dequant(wq.to(device), ws.to(device), 128)
+        assert y.dtype == torch.bfloat16
+        assert torch.equal(y.cpu().view(torch.int16), R.weight_dequant(wq, ws, 128, torch.bfloat16).view(torch.int16)), (M, N)
+    for shape in ((256, 256), (64, 1024), (128, 512), (1024, 4096), (2048, 8192), (256, 128), (128, 384)):
+        x = torch.randn(shape, generator=_g(sum(shape))).to(torch.bfloat16)
+        q, sc = act_quant(x.to(device), block_size=128)
+        q_ref, s_ref = R.quantize_act_1x128(x, 128, None)
+        assert torch.equal(sc.cpu(), s_ref) and torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8)), shape
+    for tokens in (512, 513):
+        x = torch.randn(tokens, 2048, generator=_g(tokens)).to(torch.bfloat16)
+        for group in (16, 32, 64, 128):
+            for col, aligned, pow2 in ((False, False, False), (True, False, False), (True, True, False), (True, False, True), (True, True, True)):
+                q, sc = per_token_group_quant_8bit(x.to(device), group_size=group, eps=1e-10, dst_dtype=torch.float8_e4m3fn,
+                                                   column_major_scales=col, scale_tma_aligned=aligned, scale_ue8m0=pow2)
+                q_ref, s_ref = R.quantize_act_1x128(x, group, 1e-10, ue8m0=pow2)
+                assert torch.equal(sc.cpu(), s_ref) and torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8)), (tokens, group, col, aligned, pow2)
+
+
 def test_quantize_then_gemm_end_to_end(device):
     """bf16 activations -> HIP quantizer -> block-scaled GEMM, against the oracle on the same bf16 input."""
     from tilegym_amd.suites.unsloth.ops import act_quant
