@@ -276,6 +276,25 @@ def test_gemm_alpha_beta(device, alpha, beta, M, N, K, kernel):
         assert torch.equal(c2, c)
 
 
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.5, 2.0)])
+@pytest.mark.parametrize("size", [4096, 8192])
+def test_gemm_alpha_beta_reference_test_sizes(device, size, alpha, beta):
+    """m = n = k = 4096 and 8192 as in tests/suites/flashinfer/test_flashinfer_gemm_alpha_beta.py:45-55 (fp8 in,
+    bf16 out); the oracle is evaluated on 128 sampled rows (a row of the output depends on its own rows of a and c)."""
+    g = _g(size)
+    a = torch.rand(size, size, generator=g).to(torch.float16).to(FP8)
+    b = torch.rand(size, size, generator=g).to(torch.float16).to(FP8)
+    c0 = torch.rand(size, size, generator=g).to(torch.bfloat16)
+    c = c0.clone().to(device)
+    out = gemm_alpha_beta(a.to(device), b.to(device), c, False, True, alpha, beta)
+    assert out.data_ptr() == c.data_ptr()
+    rows = torch.randperm(size, generator=g)[:128].sort().values
+    rows[0], rows[-1] = 0, size - 1
+    ref = R.ref_gemm_alpha_beta(a[rows], b, c0[rows].clone(), False, True, alpha, beta)
+    check(c[rows.to(device)], ref, what=f"{size}^3 alpha={alpha} beta={beta}")
+    assert torch.isfinite(c.float()).all()
+
+
 # ----------------------------------------------------------------------------- block scaled
 @pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 256, 256), (512, 1024, 512), (1024, 2048, 1024)])
 def test_block_scaled_reference_test_shapes(device, M, N, K):
@@ -356,8 +375,8 @@ def _ragged_inputs(sizes, N, K, seed, total_extra=0):
     return a, b, a_s, b_s, ptr
 
 
-@pytest.mark.parametrize("groups,m", [(4, 128), (16, 128), (4, 512)])
-@pytest.mark.parametrize("n,k", [(2048, 2048)])
+@pytest.mark.parametrize("groups,m", [(4, 128), (16, 128), (4, 512), (16, 512)])
+@pytest.mark.parametrize("n,k", [(2048, 2048), (4096, 4096)])
 def test_ragged_reference_test_shapes(device, groups, m, n, k):
     """Group counts / segment sizes of Test_FlashInfer_RaggedBlockScaledBMM
     (tests/suites/flashinfer/test_flashinfer_ragged_block_scaled_bmm.py:216-223); that test allows atol=rtol=1."""
@@ -797,6 +816,29 @@ def test_fused_experts_fp8_small(device, in_dtype):
     assert ok, rep
     with pytest.raises(NotImplementedError):
         fused_experts_impl(hidden.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device), use_fp8_w8a8=False)
+
+
+@pytest.mark.parametrize("T,H,I,E,k", [(16, 512, 256, 8, 2), (32, 1024, 512, 16, 4), (64, 1024, 512, 20, 8)])
+def test_fused_moe_fp8_at_the_reference_tests_configurations(device, T, H, I, E, k):
+    """Token / width / expert counts and data recipe of Test_MOE.test_op (tests/ops/test_moe.py:73-145: hidden N(0, 0.5),
+    weights N(0, 0.1), topk_ids drawn with randint, so a token may name one expert twice, softmax of N(0,1) routing
+    weights) through the block-scaled FP8 layer, against the oracle."""
+    from tilegym_amd.ops import fused_moe
+
+    g = _g(T + E)
+    hidden = (torch.randn(T, H, generator=g) * 0.5).to(torch.float16)
+    w1q, w1s = R.quantize_weight_128x128(torch.randn(E * 2 * I, H, generator=g) * 0.1)
+    w2q, w2s = R.quantize_weight_128x128(torch.randn(E * H, I, generator=g) * 0.1)
+    w1q, w1s = w1q.reshape(E, 2 * I, H), w1s.reshape(E, 2 * I // 128, H // 128)
+    w2q, w2s = w2q.reshape(E, H, I), w2s.reshape(E, H // 128, I // 128)
+    ids = torch.randint(0, E, (T, k), generator=g)
+    tw = torch.softmax(torch.randn(T, k, generator=g), dim=-1).to(torch.float16)
+    ref = R.ref_fused_experts_fp8(hidden, w1q, w2q, w1s, w2s, tw.float(), ids.to(torch.int32))
+    out = fused_moe(hidden.to(device), w1q.to(device), w2q.to(device), tw.to(device), ids.to(device),
+                    w1_scale=w1s.to(device), w2_scale=w2s.to(device))
+    assert out.dtype == torch.float16 and out.shape == (T, H)
+    ok, rep = R.compare_to_oracle(out, ref, RTOL, ATOL)
+    assert rep["matched"] >= 0.999 and rep["max_rel_to_sigma"] <= 0.1, rep
 
 
 def test_launches_replay_from_a_hip_graph(device):
