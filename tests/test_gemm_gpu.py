@@ -276,6 +276,42 @@ def test_gemm_alpha_beta(device, alpha, beta, M, N, K, kernel):
         assert torch.equal(c2, c)
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (1024, 1024, 1023), (8192, 8192, 8192), (8, 8, 8), (3072, 6144, 2720)])
+def test_matmul_reference_test_shapes(device, m, n, k):
+    """Shapes and layout (a (m,k), b (k,n), no transposes) of Test_Matmul.test_op (tests/ops/test_matmul.py:15-21),
+    e4m3 operands drawn as there (N(0, 0.3), :64-66), per-tensor scales, bf16 out; K = 1023, 8 and 2720 take the
+    paths for K % 128 != 0.  The oracle is evaluated on at most 128 sampled rows."""
+    g = _g(m + k)
+    a, b = fp8_randn((m, k), g, 0.3), fp8_randn((k, n), g, 0.3)
+    sa, sb = torch.tensor(0.75), torch.tensor(1.5)
+    out = matmul(a.to(device), b.to(device), scale_a=sa.to(device), scale_b=sb.to(device), out_dtype=torch.bfloat16)
+    assert out.shape == (m, n) and out.dtype == torch.bfloat16
+    rows = _rows_subset(m, 128)
+    ref = R.ref_gemm_per_tensor(a[rows], b, sa, sb)
+    check(out[rows.to(device)], ref, what=f"matmul {m}x{n}x{k}")
+    assert torch.isfinite(out.float()).all()
+    plain = matmul(a.to(device), b.to(device))              # the reference's own call: output typed like a
+    assert plain.dtype == FP8 and plain.shape == (m, n)
+
+
+@pytest.mark.parametrize("transpose_b", [True, False])
+@pytest.mark.parametrize("group_k", [[1024, 512, 256, 128], [128, 128, 128, 128]])
+@pytest.mark.parametrize("group_n", [[1024, 512, 256, 128], [128, 128, 128, 128]])
+@pytest.mark.parametrize("group_m", [[1024, 512, 256, 128], [256, 256, 256, 256]])
+def test_group_gemm_reference_test_shapes(device, group_m, group_n, group_k, transpose_b):
+    """The group shapes of Test_GroupGemm.test_op (tests/ops/test_group_gemm.py:32-53), operands drawn as there
+    (rand in [0,1), :81-88) and cast to e4m3, bf16 out."""
+    g = _g(sum(group_m) + sum(group_n) + sum(group_k) + transpose_b)
+    As = [torch.rand(M, K, generator=g).to(torch.float16).to(FP8) for M, K in zip(group_m, group_k)]
+    Bs = [torch.rand((N, K) if transpose_b else (K, N), generator=g).to(torch.float16).to(FP8) for N, K in zip(group_n, group_k)]
+    outs = group_gemm([x.to(device) for x in As], [x.to(device) for x in Bs], transpose_b=transpose_b, out_dtype=torch.bfloat16)
+    refs = R.ref_group_gemm(As, Bs, transpose_b=transpose_b, out_dtype=torch.bfloat16)
+    assert len(outs) == len(refs) == 4
+    for i, (o, r) in enumerate(zip(outs, refs)):
+        assert o.shape == (group_m[i], group_n[i])
+        check(o, r, what=f"group {i}")
+
+
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.5, 2.0)])
 @pytest.mark.parametrize("size", [4096, 8192])
 def test_gemm_alpha_beta_reference_test_sizes(device, size, alpha, beta):
