@@ -109,6 +109,25 @@ def test_host_side_errors_mirror_the_reference():
         matmul(a, torch.zeros(8, 128).to(FP8), trans_b=True, out_dtype=torch.bfloat16)
 
 
+def test_quantizer_operators_have_no_host_path():
+    from tilegym_amd.suites.flashinfer.ops import per_token_group_quant_8bit
+    from tilegym_amd.suites.unsloth.ops import act_quant, weight_dequant
+
+    x = torch.zeros(4, 256, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        act_quant(x, 128)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        per_token_group_quant_8bit(x, 64)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        weight_dequant(torch.zeros(128, 128).to(FP8), torch.ones(1, 1))
+    with pytest.raises(AssertionError):
+        act_quant(x, 96)                                               # last dim not divisible
+    with pytest.raises(AssertionError):
+        per_token_group_quant_8bit(x, 64, scale_ue8m0=True)            # needs column_major_scales, as in the reference
+    with pytest.raises(NotImplementedError):
+        per_token_group_quant_8bit(x, 64, dst_dtype=torch.int8)
+
+
 def test_moe_align_host_logic_matches_known_answer():
     from tilegym_amd.ops import moe_align_block_size
     from tilegym_amd.ops.hip.moe import _moe_align_torch_ops

@@ -1,6 +1,6 @@
 """Seeded synthetic workloads: the five FP8 GEMM configurations the benchmark and the parity
 tests run.  Inputs are drawn on the CPU with ``torch.Generator().manual_seed(seed)`` in fp32 and
-quantized with this package's quantizers; callers move them to the device.
+quantized on the CPU by the small generators below; callers move them to the device.
 
 LLAMA_SHAPES are the Llama-3.1-8B projection shapes (N, K): QKV, O, gate+up, down.
 """
@@ -12,7 +12,8 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from . import quant
+FP8 = torch.float8_e4m3fn
+FP8_MAX = 448.0
 
 LLAMA_SHAPES: Dict[str, Tuple[int, int]] = {
     "qkv": (6144, 4096),
@@ -25,6 +26,39 @@ PREFILL_M = 8192
 BLOCK_SCALED_SHAPES = ((12288, 5120), (5120, 12288))
 BLOCK_SCALED_M = (16, 4096)
 MOE = dict(hidden=2048, inter=1408, experts=64, top_k=6, tokens=4096)
+
+
+# ---- host-side input generators: fp32 -> e4m3 codes and scales, plain torch on the CPU.  They only make the
+# ---- synthetic operands below; the operators of this package run on the device through the HIP library.
+def _quantize_per_tensor(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One fp32 scale for the whole tensor: scale = amax/448 (1.0 for an all-zero tensor)."""
+    xf = x.float()
+    amax = xf.abs().amax()
+    scale = torch.where(amax == 0, torch.ones_like(amax), amax / FP8_MAX)
+    q = (xf / scale).clamp(-FP8_MAX, FP8_MAX).to(FP8)
+    return q, scale.reshape(1)
+
+
+def _quantize_1x128(x: torch.Tensor, eps: float = 1e-10) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per (row, 128-group) scale max(amax, eps)/448, row-major scales (..., K/128)."""
+    xb = x.float().reshape(-1, 128)
+    s = xb.abs().amax(dim=-1, keepdim=True).clamp(min=eps) / FP8_MAX
+    q = (xb / s).clamp(-FP8_MAX, FP8_MAX).to(FP8).reshape(x.shape)
+    return q, s.reshape(*x.shape[:-1], x.shape[-1] // 128)
+
+
+def _quantize_weight_128x128(w: torch.Tensor, block_n: int = 128, block_k: int = 128):
+    """Per (block_n x block_k) block quantization of a (N, K) weight -> (q, Bs (ceil(N/bn), ceil(K/bk)))."""
+    N, K = w.shape
+    nb, kb = -(-N // block_n), -(-K // block_k)
+    wp = torch.zeros(nb * block_n, kb * block_k, dtype=torch.float32)
+    wp[:N, :K] = w.float()
+    blocks = wp.reshape(nb, block_n, kb, block_k)
+    amax = blocks.abs().amax(dim=(1, 3))
+    s = torch.where(amax == 0, torch.ones_like(amax), amax / FP8_MAX)
+    q = (blocks / s[:, None, :, None]).clamp(-FP8_MAX, FP8_MAX)
+    q = q.reshape(nb * block_n, kb * block_k)[:N, :K].contiguous().to(FP8)
+    return q, s
 
 
 @dataclass
@@ -94,8 +128,8 @@ def per_tensor_case(M: int, N: int, K: int, seed: int = 0, w_std: float = 1.0, o
         mask = torch.rand(M, K, generator=g) < 1e-3
         a = torch.where(mask, a * 20.0, a)
     w = torch.randn(N, K, generator=g) * w_std
-    qa, sa = quant.quantize_per_tensor(a)
-    qb, sb = quant.quantize_per_tensor(w)
+    qa, sa = _quantize_per_tensor(a)
+    qb, sb = _quantize_per_tensor(w)
     if not trans_b:
         qb = qb.view(torch.uint8).t().contiguous().view(torch.float8_e4m3fn)
     return DenseCase(name or f"pt_{M}x{N}x{K}", qa, qb, sa, sb, trans_b, False)
@@ -130,8 +164,8 @@ def block_scaled_case(M: int, N: int, K: int, seed: int = 0, name: Optional[str]
     g = _gen(seed)
     a = torch.randn(M, K, generator=g)
     w = _block_weights(N, K, g)
-    qa, sa = quant.per_token_group_quant_fp8(a, 128)
-    qb, sb = quant.weight_quant_block(w)
+    qa, sa = _quantize_1x128(a)
+    qb, sb = _quantize_weight_128x128(w)
     return DenseCase(name or f"c4_block_{M}x{N}x{K}", qa, qb, sa, sb, True, True)
 
 
@@ -168,11 +202,11 @@ def moe_grouped_case(which: str = "gate_up", seed: int = 0, tokens: Optional[int
     else:
         a = torch.randn(T * k, I, generator=g)
         N, K = H, I
-    qa, sa = quant.per_token_group_quant_fp8(a.contiguous(), 128)
+    qa, sa = _quantize_1x128(a.contiguous())
     qb = torch.empty(E, N, K, dtype=torch.float8_e4m3fn)
     sb = torch.empty(E, -(-N // 128), -(-K // 128))
     for e in range(E):
-        q, s = quant.weight_quant_block(_block_weights(N, K, g))
+        q, s = _quantize_weight_128x128(_block_weights(N, K, g))
         qb[e], sb[e] = q, s
     return GroupedCase(f"c5_moe_{which}", qa, qb, sa, sb, indptr,
                        {"topk_ids": ids, "topk_weights": tw, "order": order, "top_k": k})
