@@ -14,7 +14,9 @@ time of K steps), with:
                 are rotated through > 512 MB so that launches do not hit the 256 MB memory-side cache)
   cpu_baseline  the torch CPU oracle (dequantize -> fp32 matmul -> bf16) timed on this host's cores
                 on a bounded sample of the same workload
-Kernel durations are measured with HIP events on the stream the kernels are launched on.
+Kernel durations are measured with HIP events on the stream the kernels are launched on.  Compute-bound
+workloads first run untimed for RAMP_MS milliseconds (see _ramp): the device needs ~30 ms under load to
+reach its steady state after idle time, and the timed K steps are meant to measure that state.
 """
 
 from __future__ import annotations
@@ -80,6 +82,24 @@ def _events_ms(fn, iters, stream):
     end.record(stream)
     torch.cuda.synchronize()
     return start.elapsed_time(end)
+
+
+RAMP_MS = 100.0
+
+
+def _ramp(fn, min_ms=RAMP_MS):
+    """Untimed: keep the device under the load of fn(i) for at least `min_ms`.  After idle time an MI355X
+    runs MFMA-bound kernels 10-20 % slower for its first ~30 ms under load (a (8192, 6144, 4096) GEMM goes
+    192 -> 157 us over ~150 back-to-back launches, and back to 190 us after two idle seconds); HBM-bound
+    launches show no such drift.  Compute-bound workloads are therefore measured after this phase, which is
+    part of the warm-up, never of the timed region."""
+    t0 = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t0) * 1e3 < min_ms:
+        for _ in range(4):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
 
 
 def _graph_ms(fn, launches, replays, stream):
@@ -154,8 +174,10 @@ def _copies_for(nbytes):
     return max(2, min(64, -(-ROTATE_BYTES // max(1, int(nbytes)))))
 
 
-def measure_shape(runner, steps, warmup, stream, use_graph):
+def measure_shape(runner, steps, warmup, stream, use_graph, ramp=False):
     from tilegym_amd import _lib
+    if ramp:
+        _ramp(runner)
     for i in range(max(1, warmup)):
         runner(i)
     torch.cuda.synchronize()
@@ -269,14 +291,15 @@ def main():
     # ------------------------------------------------------------------ prefill (headline)
     if args.workload in ("prefill", "all"):
         runners = [DenseRunner(W.llama_prefill_case(p), device, copies=2) for p in W.LLAMA_SHAPES]
-        for w in range(max(1, args.warmup)):
-            for r in runners:
-                r(w)
-        torch.cuda.synchronize()
 
         def step(i):
             for r in runners:
                 r(i)
+
+        _ramp(step)
+        for w in range(max(1, args.warmup)):
+            step(w)
+        torch.cuda.synchronize()
 
         ms = _events_ms(step, args.steps, stream)
         total_flops = sum(r.case.flops() for r in runners)
@@ -340,7 +363,7 @@ def main():
                 case = W.DenseCase(f"c4_block_M{M}_{N}x{K}", big.a[:M].contiguous(), big.b, big.scale_a[:M].contiguous(), big.scale_b, True, True)
                 r = DenseRunner(case, device, copies=_copies_for(case.algorithmic_bytes()) if M <= 64 else 2)
                 shapes.append(measure_shape(r, args.steps if M > 64 else max(args.steps, 64), args.warmup, stream,
-                                            use_graph=(M <= 64 and not args.no_graph)))
+                                            use_graph=(M <= 64 and not args.no_graph), ramp=M > 64))
                 del r
             torch.cuda.empty_cache()
         detail["block_scaled"] = shapes
@@ -348,7 +371,7 @@ def main():
         shapes = []
         for which in ("gate_up", "down"):
             r = RaggedRunner(W.moe_grouped_case(which), device, copies=2)
-            shapes.append(measure_shape(r, args.steps, args.warmup, stream, use_graph=False))
+            shapes.append(measure_shape(r, args.steps, args.warmup, stream, use_graph=False, ramp=True))
             del r
             torch.cuda.empty_cache()
         detail["moe_grouped"] = shapes
@@ -361,6 +384,7 @@ def main():
         hidden = torch.randn(T, H, device=device).to(torch.bfloat16)
         w1, w2, s1, s2 = up.b.to(device), down.b.to(device), up.b_scale.to(device), down.b_scale.to(device)
         fn = lambda i: fused_moe(hidden, w1, w2, tw, ids, w1_scale=s1, w2_scale=s2)  # noqa: E731
+        _ramp(fn)
         for w in range(max(2, args.warmup)):
             fn(w)
         n = max(args.steps, 20)
@@ -436,7 +460,8 @@ def main():
                                 "moe": "config 5: DeepSeek-V2-Lite MoE grouped GEMMs",
                                 "quant": "producers: 1x128 activation quantizer, moe_align_block_size",
                                 "all": "config 3 (headline) + configs 2, 4, 5 + producers"}[args.workload],
-                   "device": props.name, "compute_units": props.multi_processor_count},
+                   "device": props.name, "compute_units": props.multi_processor_count,
+                   "untimed_load_ramp_ms": RAMP_MS},
     }
     line.update(out)
     if not args.no_cpu_baseline:
