@@ -907,7 +907,8 @@ def test_launches_replay_from_a_hip_graph(device):
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        work()  # warm-up on the capture stream (workspace allocation happens here, not under capture)
+        work()  # warm-up on a side stream; torch.cuda.graph captures on a stream of its own, so the workspace of the
+        # captured split-K GEMM is allocated under capture, from the graph's pool (see _lib.workspace_for)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
@@ -922,6 +923,40 @@ def test_launches_replay_from_a_hip_graph(device):
         torch.cuda.synchronize()
         assert torch.equal(g_moe, eager_moe), f"MoE layer differs on replay {rep}"
         assert torch.equal(g_mm, eager_mm), f"split-K GEMM differs on replay {rep}"
+
+
+def test_graph_workspace_survives_a_larger_eager_gemm(device):
+    """A captured split-K GEMM keeps writing its partial sums to the workspace it was captured with.  A later,
+    larger GEMM on the same stream makes the binding allocate a bigger workspace: the captured one must stay
+    alive (never returned to the allocator), so that tensors allocated afterwards cannot land in it and be
+    overwritten by a replay."""
+    g = _g(41)
+    a = fp8_randn((16, 14336), g).to(device)
+    b = fp8_randn((4096, 14336), g, 0.05).to(device)
+    one = torch.ones(1, device=device)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        eager = matmul(a, b, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        assert _lib.last_config()["SPLIT_K"] > 1
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = matmul(a, b, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        # a larger split-K problem on the same stream: the binding has to grow that stream's workspace
+        a2 = fp8_randn((64, 14336), g).to(device)
+        big = matmul(a2, b, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        assert _lib.last_config()["SPLIT_K"] > 1
+        torch.cuda.synchronize()
+        # fill freshly allocated memory with a pattern, replay, and check that neither side was disturbed
+        fresh = [torch.full((1 << 20,), 3, dtype=torch.int32, device=device) for _ in range(16)]
+        for rep in range(3):
+            captured.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(captured, eager), f"replay {rep} differs"
+            assert all(int(t.min()) == 3 and int(t.max()) == 3 for t in fresh), "a replay wrote into memory it no longer owns"
+        del big
 
 
 def test_fused_moe_more_tokens_than_one_chunk(device):

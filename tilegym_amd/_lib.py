@@ -180,20 +180,32 @@ def last_config() -> Dict[str, int]:
 
 
 # ---------------------------------------------------------------------------- workspaces
-_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+# (device, stream handle, under capture?) -> every scratch tensor ever handed out for that key, newest last.
+# tg_fp8_gemm bakes the raw workspace pointer into whatever it enqueues, and a HIP graph captured from such
+# a call keeps writing split-K partial sums there on every replay; a buffer that is replaced by a larger
+# one is therefore kept alive for the life of the process instead of going back to the allocator (where
+# another tensor could receive the block while a graph still writes to it).  Buffers at least double, so a
+# key holds a handful.
+_workspaces: Dict[Tuple[int, int, bool], list] = {}
+_WS_MIN_BYTES = 1 << 20
 
 
 def workspace_for(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
-    """Scratch buffer for the current stream of ``device`` (grown on demand).  One buffer per
-    (device, stream): calls on one stream are ordered, so they can share it."""
+    """Scratch buffer for the current stream of ``device`` (grown on demand, never freed).  One live buffer
+    per (device, stream): calls on one stream are ordered, so they can share it.  Calls made while the
+    stream is being captured get buffers of their own (allocated from the capturing graph's pool and kept
+    alive here too), so eager calls and graph replays never share scratch memory."""
     if nbytes <= 0:
         return None
     stream = torch.cuda.current_stream(device)
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (index, stream.cuda_stream, bool(torch.cuda.is_current_stream_capturing()))
+    held = _workspaces.setdefault(key, [])
+    if held and held[-1].numel() >= nbytes:
+        return held[-1]
+    size = max(int(nbytes), _WS_MIN_BYTES, 2 * held[-1].numel() if held else 0)
+    ws = torch.empty(size, dtype=torch.uint8, device=device)
+    held.append(ws)
     return ws
 
 
