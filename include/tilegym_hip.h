@@ -95,6 +95,24 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
                     int32_t trans_b, float alpha, float beta, const tg_tensor* workspace,
                     const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream);
 
+/*
+ * tg_fp8_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, schedules
+ * and results as tg_fp8_gemm, without the workspace argument: split-K partial sums and the K-contiguous copy of
+ * a (K,N) weight go to a TG_STATIC_SCRATCH_BYTES array inside the library's device image (one copy per GPU,
+ * held until the process ends).  The call allocates nothing and frees nothing.  A problem whose schedule needs
+ * more scratch than the array holds returns TG_ERR_INVALID (the text says how much): call tg_fp8_gemm with a
+ * caller-owned workspace for it.  All calls on one GPU share that GPU's array, whatever the stream: calls that
+ * overlap in time on one GPU race on it; calls on one stream never overlap.  Nothing in the array needs to start
+ * at zero (no atomics are used), so nothing is cleared between calls.  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress); make that call outside graph capture.
+ */
+#define TG_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
+int32_t tg_fp8_gemm_static_scratch(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                                   const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
+                                   int32_t trans_b, float alpha, float beta, const int32_t* cfg, int32_t ncfg,
+                                   int32_t device_id, uint64_t hip_stream);
+
 /* Bytes of workspace that let tg_fp8_gemm use every schedule for this problem
  * (trans_b == 0 adds room for a K-contiguous copy of B).  Never fails; returns 0 for
  * non-positive sizes. */

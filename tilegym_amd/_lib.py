@@ -95,6 +95,9 @@ def load():
     L.tg_fp8_gemm.restype = ctypes.c_int32
     L.tg_fp8_gemm.argtypes = [P, P, P, P, P, ctypes.c_int32, ctypes.c_int32, ctypes.c_float,
                               ctypes.c_float, P, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_gemm_static_scratch.restype = ctypes.c_int32
+    L.tg_fp8_gemm_static_scratch.argtypes = [P, P, P, P, P, ctypes.c_int32, ctypes.c_int32, ctypes.c_float,
+                                             ctypes.c_float, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     L.tg_fp8_ragged_gemm.restype = ctypes.c_int32
     L.tg_fp8_ragged_gemm.argtypes = [P, P, P, P, P, P, I32P, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     L.tg_fp8_moe_gemm.restype = ctypes.c_int32
@@ -242,6 +245,23 @@ def fp8_gemm(c, a, b, scale_a=None, scale_b=None, trans_a=False, trans_b=True, a
                        int(bool(trans_b)), float(alpha), float(beta), _ref(dws), cfg, ncfg, dev,
                        _stream_handle(a))
     check_rc(rc, "tg_fp8_gemm")
+
+
+STATIC_SCRATCH_BYTES = 32 * 1024 * 1024
+
+
+def fp8_gemm_static_scratch(c, a, b, scale_a=None, scale_b=None, trans_a=False, trans_b=True, alpha=1.0, beta=0.0,
+                            kernel_configs=None) -> None:
+    """tg_fp8_gemm_static_scratch: tg_fp8_gemm whose scratch is an array inside the library (no allocation
+    anywhere on the way; problems that need more than STATIC_SCRATCH_BYTES raise)."""
+    L = load()
+    dev = _device_index(a)
+    cfg, ncfg = make_cfg(kernel_configs)
+    dc, da, db = make_tensor_desc(c), make_tensor_desc(a), make_tensor_desc(b)
+    dsa, dsb = make_tensor_desc(scale_a), make_tensor_desc(scale_b)
+    rc = L.tg_fp8_gemm_static_scratch(_ref(dc), _ref(da), _ref(db), _ref(dsa), _ref(dsb), int(bool(trans_a)),
+                                      int(bool(trans_b)), float(alpha), float(beta), cfg, ncfg, dev, _stream_handle(a))
+    check_rc(rc, "tg_fp8_gemm_static_scratch")
 
 
 def fp8_ragged_gemm(c, a, b, a_scale, b_scale, m_indptr, kernel_configs=None) -> None:

@@ -4,9 +4,15 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/tilegym_hip.h"
 #include "tg_host.h"
+
+// Scratch memory of tg_fp8_gemm_static_scratch: one copy per device the library is loaded on, held until
+// the process ends.  In host code this name is only a handle for hipGetSymbolAddress; the device address
+// is looked up once per device (scratch_address below) and that pointer is what kernels receive.
+static __device__ __align__(256) unsigned char scratch[TG_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -107,6 +113,24 @@ int compute_units(int dev) {
         cached[dev] = n;
     }
     return cached[dev];
+}
+
+// Device address of `scratch` on device `dev`, which must be the current device.  Looked up on the first
+// call per device and kept; every device holds its own copy of the array at its own address.
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[64] = {nullptr};
+hipError_t scratch_address(int dev, uint8_t** out) {
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) { (void)hipGetLastError(); return e; }
+        if (!ptr) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = reinterpret_cast<uint8_t*>(g_scratch_ptr[dev]);
+    return hipSuccess;
 }
 
 struct Schedule {
@@ -270,6 +294,14 @@ struct Resolved {
     const float* Bs;
 };
 
+// Body of tg_fp8_gemm and tg_fp8_gemm_static_scratch.  static_scratch: the workspace is the library's
+// own `scratch` array instead of a caller's buffer, and a problem whose schedule needs more than it holds
+// is rejected instead of run with a smaller split.
+int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b, const tg_tensor* scale_a,
+                      const tg_tensor* scale_b, int32_t trans_a, int32_t trans_b, float alpha, float beta,
+                      const tg_tensor* workspace, bool static_scratch, const int32_t* cfg, int32_t ncfg,
+                      int32_t device_id, uint64_t hip_stream);
+
 }  // namespace
 
 extern "C" {
@@ -316,6 +348,26 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
                     const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
                     int32_t trans_b, float alpha, float beta, const tg_tensor* workspace,
                     const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream) {
+    return fp8_gemm_impl(c, a, b, scale_a, scale_b, trans_a, trans_b, alpha, beta, workspace, false, cfg, ncfg,
+                         device_id, hip_stream);
+}
+
+int32_t tg_fp8_gemm_static_scratch(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
+                                   const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
+                                   int32_t trans_b, float alpha, float beta, const int32_t* cfg, int32_t ncfg,
+                                   int32_t device_id, uint64_t hip_stream) {
+    return fp8_gemm_impl(c, a, b, scale_a, scale_b, trans_a, trans_b, alpha, beta, nullptr, true, cfg, ncfg,
+                         device_id, hip_stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b, const tg_tensor* scale_a,
+                      const tg_tensor* scale_b, int32_t trans_a, int32_t trans_b, float alpha, float beta,
+                      const tg_tensor* workspace, bool static_scratch, const int32_t* cfg, int32_t ncfg,
+                      int32_t device_id, uint64_t hip_stream) {
     g_err[0] = 0;
     int32_t rc;
     if ((rc = check_tensor(a, "a", 2)) || (rc = check_tensor(b, "b", 2)) || (rc = check_tensor(c, "c", 2))) return rc;
@@ -363,8 +415,17 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
 
     // ---- workspace carving: [split-K partial sums ...][optional K-contiguous copy of B]
-    const int64_t ws_bytes = workspace ? numel(workspace) * elem_size(workspace->dtype) : 0;
+    int64_t ws_bytes = workspace ? numel(workspace) * elem_size(workspace->dtype) : 0;
     uint8_t* ws = workspace ? reinterpret_cast<uint8_t*>(workspace->ptr) : nullptr;
+    if (static_scratch) {
+        const hipError_t e = scratch_address(device_id, &ws);
+        if (e != hipSuccess) return fail(TG_ERR_DEVICE, "cannot locate the static scratch buffer on device %d: %s", device_id, hipGetErrorString(e));
+        ws_bytes = TG_STATIC_SCRATCH_BYTES;
+        const int64_t copy_bytes = (!trans_b && !trans_a && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0) ? (N * K + 255) / 256 * 256 : 0;
+        if (copy_bytes > ws_bytes)
+            return fail(TG_ERR_INVALID, "the K-contiguous copy of a (K,N) weight needs %lld bytes, the static scratch buffer holds %lld: "
+                        "pass b as (N,K) with trans_b=1 or call tg_fp8_gemm with a workspace", (long long)copy_bytes, (long long)ws_bytes);
+    }
     int64_t ws_free = ws_bytes;
     uint8_t* ws_cursor = ws;
 
@@ -392,6 +453,14 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
     const bool pipe_ok = !block_scaled && beta == 0.0f && (K % 128) == 0 &&
                          (out_type == tg::OUT_BF16 || out_type == tg::OUT_F16);
     Schedule s = choose_dense(M, N, K, block_scaled, fast_layout, pipe_ok, cfg, ncfg, ws_free);
+    if (static_scratch) {
+        // same schedule as tg_fp8_gemm with a full-size workspace, or an error: never a silently smaller split
+        const Schedule full = choose_dense(M, N, K, block_scaled, fast_layout, pipe_ok, cfg, ncfg, INT64_MAX / 2);
+        if (full.split_k != s.split_k)
+            return fail(TG_ERR_INVALID, "split-K %d of this problem needs %lld bytes of partial sums, the static scratch buffer has %lld free: "
+                        "call tg_fp8_gemm with a workspace, or force a smaller SPLIT_K", full.split_k,
+                        (long long)full.split_k * M * N * 4, (long long)ws_free);
+    }
 
     tg::GemmParams p{};
     p.A = reinterpret_cast<const uint8_t*>(a->ptr);
@@ -484,6 +553,10 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
     }
     return TG_OK;
 }
+
+}  // namespace
+
+extern "C" {
 
 // Shared validation of the two grouped entry points.
 static int32_t grouped_common(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
