@@ -1,0 +1,208 @@
+// 256x256 per-tensor tile with a hand-ordered K loop (prefill shapes): C[m,n] = sum_k A[m,k] * B[n,k].
+//
+// Same tile, wave grid (4 x 2 waves, 64 x 128 per wave), slab layout, swizzles, fragment addressing,
+// per-accumulator MFMA order and epilogue arithmetic as
+// fp8_gemm_tile_kernel<256, 256, 4, 2, false, GROUP_DENSE, false>: identical results.  What differs is
+// the schedule of one K step.  In the generic kernel four loader waves issue their sixteen direct
+// loads in two bursts of eight; while a wave waits for room in the address path (about 14 clocks per
+// 1 KiB load for the whole compute unit, whoever issues it) it issues no MFMAs, so a loader wave needs
+// load time PLUS its 1024 clocks of MFMA issue per step and the step lasts ~2.6 k clocks instead of
+// the 2048 the matrix pipe needs.  Here
+//   * all eight waves load (eight 1 KiB loads per wave and step), one load behind every group of
+//     four MFMAs: the address path sees one request per ~32 clocks and never backs up;
+//   * two activation slabs and three weight slabs (160 KiB, all of LDS) let one barrier per step do:
+//     a step requests B(k+2) between its first MFMAs and, after its barrier, A(k+2), always into slabs
+//     nobody reads any more.  The weights get the long lead (1.25 - 2 steps): on the big projections
+//     they stream from HBM, while the activation panel of a tile row is re-read by every tile of that
+//     row and sits in the L2 / memory-side cache (measured on 8192 x 28672 x 4096: 2950 clocks per step
+//     with the three slabs on the activation side, 2430 this way; 2270 when nothing misses);
+//   * the barrier sits in front of the last eight MFMAs of a step, which are ordered by row group so
+//     that the activation fragments of step k+1 are read into the registers those MFMAs release:
+//     the matrix pipe has work while the fragment reads of the next step are in flight.
+// The order is pinned with scheduling fences: the direct loads are inline assembly (see
+// direct_load_b128), which the compiler's own interleaving hints cannot see.
+#pragma once
+
+#include "fp8_gemm_tile.h"
+
+namespace tg {
+
+__global__ void __launch_bounds__(512, 1) fp8_gemm_tile256_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int BM = 256, BN = 256, WGM = 4, WGN = 2, NW = 8;
+    constexpr int WTN = BN / WGN;                 // 128 columns per wave
+    constexpr int TM = 4, TN = WTN / 16;          // 4 row groups x 8 column tiles per wave
+    constexpr int SLAB = 256 * kKBlock;           // 32 KiB
+    constexpr int A_STAGES = 2, B_STAGES = 3;
+    constexpr int IT = 256 / (8 * NW);            // 4 loads per wave, slab and step
+    static_assert(TN == 8 && IT == 4, "schedule below is written for 8 column tiles and 4 + 4 loads");
+
+    __shared__ __align__(1024) uint8_t sA[A_STAGES * SLAB];
+    __shared__ __align__(1024) uint8_t sB[B_STAGES * SLAB];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int K = p.K;
+    const int tiles_n = (p.N + BN - 1) / BN, tiles_m = (p.M + BM - 1) / BM;
+    const int pid = xcd_remap((int)blockIdx.x, tiles_m * tiles_n);
+    constexpr int GM = 8;
+    const int width = GM * tiles_n;
+    const int group = pid / width, first_m = group * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    const int tile_m = first_m + (pid % width) % gsz, tile_n = (pid % width) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int rows_valid = min(BM, p.M - m0);
+    const int nsteps = p.kblocks, last = nsteps - 1;
+
+    // ---- direct loads: pass i of wave w fills slab rows 8*(i*8 + w) .. +7 (lane l: row + l/8, chunk position l%8)
+    const int lrow = lane >> 3;
+    const int lj = (lane & 7) ^ swz16(lrow);
+    const int ljb = (lane & 7) ^ swz_w(((wave & 1) << 3) | lrow);
+    uint32_t a_off[IT], b_off[IT];
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int r = (i * NW + wave) * 8 + lrow;
+        a_off[i] = (uint32_t)(m0 + min(r, rows_valid - 1)) * (uint32_t)K + lj * 16;
+        b_off[i] = (uint32_t)min(n0 + r, p.N - 1) * (uint32_t)K + ljb * 16;
+    }
+    const v4i rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(p.B);
+    const uint32_t ldsA = lds_address(sA) + wave * 1024, ldsB = lds_address(sB) + wave * 1024;
+    auto load_a = [&](int i, int kstep, int stage) {
+        direct_load_b128(rsrc_a, ldsA + stage * SLAB + i * NW * 1024, a_off[i], min(kstep, last) * kKBlock);
+    };
+    auto load_b = [&](int i, int kstep, int stage) {
+        direct_load_b128(rsrc_b, ldsB + stage * SLAB + i * NW * 1024, b_off[i], min(kstep, last) * kKBlock);
+    };
+
+    // ---- fragment addresses (see fp8_gemm_tile.h)
+    const int li = lane & 15, lg = lane >> 4;
+    const uint32_t frag0 = wm * 16 * kKBlock + li * kKBlock + ((lg ^ swz16(li)) << 4), frag1 = frag0 ^ 64;
+    const int wrow = ((li >> 2) << 3) | (li & 3);
+    const uint32_t wfrag0 = wn * WTN * kKBlock + wrow * kKBlock + ((lg ^ swz_w(wrow)) << 4), wfrag1 = wfrag0 ^ 64;
+    auto read_a = [&](int tm, const uint8_t* cA) {
+        const uint8_t* base = cA + tm * (WGM * 16 * kKBlock);
+        return join(*reinterpret_cast<const v4i*>(base + frag0), *reinterpret_cast<const v4i*>(base + frag1));
+    };
+    auto read_w = [&](int tn, const uint8_t* cB) {
+        const uint8_t* base = cB + ((tn >> 1) * 32 + (tn & 1) * 4) * kKBlock;
+        return join(*reinterpret_cast<const v4i*>(base + wfrag0), *reinterpret_cast<const v4i*>(base + wfrag1));
+    };
+
+    v4f acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    constexpr int kWaitBut8 = 0x0F70 | 8, kWaitBut4 = 0x0F70 | 4, kWaitAll = 0x0F70;
+    constexpr int kWaitLds = 0xC07F;  // lgkmcnt(0)
+#define TG_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+    // ---- prologue: A(0), B(0), B(1), A(1); the first two must have landed
+#pragma unroll
+    for (int i = 0; i < IT; ++i) load_a(i, 0, 0);
+#pragma unroll
+    for (int i = 0; i < IT; ++i) load_b(i, 0, 0);
+#pragma unroll
+    for (int i = 0; i < IT; ++i) load_b(i, 1, 1);
+#pragma unroll
+    for (int i = 0; i < IT; ++i) load_a(i, 1, 1);
+    __builtin_amdgcn_s_waitcnt(kWaitBut8);   // B(1), A(1) may be in flight
+    __builtin_amdgcn_s_barrier();
+    v8i af[TM], wf[4];
+    wf[0] = read_w(0, sB);
+    wf[1] = read_w(1, sB);
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) af[tm] = read_a(tm, sA);
+
+    // ---- main loop.  On entry to step k: A(k) and B(k) are in LDS and visible to every wave; the reads of af (fragments
+    // of A(k)) and wf[0], wf[1] (column tiles 0, 1 of B(k)) are issued; B(k+1) and A(k+1) are requested.
+    // Requests of a wave in order: ... B(k+1) x4 | A(k+1) x4 | B(k+2) x4 |: at the wait of step k all but the last four
+    // have landed, i.e. B(k+1) and A(k+1).
+    int sa = 0, sb = 0;  // slabs that hold A(k) and B(k)
+    for (int k = 0; k < nsteps; ++k) {
+        const int sa1 = sa ^ 1;                              // holds/receives A(k+1)
+        const int sb1 = sb == B_STAGES - 1 ? 0 : sb + 1;     // holds B(k+1)
+        const int sb2 = sb1 == B_STAGES - 1 ? 0 : sb1 + 1;   // receives B(k+2)  (free: held B(k-1))
+        const uint8_t* cB = sB + sb * SLAB;
+        TG_FENCE();
+        // column tiles 0 .. 5: four MFMAs, one direct load (B(k+2) goes to the slab B(k-1) had), the weight fragment of
+        // the column tile after next
+#pragma unroll
+        for (int tn = 0; tn < 6; ++tn) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_e4m3(wf[tn & 3], af[tm], acc[tn][tm]);
+            TG_FENCE();
+            if (tn < 4) load_b(tn, k + 2, sb2);
+            wf[(tn + 2) & 3] = read_w(tn + 2, cB);
+            TG_FENCE();
+        }
+        // B(k+1) and A(k+1) have landed (all but the four requests of B(k+2)); all my reads of B(k) are done
+        __builtin_amdgcn_s_waitcnt(kWaitBut4);
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+        __builtin_amdgcn_s_barrier();
+        TG_FENCE();
+        // column tiles 6 and 7 by row group: each pair of MFMAs releases one activation fragment, which is refilled from
+        // A(k+1) at once; the first two weight fragments of step k+1 are read first.  A(k)'s slab is free (every wave
+        // read its fragments before this barrier) and receives A(k+2).
+        const uint8_t* nA = sA + sa1 * SLAB;
+        const uint8_t* nB = sB + sb1 * SLAB;
+        wf[0] = read_w(0, nB);
+        wf[1] = read_w(1, nB);
+        TG_FENCE();
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+            acc[6][tm] = mfma_e4m3(wf[2], af[tm], acc[6][tm]);
+            acc[7][tm] = mfma_e4m3(wf[3], af[tm], acc[7][tm]);
+            TG_FENCE();
+            af[tm] = read_a(tm, nA);
+            load_a(tm, k + 2, sa);
+            TG_FENCE();
+        }
+        sa = sa1;
+        sb = sb1;
+    }
+#undef TG_FENCE
+    __builtin_amdgcn_s_waitcnt(kWaitAll);  // the re-fetches past the end must land before the workgroup's LDS is released
+    // the fragment reads issued for the step after the last one are never used; keep the compiler from deleting the
+    // loop-carried registers' last assignment in a way that changes the loop body
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) asm volatile("" : : "v"(af[tm]));
+    asm volatile("" : : "v"(wf[0]), "v"(wf[1]));
+
+    // ---- epilogue, straight from the accumulators (as fp8_gemm_tile.h)
+    float scale = p.alpha;
+    if (p.As) scale *= p.As[0];
+    if (p.Bs) scale *= p.Bs[0];
+    const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;
+    int dsts[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+        const int rt = (tm * WGM + wm) * 16 + li;
+        dsts[tm] = rt < rows_valid ? m0 + rt : -1;
+    }
+    auto emit = [&](auto type_tag) {
+        constexpr int OT = decltype(type_tag)::value;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+            for (int tp = 0; tp < TN / 2; ++tp) {
+                const int col = n0 + wn * WTN + tp * 32 + lg * 8;
+                if (dsts[tm] < 0 || col >= p.N) continue;
+                store8(p.C, OT, dsts[tm], col, p.N, acc[2 * tp][tm] * scale, acc[2 * tp + 1][tm] * scale, p.beta, vec_ok);
+            }
+        }
+    };
+    if (p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
+    else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
+    else emit(std::integral_constant<int, OUT_F16>{});
+#endif
+}
+
+inline hipError_t launch_tile256(const GemmParams& p, int grid_x, hipStream_t stream) {
+    hipLaunchKernelGGL(fp8_gemm_tile256_kernel, dim3(grid_x, 1, 1), dim3(512, 1, 1), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace tg

@@ -543,7 +543,11 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         }
         const bool split = pc.split_k > 1;
         const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128;
+        // hand-ordered K loop for the dense per-tensor 256x256 tile (WAVES = 4 asks for the generic form with four loader waves)
+        const bool ordered = s.kernel == 1 && !block_scaled && !split && s.bm == 256 && s.bn == 256 &&
+                             cfg_get(cfg, ncfg, TG_CFG_WAVES) != 4;
         hipError_t e = s.kernel == 4 ? tg::run_pipe(8, s.waves, pc, gx, stream)
+                     : ordered ? tg::run_tile256(pc, gx, stream)
                      : deep ? tg::run_tile_deep(split, pc, gx, pc.split_k, stream)
                      : block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
                                     : tg::run_tile_per_tensor(s.bm, s.bn, split, pc, gx, pc.split_k, stream);
