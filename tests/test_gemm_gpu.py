@@ -141,6 +141,32 @@ def test_per_tensor_stream(device, M, N, K, split):
     check(out, ref, what=f"stream M={M} N={N} K={K} split={split}")
 
 
+@pytest.mark.parametrize("M", [1, 5, 8, 16])
+@pytest.mark.parametrize("N,K", [(1000, 1024), (520, 14336), (264, 2064), (256, 9216), (72, 512)])
+def test_per_tensor_stream_eight_waves(device, M, N, K):
+    """The streaming kernel with eight waves per workgroup splitting K (long K over few weight rows, one launch):
+    more waves than 1 KiB pieces, K tails inside a piece, ragged N."""
+    g = _g(M * 17 + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
+    ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "stream", "WAVES": 8})
+    cfg = used("stream")
+    assert cfg["WAVES"] == 8 and cfg["SPLIT_K"] == 1
+    check(out, ref, what=f"stream 8 waves M={M} N={N} K={K}")
+
+
+def test_stream_eight_waves_is_the_default_for_long_k_few_rows(device):
+    g = _g(5)
+    a, b = fp8_randn((4, 14336), g), fp8_randn((4096, 14336), g, 0.02)
+    ref = R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
+    cfg = used("stream")
+    assert cfg["WAVES"] == 8 and cfg["SPLIT_K"] == 1, cfg
+    check(out, ref, what="down projection, M=4")
+
+
 @pytest.mark.parametrize("M", [1, 3, 8, 16])
 @pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 1), (264, 2064, 1), (128, 16384, 4), (72, 512, 1), (4096, 3072, 2)])
 def test_per_tensor_stream_wide(device, M, N, K, split):

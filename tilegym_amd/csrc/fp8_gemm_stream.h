@@ -19,10 +19,9 @@ namespace tg {
 
 constexpr int kStreamChunk = 1024;  // bytes of one row fetched by one load instruction
 
-template <int MT, int NBUF, bool BLOCKSCALE>
-__global__ void __launch_bounds__(256) fp8_gemm_stream_kernel(const GemmParams p) {
+template <int MT, int NBUF, bool BLOCKSCALE, int NW = 4>
+__global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    constexpr int NW = 4;
     constexpr int BUF = 16 * kStreamChunk;
     __shared__ __align__(1024) uint8_t sW[NW * NBUF * BUF];
 
@@ -353,10 +352,10 @@ inline hipError_t launch_stream_wide(const GemmParams& p, int grid_x, int grid_y
     return hipGetLastError();
 }
 
-template <int MT, int NBUF, bool BLOCKSCALE>
+template <int MT, int NBUF, bool BLOCKSCALE, int NW = 4>
 inline hipError_t launch_stream(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
-    auto kern = fp8_gemm_stream_kernel<MT, NBUF, BLOCKSCALE>;
-    hipLaunchKernelGGL(kern, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
+    auto kern = fp8_gemm_stream_kernel<MT, NBUF, BLOCKSCALE, NW>;
+    hipLaunchKernelGGL(kern, dim3(grid_x, grid_y, 1), dim3(64 * NW, 1, 1), 0, stream, p);
     return hipGetLastError();
 }
 

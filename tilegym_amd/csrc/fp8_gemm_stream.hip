@@ -4,7 +4,10 @@
 
 namespace tg {
 
-hipError_t run_stream(int mt, int nbuf, bool bs, const GemmParams& p, int gx, int gy, hipStream_t s) {
+hipError_t run_stream(int mt, int nbuf, int waves, bool bs, const GemmParams& p, int gx, int gy, hipStream_t s) {
+    // eight waves per workgroup (one 16 KiB buffer each, one workgroup per compute unit): long K over few weight rows
+    if (waves == 8 && mt == 1 && nbuf == 1)
+        return bs ? launch_stream<1, 1, true, 8>(p, gx, gy, s) : launch_stream<1, 1, false, 8>(p, gx, gy, s);
 #define TG_CASE(MT, NBUF)                                                   \
     if (mt == MT && nbuf == NBUF)                                           \
         return bs ? launch_stream<MT, NBUF, true>(p, gx, gy, s) : launch_stream<MT, NBUF, false>(p, gx, gy, s);

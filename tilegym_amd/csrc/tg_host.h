@@ -33,7 +33,7 @@ hipError_t run_tile_list(int bm, int bn, const GemmList& gl, int gx, hipStream_t
 // register-pipelined 256x256 tile: per-tensor scales, dense, beta == 0, bf16/f16 output, K % 128 == 0
 hipError_t run_pipe(int waves, int loaders, const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_skinny(int mt, int rg, int nw, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
-hipError_t run_stream(int mt, int nbuf, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
+hipError_t run_stream(int mt, int nbuf, int waves, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
 // 64 weight rows per workgroup, activation piece shared through LDS: M <= 16
 hipError_t run_stream_wide(bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
 // C <- epilogue(sum_z partials[z]) for the split-K schedules (fixed z order: bit-reproducible)

@@ -205,6 +205,14 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         int64_t wide_split = cdiv(448, wide_wgs);
         if (wide_split > pieces) wide_split = pieces;
         const bool wide_auto = N >= 16384 || (N * K >= ((int64_t)48 << 20) && wide_wgs * wide_split >= 320);
+        // long K over few weight rows (at most ~one 16-row workgroup per compute unit): eight waves split K inside the
+        // workgroup, one launch, no partial sums (4096 x 14336: 12.4 / 14.3 us at M = 1 / 8 against 14.1 / 14.8 for the
+        // wide form with split-K and its reduction; at M = 16 every wave's own activation loads make it lose, 17.0 vs 15.4)
+        const int want_waves = cfg_get(cfg, ncfg, TG_CFG_WAVES);
+        if (want_rg != 4 && want_split <= 1 && ((want_waves == 8 && M <= 16) || (want_waves < 0 && want_rg < 0 && M <= 8 && pieces >= 8 && wgs <= 320))) {
+            s.waves = 8;
+            return s;
+        }
         if (M <= 16 && (want_rg == 4 || (want_rg < 0 && wide_auto))) {
             s.row_groups = 4;
             if (want_split > 1) s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, want_split);
@@ -508,9 +516,9 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         // measured: one 16 KiB buffer per wave and two workgroups per compute unit beat two buffers and
         // one workgroup, except for long K where they tie
         if (nbuf != 1 && nbuf != 2) nbuf = (per_wave >= 3 && s.mt == 1 && !block_scaled) ? 2 : 1;
-        if (s.mt != 1) nbuf = 1;
+        if (s.mt != 1 || s.waves == 8) nbuf = 1;
         hipError_t e = s.row_groups == 4 ? tg::run_stream_wide(block_scaled, p, (int)cdiv(N, 64), s.split_k, stream)
-                                         : tg::run_stream(s.mt, nbuf, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
+                                         : tg::run_stream(s.mt, nbuf, s.waves, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "stream kernel launch failed: %s", hipGetErrorString(e));
         if (s.split_k > 1 && tg::run_splitk_reduce(p, block_scaled, stream) != hipSuccess)
             return fail(TG_ERR_LAUNCH, "split-K reduction launch failed");
