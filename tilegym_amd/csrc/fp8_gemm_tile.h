@@ -191,47 +191,6 @@ __device__ __forceinline__ void store8(void* C, int out_type, int64_t row, int c
     }
 }
 
-// Instruction-order hint for one K step of a wave: the LDS fragment reads and the direct
-// global->LDS loads of the next stage are spread between the MFMAs instead of being issued in
-// bursts (all waves of a workgroup run in phase, so a burst of memory instructions leaves the
-// matrix pipe idle).  Order requested from the scheduler: the reads of the first two column
-// tiles, then per column tile: TM MFMAs, a share of the direct loads, the two reads of the column
-// tile after next.
-#define TG_SGB_MFMA 0x008
-#define TG_SGB_VMEM_READ 0x020
-#define TG_SGB_DS_READ 0x100
-template <int TM, int TN, int LOADS>
-__device__ __forceinline__ void pipeline_hint() {
-    constexpr int PER = (LOADS + TN - 1) / TN;  // direct loads issued per column tile
-    __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 4, 0);  // wf[0], wf[1]
-#define TG_GROUP(i)                                                                         \
-    if constexpr (TN > (i)) {                                                                \
-        __builtin_amdgcn_sched_group_barrier(TG_SGB_MFMA, TM, 0);                            \
-        if constexpr ((i) * PER < LOADS)                                                     \
-            __builtin_amdgcn_sched_group_barrier(TG_SGB_VMEM_READ, PER, 0);                  \
-        if constexpr ((i) + 2 < TN) __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 2, 0); \
-    }
-    TG_GROUP(0) TG_GROUP(1) TG_GROUP(2) TG_GROUP(3) TG_GROUP(4) TG_GROUP(5) TG_GROUP(6) TG_GROUP(7)
-#undef TG_GROUP
-}
-
-// Block-scaled variant: after the MFMAs of a column tile, the 4*TM multiply-adds that fold the
-// previous column tile's products into the accumulators.
-#define TG_SGB_VALU 0x002
-template <int TM, int TN, int LOADS>
-__device__ __forceinline__ void pipeline_hint_scaled() {
-    __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 4, 0);
-#define TG_GROUP(i)                                                                         \
-    if constexpr (TN > (i)) {                                                                \
-        __builtin_amdgcn_sched_group_barrier(TG_SGB_MFMA, TM, 0);                            \
-        if constexpr ((i) > 0) __builtin_amdgcn_sched_group_barrier(TG_SGB_VALU, 4 * TM, 0); \
-        if constexpr ((i) + 2 < TN) __builtin_amdgcn_sched_group_barrier(TG_SGB_DS_READ, 2, 0); \
-    }
-    TG_GROUP(0) TG_GROUP(1) TG_GROUP(2) TG_GROUP(3) TG_GROUP(4) TG_GROUP(5) TG_GROUP(6) TG_GROUP(7)
-#undef TG_GROUP
-    __builtin_amdgcn_sched_group_barrier(TG_SGB_VALU, 4 * TM, 0);
-}
-
 // Body of the tiled kernel for workgroup `bid` of problem `p` (the kernels below only differ in
 // how a workgroup finds its problem).
 template <int BM, int BN, int WGM, int WGN, bool BLOCKSCALE, int GROUP, bool SPLIT>
@@ -241,7 +200,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     constexpr int NW = WGM * WGN;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 16, TN = WTN / 16;
-    constexpr int NL = NW == 8 ? 4 : NW;  // waves that issue the direct global->LDS loads
+    constexpr int NL = NW;                // every wave issues its share of the direct global->LDS loads
     constexpr int RPP = 8 * NL;           // slab rows filled per pass of the loader waves
     constexpr int A_IT = BM / RPP, B_IT = BN / RPP;
     static_assert(NW == 4 || NW == 8, "wave grid");
@@ -338,7 +297,6 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // NL is even, so bit 3 of the row is the parity of the loader wave.
     const int ljb = (lane & 7) ^ swz_w(((wave & 1) << 3) | lrow);
     // (with NL == NW every wave loads: no test, and so no branch inside the K loop)
-    const bool loader = NL == NW || wave < NL;
     uint32_t b_off[B_IT];
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
@@ -350,16 +308,16 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
         b_off[i] = (uint32_t)n * (uint32_t)K + ljb * 16;
     }
     const v4i rsrc_b = make_rsrc(Bbase);
-    auto issue_b = [&](int kstep, uint8_t* dB) {
-        if (!loader) return;
+    auto issue_b1 = [&](int i, int kstep, uint8_t* dB) {  // piece i of this wave's share of a weight slab
         const int k0 = kstep * kKBlock;
         const uint32_t dst = lds_address(dB) + wave * 1024;
+        // the 64-row tile serves M <= 64: one row tile, every weight byte is read once
+        if constexpr (BM == 64) direct_load_b128_nt(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
+        else direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
+    };
+    auto issue_b = [&](int kstep, uint8_t* dB) {
 #pragma unroll
-        for (int i = 0; i < B_IT; ++i) {
-            // the 64-row tile serves M <= 64: one row tile, every weight byte is read once
-            if constexpr (BM == 64) direct_load_b128_nt(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
-            else direct_load_b128(rsrc_b, dst + i * NL * 1024, b_off[i], k0);
-        }
+        for (int i = 0; i < B_IT; ++i) issue_b1(i, kstep, dB);
     };
     issue_b(ks, sB0);
 
@@ -403,9 +361,10 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     if constexpr (BLOCKSCALE || GROUP != GROUP_DENSE) __syncthreads();
 
     // ---------------------------------------------------------------- loader set-up
-    // The first NL waves of the workgroup issue every direct load (one loader per SIMD when there
-    // are two waves per SIMD: while a loader waits for room in the memory pipeline, the other
-    // wave of its SIMD keeps the matrix pipe fed).  Pass i of loader w fills the 8-row group
+    // Every wave issues its share of the direct loads, one or two behind each column tile's MFMAs (see the
+    // main loop): the address path takes ~14 clocks per 1 KiB load for the whole compute unit, whoever
+    // issues it, and a wave that waits for room there issues no MFMAs, so bursts of loads from a few
+    // loader waves put load time and MFMA time of those waves in series.  Pass i of wave w fills the 8-row group
     // g = i*NL + w: lane l lands at row 8g + l/8, chunk position l%8, and therefore fetches
     // logical chunk (l%8) ^ swz16(row) = (l%8) ^ (l/8).
     const int lj = (lane & 7) ^ swz16(lrow);
@@ -462,19 +421,19 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // K offset, no 64-bit address arithmetic in the loop.  K is a multiple of 128 here (the host
     // sends other K to the fallback kernel), so every lane's 16 bytes are in range.
     const v4i rsrc_a = make_rsrc(p.A);
+    auto issue_a1 = [&](int i, int kstep, uint8_t* dA) {
+        direct_load_b128(rsrc_a, lds_address(dA) + wave * 1024 + i * NL * 1024, a_off[i], kstep * kKBlock);
+    };
     auto issue_a = [&](int kstep, uint8_t* dA) {
-        if (!loader) return;
-        const int k0 = kstep * kKBlock;
-        const uint32_t dst = lds_address(dA) + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < A_IT; ++i) direct_load_b128(rsrc_a, dst + i * NL * 1024, a_off[i], k0);
+        for (int i = 0; i < A_IT; ++i) issue_a1(i, kstep, dA);
     };
     const v4i rsrc_s = make_rsrc(p.As);
     // direct load of row group ph*NL + wave of chunk `chunk` (K steps ks + 8*chunk ..), if this wave has one
     auto issue_s = [&](int chunk, int ph) {
         if constexpr (BLOCKSCALE) {
             const int g = ph * NL + wave;
-            if (p.As && loader && g < S_GROUPS) {
+            if (p.As && g < S_GROUPS) {
                 const int r = g * 8 + (lane >> 3);
                 int src;
                 if constexpr (GROUP == GROUP_DENSE) src = m0 + min(r, rows_valid - 1);
@@ -517,9 +476,12 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
                           *reinterpret_cast<const v4i*>(base + frag1));
         }
     };
-    auto mma = [&](auto ntm_tag, const uint8_t* cB) {
+    // `after_tile(tn)` runs behind the MFMAs of column tile tn (the step's direct loads are issued there)
+    auto mma = [&](auto ntm_tag, const uint8_t* cB, auto&& after_tile) {
         constexpr int NTM = decltype(ntm_tag)::value;  // this wave's row groups that hold valid rows
         if constexpr (NTM == 0) {
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) after_tile(tn);
             return;
         } else if constexpr (BLOCKSCALE) {
             // One MFMA (into a zeroed 16x16 product), then the four scale-and-add operations of the
@@ -544,6 +506,10 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
                 if (tm == 0 && tn + 1 < TN) read_w(tn + 1);
                 if (j >= 2) acc[(j - 2) / NTM][(j - 2) % NTM] += part[(j - 2) % 3] * scale_of((j - 2) / NTM, (j - 2) % NTM);
                 __builtin_amdgcn_sched_barrier(0);
+                if (tm == NTM - 1) {
+                    after_tile(tn);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
 #pragma unroll
             for (int j = NJ - 2; j < NJ; ++j) acc[j / NTM][j % NTM] += part[j % 3] * scale_of(j / NTM, j % NTM);
@@ -555,13 +521,24 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
 #pragma unroll
                 for (int tm = 0; tm < NTM; ++tm) asm volatile("" : "+v"(acc[tn][tm]));
         } else {
+            // weight fragments two column tiles ahead; the order is pinned (the direct loads are inline assembly, which
+            // the compiler's own interleaving hints cannot place)
+            v8i wf[2];
+            auto read_w = [&](int tn) {
+                const uint8_t* base = cB + b_frag_base + w_tile_row(tn) * kKBlock;
+                wf[tn & 1] = join(*reinterpret_cast<const v4i*>(base + wfrag0), *reinterpret_cast<const v4i*>(base + wfrag1));
+            };
+            read_w(0);
+            read_w(1);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
-                const uint8_t* base = cB + b_frag_base + w_tile_row(tn) * kKBlock;
-                const v8i wf = join(*reinterpret_cast<const v4i*>(base + wfrag0),
-                                    *reinterpret_cast<const v4i*>(base + wfrag1));
 #pragma unroll
-                for (int tm = 0; tm < NTM; ++tm) acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
+                for (int tm = 0; tm < NTM; ++tm) acc[tn][tm] = mfma_e4m3(wf[tn & 1], af[tm], acc[tn][tm]);
+                __builtin_amdgcn_sched_barrier(0);
+                after_tile(tn);
+                if (tn + 2 < TN) read_w(tn + 2);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
@@ -584,8 +561,11 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     //   top of step k : issue B(k+1) -> other stage (and one row group of the next chunk of activation
     //                   scales);  read A fragments (and scales) of stage k%2;  barrier
     //                   (every wave holds its A fragments: that A slab is free)
-    //   then          : issue A(k+2) -> this stage's A slab;  MFMAs with B fragments streamed from LDS
+    //   then          : MFMAs with B fragments streamed from LDS; behind each of the first column tiles' MFMAs one
+    //                   or two of the direct loads of A(k+2) -> this stage's A slab
     //   end of step k : wait for all direct loads except A(k+2);  barrier
+    // (Measured on the block-scaled and grouped forms: dealing B(k+1) over the column tiles as well, so that no load
+    // is issued in a burst, leaves the weights half a step to land and is 5-15 % slower.)
     // Steps past the end are clamped to the last step: they re-fetch it into an idle slab, which
     // keeps the loop body free of branches.
     const int nsteps = ks_end - ks, last = ks_end - 1;
@@ -609,14 +589,23 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     auto k_loop = [&](auto ntm_tag) {
         constexpr int NTM = decltype(ntm_tag)::value;
         auto step = [&](int k, uint8_t* cA, uint8_t* cB, uint8_t* oB) {
+            // the weight slab of step k+1 is requested first: it has this whole step to land
             issue_b(min(k + 1, last), oB);
             issue_s((k - ks) / kScaleChunk + 1, (k - ks) % kScaleChunk);
             read_a(ntm_tag, cA);
             read_scales(ntm_tag, k);
             lds_barrier();
-            issue_a(min(k + 2, last), cA);
-            mma(ntm_tag, cB);
-            if constexpr (!BLOCKSCALE && NTM > 0) pipeline_hint<NTM, TN, A_IT>();
+            // the activation slab of step k+2 goes into the slab whose fragments every wave holds in registers since the
+            // barrier above, one or two loads behind each of the first column tiles' MFMAs
+            constexpr int PER = (A_IT + TN - 1) / TN;
+            const int ka2 = min(k + 2, last);
+            mma(ntm_tag, cB, [&](int tn) {
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int idx = tn * PER + q;
+                    if (idx < A_IT) issue_a1(idx, ka2, cA);
+                }
+            });
             __builtin_amdgcn_s_waitcnt(kWaitAllButA);
             lds_barrier();
         };
