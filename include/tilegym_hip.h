@@ -59,12 +59,12 @@ typedef struct tg_tensor {
  * This is the C form of the reference's per-call `kernel_configs={...}` override
  * (src/tilegym/kernel_utils.py:14-36). */
 enum {
-    TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (direct weight streaming), 3 stream (weight streaming through LDS), 4 pipe (register-pipelined 256x256 tile; per-tensor scales, beta == 0, bf16/f16 out) */
+    TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (direct weight streaming), 3 stream (weight streaming through LDS) */
     TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (64/128/256)            */
     TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (128/256)               */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
     TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4); stream kernel: LDS buffers per wave (1/2) */
-    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); pipe kernel: loader waves (4/8) */
+    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup; tiled 256x256 per-tensor kernel: 4 = the generic form instead of the hand-ordered one */
     TG_CFG_COUNT = 8
 };
 
@@ -77,7 +77,8 @@ enum {
  *   unsloth w8a8_block_fp8_matmul           src/tilegym/suites/unsloth/cutile/fp8.py:388-446
  *
  * a: (M,K), or (K,M) when trans_a;  b: (K,N), or (N,K) when trans_b;  both e4m3fn, contiguous.
- * c: (M,N) contiguous, dtype bf16 / f32 / f16.  beta != 0 reads c.
+ * c: (M,N) contiguous, dtype bf16 / f32 / f16, or float8_e4m3fn (the fp32 result is rounded to nearest even and
+ *    saturates at +-448; NaN stays NaN).  beta != 0 reads c.
  * scale_a / scale_b (f32, device memory):
  *     NULL                     -> 1.0
  *     1 element                -> per-tensor scale
@@ -129,7 +130,7 @@ int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t tra
  * b_scale (Q, ceil(N/128), ceil(K/128)) f32, or NULL (ones);
  * m_indptr (Q+1) i32 DEVICE memory, non-decreasing, m_indptr[Q] <= total_m; segments need no
  * alignment and may be empty.  Rows at or past m_indptr[Q] are not written.
- * c (total_m,N) bf16/f32/f16.
+ * c (total_m,N) bf16/f32/f16 (or float8_e4m3fn, as for tg_fp8_gemm).
  */
 int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
                            const tg_tensor* a_scale, const tg_tensor* b_scale,
@@ -182,7 +183,7 @@ int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, 
  * list is run problem by problem with tg_fp8_gemm's schedules (same results).
  * Replaces the launch half of tilegym.ops.group_gemm, src/tilegym/ops/cutile/group_gemm.py:170-197.
  * c, a, b: arrays of `count` descriptor pointers; scale_a, scale_b: NULL, or arrays whose entries are NULL or
- * one-element f32 tensors.  All c_i share one dtype (bf16 / f16 / f32).  workspace: as for tg_fp8_gemm
+ * one-element f32 tensors.  All c_i share one dtype (bf16 / f16 / f32 / float8_e4m3fn).  workspace: as for tg_fp8_gemm
  * (only used on the problem-by-problem route).
  */
 int32_t tg_fp8_group_gemm(const tg_tensor* const* c, const tg_tensor* const* a, const tg_tensor* const* b,

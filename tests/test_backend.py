@@ -128,14 +128,9 @@ def test_quantizer_operators_have_no_host_path():
         per_token_group_quant_8bit(x, 64, dst_dtype=torch.int8)
 
 
-def test_moe_align_host_logic_matches_known_answer():
+def test_moe_align_has_no_cpu_path():
     from tilegym_amd.ops import moe_align_block_size
-    from tilegym_amd.ops.hip.moe import _moe_align_torch_ops
 
     ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]]) - 1
     with pytest.raises(RuntimeError, match="device tensors only"):
         moe_align_block_size(ids, 4, 4)  # no CPU path in the product
-    s, e, post, cum, mx = _moe_align_torch_ops(ids, 4, 4)  # index arithmetic of the > 512 experts path
-    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
-    assert s.numel() == 24 and e.numel() == 6 and e[:4].tolist() == [0, 1, 2, 3]
-    assert int(post) == 16 and cum.tolist() == [0, 4, 8, 12, 16] and int(mx) == 3

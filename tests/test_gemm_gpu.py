@@ -78,37 +78,35 @@ def test_per_tensor_tiled_split_k(device, split):
         assert torch.equal(again, out)
 
 
-# ----------------------------------------------------------------------------- per-tensor, register-pipelined 256x256 tile
-@pytest.mark.parametrize("loaders", [4, 8])
+# ----------------------------------------------------------------------------- per-tensor, hand-ordered 256x256 tile
+@pytest.mark.parametrize("waves", [-1, 4])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 520, 384), (257, 255, 512), (1024, 768, 1280), (40, 1000, 256), (512, 252, 640)])
-def test_per_tensor_pipe(device, M, N, K, loaders):
-    """K = 128 (two half-steps), K with an odd number of 128-byte steps (loop tail), ragged M and N,
-    N not a multiple of 8 (scalar store path), both loader-wave counts."""
-    g = _g(M + 3 * N + K + loaders)
+def test_per_tensor_ordered_256(device, M, N, K, waves):
+    """The 256x256 tile in its hand-ordered form (default) and in the generic form (WAVES = 4): K = 128 (one step: the
+    prologue's second-step loads re-fetch the first), odd numbers of steps, ragged M and N, N not a multiple of 8 (scalar
+    store path); bf16, f16, f32 outputs and beta; the two forms agree bit for bit."""
+    g = _g(M + 3 * N + K)
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
     sa, sb = torch.tensor([0.013]), torch.tensor([0.0004])
+    kc = {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "SPLIT_K": 1, "WAVES": waves}
     ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
-    out = torch.full((M + 1, N), 7.0, dtype=torch.bfloat16, device=device)  # one guard row past the end
     res = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
-                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "pipe", "WAVES": loaders})
-    cfg = used("pipe")
-    assert cfg["WAVES"] == loaders
-    check(res, ref, what=f"pipe M={M} N={N} K={K} loaders={loaders}")
+                 out_dtype=torch.bfloat16, kernel_configs=kc)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (256, 256)
+    check(res, ref, what=f"256x256 M={M} N={N} K={K} waves={waves}")
+    other = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                   out_dtype=torch.bfloat16, kernel_configs=dict(kc, WAVES=4 if waves != 4 else -1))
+    assert torch.equal(res, other), "ordered and generic 256x256 kernels differ"
     one = torch.tensor([1.0])  # keep the f16 outputs in the normal range
     ref16 = R.ref_gemm_per_tensor(a, b, one, one, trans_b=True, out_dtype=torch.float16)
     res16 = matmul(a.to(device), b.to(device), trans_b=True, scale_a=one.to(device), scale_b=one.to(device),
-                   out_dtype=torch.float16, kernel_configs={"KERNEL": "pipe"})
-    used("pipe")
-    check(res16, ref16, what=f"pipe f16 M={M} N={N} K={K}")
-    del out
-
-
-def test_pipe_falls_back_to_tiled_for_beta_and_f32(device):
-    g = _g(91)
-    a, b = fp8_randn((300, 256), g), fp8_randn((520, 256), g, 0.1)
-    out = matmul(a.to(device), b.to(device), trans_b=True, out_dtype=torch.float32, kernel_configs={"KERNEL": "pipe"})
-    used("tiled")
-    check(out, R.ref_gemm_per_tensor(a, b, trans_b=True, out_dtype=torch.float32))
+                   out_dtype=torch.float16, kernel_configs=kc)
+    check(res16, ref16, what=f"256x256 f16 M={M} N={N} K={K}")
+    ref32 = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True, out_dtype=torch.float32)
+    res32 = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                   out_dtype=torch.float32, kernel_configs=kc)
+    check(res32, ref32, what=f"256x256 f32 M={M} N={N} K={K}")
 
 
 # ----------------------------------------------------------------------------- skinny
@@ -271,6 +269,28 @@ def test_reference_default_returns_input_dtype(device):
     assert torch.allclose(out.float().cpu(), ref.float(), atol=1.0, rtol=1.0)
     ok, rep = R.compare_to_oracle(out.float(), ref.float(), 0.13, 0.02)  # one e4m3 ulp
     assert ok, rep
+
+
+@pytest.mark.parametrize("kc", [None, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256}, {"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128, "SPLIT_K": 2},
+                                {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 128}, {"KERNEL": "stream"}, {"KERNEL": "skinny"}, {"KERNEL": "fallback"}],
+                         ids=lambda k: "auto" if k is None else "-".join(str(v) for v in k.values()))
+def test_e4m3_output_is_cast_in_the_epilogue(device, kc):
+    """c of dtype float8_e4m3fn through the C ABI: every kernel family rounds its fp32 result to e4m3 (nearest even)
+    in its own epilogue and saturates at +-448 (the torch cast would give NaN from 465 up).  Integer-valued operands
+    make the fp32 result exact, so the expected codes are known bit for bit, ragged N included (scalar store path)."""
+    g = _g(77)
+    M, N, K = 40, 202, 256
+    a = torch.randint(-3, 4, (M, K), generator=g).float()
+    b = torch.randint(-2, 3, (N, K), generator=g).float()
+    exact = a @ b.t()
+    for scale in (1.0, 16.0):  # 16: most results lie beyond +-448
+        want = (exact * scale).clamp(-448, 448).to(FP8)
+        c = torch.empty(M, N, dtype=FP8, device=device)
+        _lib.fp8_gemm(c, a.to(FP8).to(device), b.to(FP8).to(device), None, None, False, True, scale, 0.0, kernel_configs=kc)
+        got = c.cpu()
+        assert torch.equal(got.view(torch.uint8), want.view(torch.uint8)), f"scale {scale}: {(got.float() != want.float()).sum().item()} codes differ"
+        if scale == 16.0:
+            assert (want.float().abs() == 448).float().mean() > 0.3 and not torch.isnan(got.float()).any()
 
 
 def test_power_of_two_scales_are_exact(device):
@@ -589,13 +609,13 @@ def test_moe_fc2_shape_top_k_1(device):
 
 @pytest.mark.parametrize("T,top_k,E,bs,dtype", [(4, 3, 4, 4, torch.int64), (1, 1, 1, 16, torch.int32), (77, 6, 64, 16, torch.int64),
                                                  (4096, 6, 64, 128, torch.int32), (1000, 2, 512, 64, torch.int64),
-                                                 (333, 8, 8, 1, torch.int32), (50, 4, 600, 32, torch.int64),
+                                                 (333, 8, 8, 1, torch.int32),
                                                  (7001, 6, 160, 256, torch.int32), (1025, 1, 3, 64, torch.int64)])
 def test_moe_align_kernel_matches_oracle(device, T, top_k, E, bs, dtype):
     """All five outputs, bit for bit, against the oracle (stable order inside an expert, sentinel
     fill, padded prefix sums); empty experts, one expert, block size 1, int32 and int64 ids, one to
     the largest number of workgroups (one per 1024 ids, at most 32), slices that end inside the last
-    workgroup, and more experts than the one-launch kernel takes (torch device ops then)."""
+    workgroup."""
     g = _g(T + E)
     ids = torch.randint(0, E, (T, top_k), generator=g)
     if E >= 8:
@@ -612,6 +632,16 @@ def test_moe_align_kernel_matches_oracle(device, T, top_k, E, bs, dtype):
         assert torch.equal(w, gt), f"{name} differs"
     again = moe_align_block_size(ids.to(dtype).to(device), bs, E)
     assert all(torch.equal(a, b) for a, b in zip(got, again))
+
+
+def test_moe_align_limits(device):
+    """More experts than the one-launch kernel takes is an explicit error (no torch-op path); an empty routing
+    gives the fill values."""
+    with pytest.raises(NotImplementedError):
+        moe_align_block_size(torch.zeros(50, 4, dtype=torch.int64, device=device), 32, 600)
+    s_, e_, post, cum, mx = moe_align_block_size(torch.zeros(0, 2, dtype=torch.int64, device=device), 16, 8)
+    want = R.moe_align_block_size_ref(torch.zeros(0, 2, dtype=torch.int64), 16, 8)
+    assert s_.numel() == want[0].numel() and int(post) == 0 and int(mx) == 0 and cum.cpu().tolist() == [0] * 9
 
 
 # ----------------------------------------------------------------------------- activation quantizers
@@ -1081,6 +1111,20 @@ def _rows_subset(M, count, seed=0):
     return idx
 
 
+def _rows_stratified(M, per_tile, seed=0, tile=256):
+    """`per_tile` rows from every `tile`-row tile of an M-row problem; over the tiles the rows walk through all sixteen
+    16-row group slots of a tile (the unit a wave owns), at a random offset inside the slot; first and last row included."""
+    g = _g(seed)
+    rows = []
+    for t in range(-(-M // tile)):
+        for j in range(per_tile):
+            slot = (t * per_tile + j) % (tile // 16)
+            r = t * tile + slot * 16 + int(torch.randint(0, 16, (1,), generator=g))
+            rows.append(min(r, M - 1))
+    rows += [0, M - 1]
+    return torch.tensor(sorted(set(rows)))
+
+
 def test_config1_full(device):
     for trans_b in (True, False):
         case = W.config1(trans_b=trans_b)
@@ -1107,14 +1151,15 @@ def test_config2_llama_decode_full(device, proj):
 
 @pytest.mark.parametrize("proj", list(W.LLAMA_SHAPES))
 def test_config3_llama_prefill_sampled_rows(device, proj):
-    """Full-size launch; the oracle is evaluated on 96 sampled activation rows (each output row
-    depends on its own activation row only) and on linearity across the whole output."""
+    """Full-size launch; the oracle is evaluated on ~98 activation rows, three from every 256-row tile and walking
+    through every 16-row group slot of a tile (each output row depends on its own activation row only), and on
+    linearity across the whole output."""
     case = W.llama_prefill_case(proj)
     d = case.to(device)
     out = matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a, scale_b=d.scale_b, out_dtype=torch.bfloat16)
     cfg = used("tiled")
     assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (256, 256)
-    rows = _rows_subset(case.M, 96)
+    rows = _rows_stratified(case.M, 3)
     ref = R.ref_gemm_per_tensor(case.a[rows], case.b, case.scale_a, case.scale_b, trans_b=True)
     check(out[rows.to(device)], ref, what=f"config 3 {proj}")
     assert torch.isfinite(out.float()).all()
@@ -1129,7 +1174,7 @@ def test_config4_block_scaled_full(device, N, K):
     d = big.to(device)
     out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16)
     used("tiled")
-    rows = _rows_subset(4096, 64)
+    rows = _rows_stratified(4096, 4)  # every 256- and 128-row tile, every 16-row group slot
     ref = R.ref_w8a8_block_fp8_matmul(big.a[rows], big.b, big.scale_a[rows], big.scale_b, None, torch.bfloat16)
     check(out[rows.to(device)], ref, what=f"config 4 M=4096 {N}x{K}")
     out16 = w8a8_block_fp8_matmul(d.a[:16].contiguous(), d.b, d.scale_a[:16].contiguous(), d.scale_b, None, torch.bfloat16)

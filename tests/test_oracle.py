@@ -329,6 +329,30 @@ def test_fused_experts_oracle_is_the_composition_of_its_steps():
     assert q.shape == (3, 200) and s.shape == (3, 2) and act.shape == (3, 200)
 
 
+def test_silu_mul_quant_oracle_against_library_silu_and_a_hand_computed_vector():
+    """ref_silu_mul_quant: its activation against torch.nn.functional.silu (a library routine, not the oracle's own
+    formula) and against values worked out by hand; a wrong sign in the exponential, sigmoid instead of SiLU, or
+    gate and up swapped fails one of them; then scales and codes from the activation's own amax."""
+    F = torch.nn.functional
+    g = _g(31)
+    for dtype in (torch.bfloat16, torch.float16):
+        x = (torch.randn(6, 2 * 256, generator=g) * 3).to(dtype)
+        q, s, act = R.ref_silu_mul_quant(x)
+        want = (F.silu(x[:, :256].float()) * x[:, 256:].float()).to(dtype)
+        assert torch.equal(act, want)
+        amax = want.float().reshape(6, 2, 128).abs().amax(-1)
+        assert torch.equal(s, amax / 448.0)
+        assert torch.equal(R.fp8_to_f32(q), (want.float().reshape(6, 2, 128) / s[..., None]).clamp(-448, 448).to(R.FP8).float().reshape(6, 256))
+    # by hand: silu(0) = 0; silu(1) = 1 / (1 + e^-1) = 0.7310586; silu(-1) = -0.2689414; silu(2) = 1.7615942; silu(-20) ~ -4.1e-8
+    gate = torch.tensor([[0.0, 1.0, -1.0, 2.0, -20.0, 3.0, 0.5, -0.5]])
+    up = torch.tensor([[5.0, 2.0, 4.0, -1.0, 1.0, 0.0, -2.0, 8.0]])
+    expect = torch.tensor([[0.0, 1.4621172, -1.0757656, -1.7615942, -4.1223e-08, 0.0, -0.6224593, -1.5101871]])
+    _, _, act = R.ref_silu_mul_quant(torch.cat([gate, up], 1).to(torch.float16))
+    assert torch.equal(act, expect.to(torch.float16))
+    _, _, act_swapped = R.ref_silu_mul_quant(torch.cat([up, gate], 1).to(torch.float16))
+    assert not torch.equal(act_swapped, act)
+
+
 def test_compare_to_oracle_flags_errors():
     ref = torch.randn(64, 64, generator=_g(13))
     ok, _ = R.compare_to_oracle(ref.to(torch.bfloat16), ref)

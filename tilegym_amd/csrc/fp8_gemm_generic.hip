@@ -58,6 +58,10 @@ __global__ void __launch_bounds__(256) fp8_gemm_generic_kernel(const GenericPara
         float* c = reinterpret_cast<float*>(p.C) + at;
         if (p.beta != 0.f) v += p.beta * (*c);
         *c = v;
+    } else if (p.out_type == OUT_F8) {
+        uint8_t* c = reinterpret_cast<uint8_t*>(p.C) + at;
+        if (p.beta != 0.f) v += p.beta * e4m3_to_f32(*c);
+        *c = f32_to_e4m3(v);
     } else {
         _Float16* c = reinterpret_cast<_Float16*>(p.C) + at;
         if (p.beta != 0.f) v += p.beta * (float)(*c);

@@ -155,6 +155,16 @@ __device__ __forceinline__ void store8(void* C, int out_type, int64_t row, int c
             }
             p[0] = lo;
             p[1] = hi;
+        } else if (out_type == OUT_F8) {
+            uint8_t* p = reinterpret_cast<uint8_t*>(C) + base;
+            if (beta != 0.0f) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    lo[q] += beta * e4m3_to_f32(p[q]);
+                    hi[q] += beta * e4m3_to_f32(p[4 + q]);
+                }
+            }
+            *reinterpret_cast<v2i*>(p) = v2i{pack_e4m3x4(lo[0], lo[1], lo[2], lo[3]), pack_e4m3x4(hi[0], hi[1], hi[2], hi[3])};
         } else if (out_type == OUT_BF16) {
             typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
             typedef float v8f __attribute__((ext_vector_type(8)));
@@ -183,6 +193,10 @@ __device__ __forceinline__ void store8(void* C, int out_type, int64_t row, int c
             float* p = reinterpret_cast<float*>(C) + base + q;
             if (beta != 0.0f) x += beta * (*p);
             *p = x;
+        } else if (out_type == OUT_F8) {
+            uint8_t* p = reinterpret_cast<uint8_t*>(C) + base + q;
+            if (beta != 0.0f) x += beta * e4m3_to_f32(*p);
+            *p = f32_to_e4m3(x);
         } else {
             _Float16* p = reinterpret_cast<_Float16*>(C) + base + q;
             if (beta != 0.0f) x += beta * (float)(*p);
@@ -587,7 +601,6 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // The loop exists once per number of row groups a wave may have to compute (NTM = 0 .. TM): the
     // waves of a workgroup can run different copies, every copy issues the same loads and barriers.
     auto k_loop = [&](auto ntm_tag) {
-        constexpr int NTM = decltype(ntm_tag)::value;
         auto step = [&](int k, uint8_t* cA, uint8_t* cB, uint8_t* oB) {
             // the weight slab of step k+1 is requested first: it has this whole step to land
             issue_b(min(k + 1, last), oB);
@@ -770,6 +783,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     };
     if (SPLIT || p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
     else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
+    else if (p.out_type == OUT_F8) emit(std::integral_constant<int, OUT_F8>{});
     else emit(std::integral_constant<int, OUT_F16>{});
 
 #endif

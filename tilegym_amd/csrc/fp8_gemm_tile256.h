@@ -196,6 +196,7 @@ __global__ void __launch_bounds__(512, 1) fp8_gemm_tile256_kernel(const GemmPara
     };
     if (p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
     else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
+    else if (p.out_type == OUT_F8) emit(std::integral_constant<int, OUT_F8>{});
     else emit(std::integral_constant<int, OUT_F16>{});
 #endif
 }

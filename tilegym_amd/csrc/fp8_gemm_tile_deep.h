@@ -143,6 +143,7 @@ __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmPa
     };
     if (SPLIT || p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
     else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
+    else if (p.out_type == OUT_F8) emit(std::integral_constant<int, OUT_F8>{});
     else emit(std::integral_constant<int, OUT_F16>{});
 #endif
 }

@@ -14,7 +14,7 @@ namespace tg {
 
 constexpr int kKBlock = 128;    // bytes of K consumed by one 16x16x128 MFMA = the quant block
 
-enum OutType { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2 };  // same numbering as the ABI dtype codes
+enum OutType { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_F8 = 7 };  // same numbering as the ABI dtype codes (7: e4m3fn)
 
 // How rows of the activation operand are found.
 // GROUP_GATHER_ACT: the gather form for a (E, 2I, K) gate/up weight whose epilogue produces
@@ -97,6 +97,20 @@ __device__ __forceinline__ float e4m3_to_f32(uint8_t c) {
     return __uint_as_float(s | ((e + 120u) << 23) | (m << 20));
 }
 
+// One fp32 value -> e4m3fn code, round to nearest even, saturating at +-448 (NaN stays NaN).
+__device__ __forceinline__ float clamp_e4m3(float x) {
+    const float c = fminf(fmaxf(x, -448.0f), 448.0f);
+    return x == x ? c : x;
+}
+// Four values -> four e4m3fn codes packed in one dword (element 0 in the low byte).
+__device__ __forceinline__ int pack_e4m3x4(float a, float b, float c, float d) {
+    int w = 0;
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_e4m3(a), clamp_e4m3(b), w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_e4m3(c), clamp_e4m3(d), w, true);
+    return w;
+}
+__device__ __forceinline__ uint8_t f32_to_e4m3(float x) { return (uint8_t)(pack_e4m3x4(x, 0.f, 0.f, 0.f) & 0xFF); }
+
 // Store 4 consecutive outputs C[row][col..col+3] = v (+ beta * old), masked against ncols.
 __device__ __forceinline__ void store4(void* C, int out_type, int64_t row, int col, int N, v4f v,
                                        float beta, bool vec_ok) {
@@ -114,6 +128,13 @@ __device__ __forceinline__ void store4(void* C, int out_type, int64_t row, int c
             v4f* p = reinterpret_cast<v4f*>(reinterpret_cast<float*>(C) + base);
             if (beta != 0.0f) v = v + beta * (*p);
             *p = v;
+        } else if (out_type == OUT_F8) {
+            uint8_t* p = reinterpret_cast<uint8_t*>(C) + base;
+            if (beta != 0.0f) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] += beta * e4m3_to_f32(p[r]);
+            }
+            *reinterpret_cast<int*>(p) = pack_e4m3x4(v[0], v[1], v[2], v[3]);
         } else {
             f16x4* p = reinterpret_cast<f16x4*>(reinterpret_cast<_Float16*>(C) + base);
             if (beta != 0.0f) {
@@ -137,6 +158,10 @@ __device__ __forceinline__ void store4(void* C, int out_type, int64_t row, int c
             float* p = reinterpret_cast<float*>(C) + base + r;
             if (beta != 0.0f) x += beta * (*p);
             *p = x;
+        } else if (out_type == OUT_F8) {
+            uint8_t* p = reinterpret_cast<uint8_t*>(C) + base + r;
+            if (beta != 0.0f) x += beta * e4m3_to_f32(*p);
+            *p = f32_to_e4m3(x);
         } else {
             _Float16* p = reinterpret_cast<_Float16*>(C) + base + r;
             if (beta != 0.0f) x += beta * (float)(*p);

@@ -30,8 +30,6 @@ hipError_t run_tile_moe_act(int bm, const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p, int gx, hipStream_t s);
 // up to kListMax per-tensor NT problems in one launch (tile 256x256, 128x128 or 64x128)
 hipError_t run_tile_list(int bm, int bn, const GemmList& gl, int gx, hipStream_t s);
-// register-pipelined 256x256 tile: per-tensor scales, dense, beta == 0, bf16/f16 output, K % 128 == 0
-hipError_t run_pipe(int waves, int loaders, const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_skinny(int mt, int rg, int nw, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
 hipError_t run_stream(int mt, int nbuf, int waves, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
 // 64 weight rows per workgroup, activation piece shared through LDS: M <= 16

@@ -53,7 +53,8 @@ int32_t check_tensor(const tg_tensor* t, const char* name, int ndim) {
     return TG_OK;
 }
 
-int32_t out_type_of(int32_t dtype) {
+// f32 / f16 / bf16 tensors (inputs of the quantizers, outputs of the dequantizer and the MoE helpers)
+int32_t io_type_of(int32_t dtype) {
     switch (dtype) {
         case TG_F32: return tg::OUT_F32;
         case TG_F16: return tg::OUT_F16;
@@ -61,6 +62,8 @@ int32_t out_type_of(int32_t dtype) {
         default: return -1;
     }
 }
+// output types of the GEMM entry points: the above plus e4m3fn (saturating round-to-nearest-even cast in the epilogue)
+int32_t out_type_of(int32_t dtype) { return dtype == TG_F8E4M3FN ? (int32_t)tg::OUT_F8 : io_type_of(dtype); }
 
 int64_t elem_size(int32_t dtype) {
     switch (dtype) {
@@ -100,21 +103,6 @@ struct DeviceGuard {
     }
 };
 
-// Compute units of a device (queried once per device; 256 on MI355X).
-int compute_units(int dev) {
-    static int cached[64] = {0};
-    if (dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
-            (void)hipGetLastError();
-            n = 256;
-        }
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
 // Device address of `scratch` on device `dev`, which must be the current device.  Looked up on the first
 // call per device and kept; every device holds its own copy of the array at its own address.
 std::mutex g_scratch_mutex;
@@ -134,7 +122,7 @@ hipError_t scratch_address(int dev, uint8_t** out) {
 }
 
 struct Schedule {
-    int kernel;  // 0 fallback, 1 tiled, 2 skinny, 3 stream, 4 pipe (register-pipelined 256x256 tile)
+    int kernel;  // 0 fallback, 1 tiled, 2 skinny, 3 stream
     int bm, bn, split_k, row_groups, mt, waves;
 };
 
@@ -172,7 +160,7 @@ int pick_split(int64_t units, int64_t target_units, int64_t kblocks, int min_ste
     return (int)cdiv(kblocks, kps);
 }
 
-Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout, bool pipe_ok,
+Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
                       const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
     Schedule s{0, -1, -1, 1, -1, -1, -1};
     const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
@@ -183,7 +171,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     // above 16 rows the streaming kernels would re-read the activations once per 16 weight rows;
     // the LDS-tiled kernel with a 64-row tile and split-K shares them across 128 weight rows
     bool skinny = M <= 16 || (M <= 64 && !tile_ok);
-    if ((want_kernel == 1 || want_kernel == 4) && tile_ok) skinny = false;
+    if (want_kernel == 1 && tile_ok) skinny = false;
     if ((want_kernel == 2 || want_kernel == 3) && M <= 64) skinny = true;
     if (!skinny && !tile_ok) return s;
     const int want_split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
@@ -262,16 +250,10 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
         else { bm = 64; bn = 128; }
     }
-    if (want_kernel == 4 && pipe_ok) { bm = 256; bn = 256; }
     s.bm = bm;
     s.bn = bn;
     const int64_t wgs = cdiv(M, bm) * cdiv(N, bn);
     s.split_k = 1;
-    if (bm == 256 && bn == 256 && pipe_ok && want_split <= 1 && want_kernel == 4) {  // opt-in: slower than the tiled kernel so far
-        s.kernel = 4;
-        s.waves = cfg_get(cfg, ncfg, TG_CFG_WAVES) == 8 ? 8 : 4;  // loader waves (of eight)
-        return s;
-    }
     if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
     } else if (want_split < 0 && bm == 64 && bn == 128 && !block_scaled) {
@@ -382,7 +364,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
     if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN)
         return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7), got %d and %d", a->dtype, b->dtype);
     const int out_type = out_type_of(c->dtype);
-    if (out_type < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16 or f32, got dtype code %d", c->dtype);
+    if (out_type < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16, f32 or float8_e4m3fn, got dtype code %d", c->dtype);
     const int64_t M = trans_a ? a->shape[1] : a->shape[0], K = trans_a ? a->shape[0] : a->shape[1];
     const int64_t N = trans_b ? b->shape[0] : b->shape[1], Kb = trans_b ? b->shape[1] : b->shape[0];
     if (K != Kb) return fail(TG_ERR_INVALID, "incompatible matrices: K of a is %lld, K of b is %lld", (long long)K, (long long)Kb);
@@ -458,12 +440,10 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
 
     const bool fast_layout = !trans_a && b_is_nk && (K % 16) == 0 && aligned16(a->ptr) &&
                              aligned16(reinterpret_cast<uint64_t>(Bnt)) && N * K < kOffsetLimit;
-    const bool pipe_ok = !block_scaled && beta == 0.0f && (K % 128) == 0 &&
-                         (out_type == tg::OUT_BF16 || out_type == tg::OUT_F16);
-    Schedule s = choose_dense(M, N, K, block_scaled, fast_layout, pipe_ok, cfg, ncfg, ws_free);
+    Schedule s = choose_dense(M, N, K, block_scaled, fast_layout, cfg, ncfg, ws_free);
     if (static_scratch) {
         // same schedule as tg_fp8_gemm with a full-size workspace, or an error: never a silently smaller split
-        const Schedule full = choose_dense(M, N, K, block_scaled, fast_layout, pipe_ok, cfg, ncfg, INT64_MAX / 2);
+        const Schedule full = choose_dense(M, N, K, block_scaled, fast_layout, cfg, ncfg, INT64_MAX / 2);
         if (full.split_k != s.split_k)
             return fail(TG_ERR_INVALID, "split-K %d of this problem needs %lld bytes of partial sums, the static scratch buffer has %lld free: "
                         "call tg_fp8_gemm with a workspace, or force a smaller SPLIT_K", full.split_k,
@@ -545,17 +525,12 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         pc.M = (int)rows;
         if (rows != M && s.split_k > 1) { pc.split_k = 1; pc.ksteps_per_split = (int)kblocks; }
         int gx = (int)(cdiv(rows, s.bm) * cdiv(N, s.bn));
-        if (s.kernel == 4) {  // persistent: one workgroup per compute unit
-            const int cus = compute_units(device_id);
-            if (gx > cus) gx = cus;
-        }
         const bool split = pc.split_k > 1;
         const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128;
         // hand-ordered K loop for the dense per-tensor 256x256 tile (WAVES = 4 asks for the generic form with four loader waves)
         const bool ordered = s.kernel == 1 && !block_scaled && !split && s.bm == 256 && s.bn == 256 &&
                              cfg_get(cfg, ncfg, TG_CFG_WAVES) != 4;
-        hipError_t e = s.kernel == 4 ? tg::run_pipe(8, s.waves, pc, gx, stream)
-                     : ordered ? tg::run_tile256(pc, gx, stream)
+        hipError_t e = ordered ? tg::run_tile256(pc, gx, stream)
                      : deep ? tg::run_tile_deep(split, pc, gx, pc.split_k, stream)
                      : block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
                                     : tg::run_tile_per_tensor(s.bm, s.bn, split, pc, gx, pc.split_k, stream);
@@ -579,7 +554,7 @@ static int32_t grouped_common(const tg_tensor* c, const tg_tensor* a, const tg_t
     if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN)
         return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7)");
     *out_type = out_type_of(c->dtype);
-    if (*out_type < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16 or f32");
+    if (*out_type < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16, f32 or float8_e4m3fn");
     *rows_a = a->shape[0];
     *K = a->shape[1];
     *E = b->shape[0];
@@ -879,7 +854,7 @@ int32_t tg_fp8_quant_group(const tg_tensor* q, const tg_tensor* scales, const tg
     if ((rc = check_tensor(x, "x", -1)) || (rc = check_tensor(q, "q", -1))) return rc;
     if (!scales) return fail(TG_ERR_NULL, "scales: null tensor descriptor");
     if (scales->ndim < 0 || scales->ndim > TG_MAX_DIMS) return fail(TG_ERR_INVALID, "scales: ndim %d out of range", scales->ndim);
-    const int x_type = out_type_of(x->dtype);
+    const int x_type = io_type_of(x->dtype);
     if (x_type < 0) return fail(TG_ERR_DTYPE, "x must be bf16, f16 or f32");
     if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
     if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
@@ -933,7 +908,7 @@ int32_t tg_fp8_weight_dequant(const tg_tensor* y, const tg_tensor* x, const tg_t
     if ((rc = check_tensor(x, "x", 2)) || (rc = check_tensor(y, "y", 2)) || (rc = check_tensor(s, "s", 2))) return rc;
     if (x->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "x must be float8_e4m3fn (dtype code 7)");
     if (s->dtype != TG_F32) return fail(TG_ERR_DTYPE, "s must be f32");
-    const int y_type = out_type_of(y->dtype);
+    const int y_type = io_type_of(y->dtype);
     if (y_type < 0) return fail(TG_ERR_DTYPE, "y must be bf16, f16 or f32");
     if (block_size < 1) return fail(TG_ERR_INVALID, "block_size must be positive");
     const int64_t M = x->shape[0], N = x->shape[1];
@@ -958,7 +933,7 @@ int32_t tg_silu_mul_quant_1x128(const tg_tensor* q, const tg_tensor* scales, con
     g_err[0] = 0;
     int32_t rc;
     if ((rc = check_tensor(x, "x", 2)) || (rc = check_tensor(q, "q", 2)) || (rc = check_tensor(scales, "scales", 2))) return rc;
-    const int x_type = out_type_of(x->dtype);
+    const int x_type = io_type_of(x->dtype);
     if (x_type != tg::OUT_BF16 && x_type != tg::OUT_F16) return fail(TG_ERR_DTYPE, "x must be bf16 or f16");
     if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
     if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
@@ -982,7 +957,7 @@ int32_t tg_moe_sum(const tg_tensor* out, const tg_tensor* x, int32_t device_id, 
     g_err[0] = 0;
     int32_t rc;
     if ((rc = check_tensor(x, "x", 3)) || (rc = check_tensor(out, "out", 2))) return rc;
-    const int x_type = out_type_of(x->dtype);
+    const int x_type = io_type_of(x->dtype);
     if ((x_type != tg::OUT_BF16 && x_type != tg::OUT_F16) || out->dtype != x->dtype)
         return fail(TG_ERR_DTYPE, "x and out must both be bf16 or both f16");
     const int64_t T = x->shape[0], k = x->shape[1], H = x->shape[2];
@@ -1014,7 +989,7 @@ int32_t tg_fp8_group_gemm(const tg_tensor* const* c, const tg_tensor* const* a, 
     for (int i = 0; i < count; ++i) {
         if ((rc = check_tensor(a[i], "a[i]", 2)) || (rc = check_tensor(b[i], "b[i]", 2)) || (rc = check_tensor(c[i], "c[i]", 2))) return rc;
         if (a[i]->dtype != TG_F8E4M3FN || b[i]->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7)");
-        if (out_type_of(c[i]->dtype) < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16 or f32");
+        if (out_type_of(c[i]->dtype) < 0) return fail(TG_ERR_DTYPE, "c must be bf16, f16, f32 or float8_e4m3fn");
         if (out_dtype < 0) out_dtype = c[i]->dtype;
         if (c[i]->dtype != out_dtype) one_launch = false;
         const int64_t M = a[i]->shape[0], K = a[i]->shape[1];

@@ -56,18 +56,17 @@ def matmul(a, b, trans_a=None, trans_b=None, static_persistent=None, use_tma=Non
     assert a.is_contiguous() and b.is_contiguous(), "operands must be contiguous"
 
     out_dtype = kwargs.get("out_dtype")
-    cast_back = None
     if out_dtype is None:
-        # reference behaviour: result in a.dtype (src/tilegym/ops/cutile/matmul.py:446)
-        cast_back = a.dtype
-        out_dtype = torch.float32
-    if out_dtype not in _OUT_DTYPES:
+        # reference behaviour: result in a.dtype (src/tilegym/ops/cutile/matmul.py:446); the kernel's epilogue casts
+        # (round to nearest even, saturating at +-448)
+        out_dtype = torch.float8_e4m3fn
+    if out_dtype not in _OUT_DTYPES and out_dtype != torch.float8_e4m3fn:
         raise NotImplementedError(f"out_dtype {out_dtype} not supported")
     sa, alpha = _split_scale(kwargs.get("scale_a"), float(kwargs.get("alpha", 1.0)))
     sb, alpha = _split_scale(kwargs.get("scale_b"), alpha)
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
     _lib.fp8_gemm(c, a, b, sa, sb, trans_a, trans_b, alpha, 0.0, kwargs.get("kernel_configs"))
-    return c.to(cast_back) if cast_back is not None else c
+    return c
 
 
 @register_impl("flashinfer.gemm.gemm_alpha_beta", backend="hip")
@@ -177,11 +176,9 @@ def group_gemm(group_A, group_B, static_persistent=True, use_tma=True, transpose
         raise ValueError(f"group_A and group_B must have same length, got {len(group_A)} and {len(group_B)}")
     transpose_b = bool(transpose_b)
     out_dtype = kwargs.get("out_dtype")
-    cast_back = None
     if out_dtype is None:
-        cast_back = group_A[0].dtype
-        out_dtype = torch.float32
-    if out_dtype not in _OUT_DTYPES:
+        out_dtype = torch.float8_e4m3fn  # A.dtype, cast in the kernels' epilogue (saturating, round to nearest even)
+    if out_dtype not in _OUT_DTYPES and out_dtype != torch.float8_e4m3fn:
         raise NotImplementedError(f"out_dtype {out_dtype} not supported")
     dev = group_A[0].device
     if not group_A[0].is_cuda:
@@ -211,4 +208,4 @@ def group_gemm(group_A, group_B, static_persistent=True, use_tma=True, transpose
 
     _lib.fp8_group_gemm(outs, list(group_A), list(group_B), as_tensors(kwargs.get("scales_a")),
                         as_tensors(kwargs.get("scales_b")), transpose_b, kwargs.get("kernel_configs"))
-    return [o.to(cast_back) for o in outs] if cast_back is not None else outs
+    return outs

@@ -50,35 +50,17 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     src/tilegym/ops/cutile/moe_align_block.py:205-268: (sorted_ids[numel + E*(bs-1)] pre-filled
     with the sentinel numel, expert_ids[ceil(that/bs)], num_tokens_post_pad[1], cumsum[E+1] of
     padded counts, max_expert_cnt[1]).  Stable within an expert.  One HIP launch for up to 512
-    experts; beyond that the same result from torch device ops."""
+    experts; more raise NotImplementedError."""
     if not topk_ids.is_cuda:
         raise RuntimeError("the hip backend works on device tensors only; topk_ids is on " + str(topk_ids.device))
-    if num_experts <= _lib.MOE_ALIGN_MAX_EXPERTS and topk_ids.numel() > 0:
-        return _lib.moe_align_block_size(topk_ids, block_size, num_experts)
-    return _moe_align_torch_ops(topk_ids, block_size, num_experts)
-
-
-def _moe_align_torch_ops(topk_ids: torch.Tensor, block_size: int, num_experts: int):
-    """The same five outputs from torch ops on the tensor's device (used beyond 512 experts)."""
-    dev = topk_ids.device
-    flat = topk_ids.reshape(-1).to(torch.int64)
-    numel = flat.numel()
-    cap = numel + num_experts * (block_size - 1)
-    nblk = -(-cap // block_size)
-    counts = torch.bincount(flat, minlength=num_experts)[:num_experts]
-    padded = (counts + block_size - 1) // block_size * block_size
-    cumsum = torch.zeros(num_experts + 1, dtype=torch.int64, device=dev)
-    cumsum[1:] = torch.cumsum(padded, 0)
-    starts_unpadded = torch.cumsum(counts, 0) - counts
-    order = torch.argsort(flat, stable=True)
-    sorted_experts = flat[order]
-    rank_in_expert = torch.arange(numel, device=dev) - starts_unpadded[sorted_experts]
-    dest = cumsum[sorted_experts] + rank_in_expert
-    sorted_ids = torch.full((cap,), numel, dtype=torch.int32, device=dev)
-    sorted_ids[dest] = order.to(torch.int32)
-    blk_start = torch.arange(nblk, device=dev, dtype=torch.int64) * block_size
-    expert_ids = torch.searchsorted(cumsum[1:].contiguous(), blk_start, right=True)
-    expert_ids = torch.where(blk_start < cumsum[-1], expert_ids, torch.zeros_like(expert_ids)).to(torch.int32)
-    post = cumsum[-1:].to(torch.int32)
-    mx = counts.max().reshape(1).to(torch.int32) if numel else torch.zeros(1, dtype=torch.int32, device=dev)
-    return sorted_ids, expert_ids, post, cumsum.to(torch.int32), mx
+    if num_experts > _lib.MOE_ALIGN_MAX_EXPERTS:
+        raise NotImplementedError(f"moe_align_block_size on the hip backend handles up to {_lib.MOE_ALIGN_MAX_EXPERTS} experts "
+                                  f"(one launch, per-expert counters in LDS); got {num_experts}")
+    if topk_ids.numel() == 0:  # nothing routed: every output is its fill value (no kernel needed)
+        dev = topk_ids.device
+        cap = num_experts * (block_size - 1)
+        nblk = -(-cap // block_size)
+        return (torch.zeros(cap, dtype=torch.int32, device=dev), torch.zeros(nblk, dtype=torch.int32, device=dev),
+                torch.zeros(1, dtype=torch.int32, device=dev), torch.zeros(num_experts + 1, dtype=torch.int32, device=dev),
+                torch.zeros(1, dtype=torch.int32, device=dev))
+    return _lib.moe_align_block_size(topk_ids, block_size, num_experts)
