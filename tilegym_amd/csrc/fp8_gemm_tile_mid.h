@@ -1,0 +1,148 @@
+// 64 x 32 and 32 x 32 per-tensor tiles whose four waves split K inside the workgroup (16 < M <= 128 against small
+// weights, one launch): C[m,n] = sum_k A[m,k] * B[n,k].
+//
+// These M are weight-streaming problems with too few output tiles to fill the chip: M = 64 against a 4096 x 4096
+// weight is 32 tiles of 64 x 128.  Splitting K across workgroups fills it, but the partial sums then need a second
+// launch that costs more than the GEMM's own roofline time.  Here the tile is narrow (32 weight rows: 128 - 900
+// workgroups on the Llama shapes) and K is split across the four waves of the workgroup instead: every wave owns a
+// contiguous quarter of the K steps and runs its own ring of LDS slabs (BM activation rows + 32 weight rows x 128
+// bytes per stage; three stages of 12 KiB for BM = 64, four of 8 KiB for BM = 32) with direct loads STAGES - 1 steps
+// ahead - no barrier in the loop, a wave only waits for its own loads - and the four partial tiles are added through
+// LDS at the end, in a fixed order.
+// The price is activation traffic: every workgroup reads all K of its activation rows (L2 hits), two bytes (BM = 64)
+// or one (BM = 32) per weight byte, and those bytes take LDS that would otherwise hold weights in flight from HBM.
+// It pays while one round of workgroups covers the problem and the weights are small (measured: 4096 x 4096 and
+// 6144 x 4096 at M <= 128); for larger weights the 64 x 128 tile with split-K across workgroups stays faster.
+// Slab layout, swizzles and fragment addressing are those of fp8_gemm_tile.h (first column-tile pair).
+#pragma once
+
+#include "fp8_gemm_tile.h"
+
+namespace tg {
+
+template <int BM, int STAGES>
+__global__ void __launch_bounds__(256, 1) fp8_gemm_tile_mid_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int BN = 32, NW = 4, AHEAD = STAGES - 1;
+    constexpr int TM = BM / 16, TN = BN / 16;
+    constexpr int A_IT = BM / 8, B_IT = BN / 8;               // 8 + 4 direct loads per wave and K step
+    constexpr int STAGE_BYTES = (BM + BN) * kKBlock;          // 12 KiB
+    constexpr int PER_STEP = A_IT + B_IT;
+    static_assert(TN == 2, "one column-tile pair per wave");
+
+    __shared__ __align__(1024) uint8_t lds[NW * STAGES * STAGE_BYTES];  // 144 KiB; reused for the reduction
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int K = p.K;
+    const int n0 = (int)blockIdx.x * BN, m0 = (int)blockIdx.y * BM;
+    const int rows_valid = min(BM, p.M - m0);
+    // this wave's K steps: a contiguous share
+    const int ks = (int)((int64_t)p.kblocks * wave / NW), ks_end = (int)((int64_t)p.kblocks * (wave + 1) / NW);
+    const int nsteps = ks_end - ks, last = max(ks_end - 1, 0);
+
+    const int lrow = lane >> 3;
+    const int lj = (lane & 7) ^ swz16(lrow);
+    uint32_t a_off[A_IT], b_off[B_IT];
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+        const int r = i * 8 + lrow;
+        a_off[i] = (uint32_t)(m0 + min(r, rows_valid - 1)) * (uint32_t)K + lj * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) {
+        const int br = i * 8 + lrow;
+        const int ljb = (lane & 7) ^ swz_w(((i & 1) << 3) | lrow);
+        b_off[i] = (uint32_t)min(n0 + br, p.N - 1) * (uint32_t)K + ljb * 16;
+    }
+    const v4i rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(p.B);
+    uint8_t* my = lds + wave * STAGES * STAGE_BYTES;
+    const uint32_t lds0 = lds_address(my);
+    auto issue = [&](int kstep, int stage) {
+        const int k0 = min(kstep, last) * kKBlock;
+        const uint32_t dst = lds0 + stage * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) direct_load_b128_nt(rsrc_b, dst + BM * kKBlock + i * 1024, b_off[i], k0);
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) direct_load_b128(rsrc_a, dst + i * 1024, a_off[i], k0);
+    };
+
+    const int li = lane & 15, lg = lane >> 4;
+    const uint32_t frag0 = li * kKBlock + ((lg ^ swz16(li)) << 4), frag1 = frag0 ^ 64;
+    const int wrow = ((li >> 2) << 3) | (li & 3);
+    const uint32_t wfrag0 = BM * kKBlock + wrow * kKBlock + ((lg ^ swz_w(wrow)) << 4), wfrag1 = wfrag0 ^ 64;
+
+    v4f acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    constexpr int kKeep = (AHEAD - 1) * PER_STEP;  // the step after the one about to be used may still be in flight
+    constexpr int kWaitStep = 0x0F70 | (kKeep & 15) | ((kKeep >> 4) << 14);
+    constexpr int kWaitAll = 0x0F70, kWaitLds = 0xC07F;
+
+    if (nsteps > 0) {
+#pragma unroll
+        for (int s = 0; s < AHEAD; ++s) issue(ks + s, s);
+        for (int i = 0; i < nsteps; ++i) {
+            const int stage = i % STAGES;
+            __builtin_amdgcn_s_waitcnt(kWaitStep);   // step i has landed (steps past the end re-fetch the last one)
+            const uint8_t* base = my + stage * STAGE_BYTES;
+            v8i af[TM], wf[TN];
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn) {
+                const uint8_t* b = base + (tn & 1) * 4 * kKBlock;
+                wf[tn] = join(*reinterpret_cast<const v4i*>(b + wfrag0), *reinterpret_cast<const v4i*>(b + wfrag1));
+            }
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                const uint8_t* a = base + tm * 16 * kKBlock;
+                af[tm] = join(*reinterpret_cast<const v4i*>(a + frag0), *reinterpret_cast<const v4i*>(a + frag1));
+            }
+            // the stage that step i-1 used is free (its fragments were consumed by the MFMAs of the last iteration)
+            issue(ks + i + AHEAD, (i + AHEAD) % STAGES);
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_e4m3(wf[tn], af[tm], acc[tn][tm]);
+        }
+        __builtin_amdgcn_s_waitcnt(kWaitAll);  // the re-fetches past the end must land before the slabs are reused
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitLds);
+    __syncthreads();
+
+    // ---- add the four partial tiles through LDS: wave w writes its 8 accumulator tiles, then every wave sums
+    // column-tile-pair rows tm = w (fixed order over the waves) and stores them
+    v4f* red = reinterpret_cast<v4f*>(lds);
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) red[((wave * TN + tn) * TM + tm) * 64 + lane] = acc[tn][tm];
+    __syncthreads();
+    const int tm = wave;  // the first TM waves each finish one row group
+    static_assert(TM <= NW, "one row group per wave in the epilogue");
+    if (tm >= TM) return;
+    v4f s0 = red[((0 * TN + 0) * TM + tm) * 64 + lane], s1 = red[((0 * TN + 1) * TM + tm) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) {
+        s0 += red[((w * TN + 0) * TM + tm) * 64 + lane];
+        s1 += red[((w * TN + 1) * TM + tm) * 64 + lane];
+    }
+    float scale = p.alpha;
+    if (p.As) scale *= p.As[0];
+    if (p.Bs) scale *= p.Bs[0];
+    const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;
+    const int rt = tm * 16 + li, col = n0 + lg * 8;
+    if (rt >= rows_valid || col >= p.N) return;
+    store8(p.C, p.out_type, m0 + rt, col, p.N, s0 * scale, s1 * scale, p.beta, vec_ok);
+#endif
+}
+
+template <int BM, int STAGES>
+inline hipError_t launch_tile_mid(const GemmParams& p, hipStream_t stream) {
+    hipLaunchKernelGGL((fp8_gemm_tile_mid_kernel<BM, STAGES>), dim3((p.N + 31) / 32, (p.M + BM - 1) / BM, 1), dim3(256, 1, 1), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace tg

@@ -137,6 +137,7 @@ void remember(const Schedule& s) {
 }
 
 bool tile_exists(int bm, int bn, bool block_scaled) {
+    if ((bm == 64 || bm == 32) && bn == 32) return !block_scaled;  // the four waves split K inside the workgroup (per-tensor only)
     if (bm == 128 && bn == 128) return true;
     if (bm == 128 && bn == 256) return true;
     if (bm == 64 && bn == 128) return true;
@@ -244,7 +245,14 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // the three-stage 64x128 kernel (per-tensor) also wins above 64 rows while its tiles fit one round of the
         // chip: 13.3 / 14.5 / 17.8 / 18.1 us against 17.1 / 18.8 / 18.7 / 21.6 for M = 96 / 128 / 256 / 512 at
         // N = K = 4096; with more tiles the larger tiles' operand reuse wins (M = 1024: 32 vs 23 us)
-        if (M <= 64 || (!block_scaled && tiles(64, 128) <= 256)) { bm = 64; bn = 128; }
+        // small weights at 16 < M <= 128: narrow tiles whose four waves split K inside the workgroup fill the chip in
+        // one launch, where the 64x128 tile needs split-K and a reduction launch (4096 x 4096 weight: 8.8 / 8.8 / 10.3 us
+        // at M = 32 / 64 / 128 against 10.4 / 12.0 / 14.7; 6144 x 4096: 9.2 / 10.9 against 11.8 / 13.3 at M = 32 / 64).
+        // Beyond one round of workgroups, or when the weights dominate (>= 32 MiB), the activation re-reads cost more.
+        const bool small_w = !block_scaled && M <= 128 && N * K <= ((int64_t)32 << 20) && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1;
+        if (small_w && M <= 64 && tiles(32, 32) <= 256) { bm = 32; bn = 32; }
+        else if (small_w && tiles(64, 32) <= 256) { bm = 64; bn = 32; }
+        else if (M <= 64 || (!block_scaled && tiles(64, 128) <= 256)) { bm = 64; bn = 128; }
         else if (tiles(256, 256) >= 200 && s256 >= s128) { bm = 256; bn = 256; }
         else if (!block_scaled && tiles(128, 256) >= 200 && tiles(256, 256) < 200) { bm = 128; bn = 256; }
         else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
@@ -254,6 +262,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     s.bn = bn;
     const int64_t wgs = cdiv(M, bm) * cdiv(N, bn);
     s.split_k = 1;
+    if (bn == 32) return s;  // K is split inside the workgroup: one launch
     if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
     } else if (want_split < 0 && bm == 64 && bn == 128 && !block_scaled) {
@@ -527,10 +536,12 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         int gx = (int)(cdiv(rows, s.bm) * cdiv(N, s.bn));
         const bool split = pc.split_k > 1;
         const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128;
+        const bool mid = s.kernel == 1 && !block_scaled && s.bn == 32;
         // hand-ordered K loop for the dense per-tensor 256x256 tile (WAVES = 4 asks for the generic form with four loader waves)
         const bool ordered = s.kernel == 1 && !block_scaled && !split && s.bm == 256 && s.bn == 256 &&
                              cfg_get(cfg, ncfg, TG_CFG_WAVES) != 4;
-        hipError_t e = ordered ? tg::run_tile256(pc, gx, stream)
+        hipError_t e = mid ? tg::run_tile_mid(s.bm, pc, stream)
+                     : ordered ? tg::run_tile256(pc, gx, stream)
                      : deep ? tg::run_tile_deep(split, pc, gx, pc.split_k, stream)
                      : block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
                                     : tg::run_tile_per_tensor(s.bm, s.bn, split, pc, gx, pc.split_k, stream);
