@@ -38,20 +38,29 @@ KERNEL_SYMBOLS = {"tiled": "fp8_gemm_tile_kernel", "skinny": "fp8_gemm_skinny_ke
                   "fallback": "fp8_gemm_generic_kernel"}
 ROTATE_BYTES = 640 << 20
 
-# HBM bytes per launch (reads + writes) from the hardware counters FETCH_SIZE and WRITE_SIZE, collected in
-# two profiler passes of this program and scaled by what the same counters read for --calibrate-copy's
-# elementwise add of known size (reads x2.000, writes x1.000); figures and commands are in
-# profiles/fp8_gemm_tile_kernel_prefill_pmc.txt and profiles/fp8_gemm_stream_wide_kernel_decode_pmc.txt.
-# Decode entries are the average over M = 1, 8, 16 of one projection (same grid).
-KIB = 1024
-MEASURED_TRAFFIC = {
-    "c3_prefill_qkv_M8192": (147790.8 * 2 + 98759.7) * KIB,
-    "c3_prefill_gate_up_M8192": (689180.8 * 2 + 460607.7) * KIB,
-    "c2_decode_qkv": (12471.9 * 2 + 100.0) * KIB,
-    "c2_decode_o": (8375.9 * 2 + 66.7) * KIB,
-    "c2_decode_gate_up": (57522.9 * 2 + 467.1) * KIB,
-    "c2_decode_down": (29179.7 * 2 + 933.6) * KIB,
-}
+# HBM bytes per launch (reads + writes) come from the hardware counters FETCH_SIZE and WRITE_SIZE, collected in two profiler
+# passes of this program and scaled by what the same counters read for --calibrate-copy's elementwise add of known size.
+# The figures live in profiles/hbm_traffic_per_launch.txt, one line per measured shape together with the kernel and
+# schedule they were measured on; a run whose schedule differs from the recorded one reports "traffic": null (the
+# recorded figure would describe another kernel).
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.txt")
+TRAFFIC_FIELDS = ("shape", "kernel_symbol", "block_m", "block_n", "split_k", "row_groups", "waves", "fetch_kib", "write_kib",
+                  "read_scale", "write_scale")
+
+
+def load_traffic_table(path=TRAFFIC_FILE):
+    table = {}
+    try:
+        with open(path) as f:
+            for line in f:
+                line = line.split("#", 1)[0].split()
+                if len(line) != len(TRAFFIC_FIELDS):
+                    continue
+                rec = dict(zip(TRAFFIC_FIELDS, line))
+                table[rec["shape"]] = rec
+    except OSError:
+        pass
+    return table
 
 
 def kernel_symbol(shape):
@@ -68,11 +77,20 @@ def kernel_symbol(shape):
     return KERNEL_SYMBOLS[shape["kernel"]]
 
 
-def measured_traffic(shape_name):
-    for key, val in MEASURED_TRAFFIC.items():
-        if shape_name == key or (key.startswith("c2_decode") and shape_name.startswith(key + "_M") and not shape_name.endswith("M64")):
-            return int(val)
-    return None   # operand footprint to rotate through (> 2x the 256 MB memory-side cache)
+def measured_traffic(shape, table=None):
+    """(bytes per launch, note) for a measured shape: the recorded counter figures if they were taken on the kernel and
+    schedule this run used, else (None, why)."""
+    table = load_traffic_table() if table is None else table
+    rec = table.get(shape["name"])
+    if rec is None:
+        return None, "no counter pass recorded for this shape"
+    ran = {"kernel_symbol": kernel_symbol(shape), "block_m": shape["block_m"], "block_n": shape["block_n"],
+           "split_k": shape["split_k"], "row_groups": shape["row_groups"], "waves": shape["waves"]}
+    diff = [k for k, v in ran.items() if str(v) != rec[k]]
+    if diff:
+        return None, "recorded on another schedule (" + ", ".join(f"{k}: recorded {rec[k]}, ran {ran[k]}" for k in diff) + ")"
+    nbytes = (float(rec["fetch_kib"]) * float(rec["read_scale"]) + float(rec["write_kib"]) * float(rec["write_scale"])) * 1024
+    return int(nbytes), f"FETCH_SIZE x {rec['read_scale']} + WRITE_SIZE x {rec['write_scale']}, {os.path.relpath(TRAFFIC_FILE, ROOT)}"
 
 
 def _events_ms(fn, iters, stream):
@@ -310,11 +328,13 @@ def main():
         ms_per_step = ms / args.steps
         shapes = [measure_shape(r, args.steps, 1, stream, use_graph=False) for r in runners]
         dom = max(shapes, key=lambda s: s["us"])
+        traffic, traffic_note = measured_traffic(dom)
         out.update({
             "value": round(total_flops / (ms_per_step * 1e-3) * 1e-12, 2),
             "ms_per_step": round(ms_per_step, 4),
             "roofline": {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                         "frac": dom["frac_mfma"], "traffic": measured_traffic(dom["name"]), "kernel": f"fp8_gemm_tile_kernel<{dom['block_m']},{dom['block_n']}> per-tensor",
+                         "frac": dom["frac_mfma"], "traffic": traffic, "traffic_source": traffic_note,
+                         "kernel": f"{kernel_symbol(dom)} ({dom['block_m']}x{dom['block_n']} tile, per-tensor scales)",
                          "shape": dom["name"], "us_per_launch": dom["us"]},
         })
         detail["prefill"] = shapes
@@ -344,12 +364,13 @@ def main():
         tot_us = sum(s["us"] for s in shapes)
         small = [s for s in shapes if int(s["name"].rsplit("M", 1)[1]) <= 16]
         dom = max(small, key=lambda s: s["us"])
+        traffic, traffic_note = measured_traffic(dom)
         dec = {
             "metric": "FP8 GEMM decode GB/s (algorithmic bytes, cold cache)", "value": round(tot_b / tot_us * 1e-3, 1), "unit": "GB/s",
             "us_per_step": round(tot_us, 2),
             "frac_hbm_M_le_16": round(sum(s["bytes"] for s in small) / sum(s["us"] for s in small) * 1e-3 / PEAK_HBM_GBS, 4),
             "roofline": {"bound": "hbm", "achieved": dom["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
-                         "traffic": measured_traffic(dom["name"]), "kernel": kernel_symbol(dom) + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
+                         "traffic": traffic, "traffic_source": traffic_note, "kernel": kernel_symbol(dom) + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
         }
         detail["decode"] = shapes
         if "value" in out:
@@ -409,11 +430,16 @@ def main():
             for w in range(max(1, args.warmup)):
                 fn(w)
             n = max(args.steps, 32)
+            us_alloc = _events_ms(fn, n, stream) * 1e3 / n
+            q_out, s_out = _lib.fp8_quant_1x128(xs[0], 0.0, False)
+            fn = lambda i: _lib.fp8_quant_1x128(xs[i % len(xs)], 0.0, False, q=q_out, scales=s_out)  # noqa: E731
+            fn(0)
             us = _events_ms(fn, n, stream) * 1e3 / n
             nbytes = M * K * 3 + M * (K // 128) * 4
             shapes.append({"name": f"act_quant_1x128_bf16_{M}x{K}", "kernel": "act_quant_group_kernel", "us": round(us, 2),
                            "gbs": round(nbytes / us * 1e-3, 1), "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
-                           "note": "includes the torch allocation of the two outputs"})
+                           "us_with_output_allocation": round(us_alloc, 2),
+                           "note": "outputs pre-allocated; us_with_output_allocation includes torch.empty of the two outputs"})
             del xs
             torch.cuda.empty_cache()
         for (N, K) in ((28672, 4096), (12288, 5120)):
@@ -424,11 +450,16 @@ def main():
             for w in range(max(1, args.warmup)):
                 fn(w)
             n = max(args.steps, 32)
+            us_alloc = _events_ms(fn, n, stream) * 1e3 / n
+            y_out = _lib.fp8_weight_dequant(ws[0], sc, 128, torch.bfloat16)
+            fn = lambda i: _lib.fp8_weight_dequant(ws[i % len(ws)], sc, 128, torch.bfloat16, out=y_out)  # noqa: E731
+            fn(0)
             us = _events_ms(fn, n, stream) * 1e3 / n
             nbytes = N * K * 3 + sc.numel() * 4
             shapes.append({"name": f"weight_dequant_bf16_{N}x{K}", "kernel": "weight_dequant_kernel", "us": round(us, 2),
                            "gbs": round(nbytes / us * 1e-3, 1), "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
-                           "note": "includes the torch allocation of the output"})
+                           "us_with_output_allocation": round(us_alloc, 2),
+                           "note": "output pre-allocated; us_with_output_allocation includes torch.empty of the output"})
             del ws
             torch.cuda.empty_cache()
         ids = W.moe_routing(4096, 64, 6, seed=0)[1].to(device)

@@ -333,12 +333,15 @@ def moe_align_block_size(topk_ids, block_size: int, num_experts: int):
     return sorted_ids, expert_ids, post, cumsum, mx
 
 
-def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = False):
-    """(q e4m3fn like x, scales (..., K/128) f32) through tg_fp8_quant_1x128."""
+def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = False, q=None, scales=None):
+    """(q e4m3fn like x, scales (..., K/128) f32) through tg_fp8_quant_1x128; ``q`` / ``scales`` may be given
+    (pre-allocated outputs of those shapes)."""
     L = load()
     x = x.contiguous()
-    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
-    scales = torch.empty(x.shape[:-1] + (x.shape[-1] // 128,), dtype=torch.float32, device=x.device)
+    if q is None:
+        q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    if scales is None:
+        scales = torch.empty(x.shape[:-1] + (x.shape[-1] // 128,), dtype=torch.float32, device=x.device)
     rc = L.tg_fp8_quant_1x128(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
                               float(eps), 1 if flashinfer_rule else 0, _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_fp8_quant_1x128")
@@ -360,11 +363,12 @@ def fp8_quant_group(x: torch.Tensor, group_size: int, eps: float, rule: int, sca
     return q, scales
 
 
-def fp8_weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, dtype: torch.dtype) -> torch.Tensor:
-    """y (M, N) of ``dtype`` = float(x) * s[i // block_size, j // block_size] through tg_fp8_weight_dequant."""
+def fp8_weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, dtype: torch.dtype, out=None) -> torch.Tensor:
+    """y (M, N) of ``dtype`` = float(x) * s[i // block_size, j // block_size] through tg_fp8_weight_dequant
+    (``out``: a pre-allocated y)."""
     L = load()
     x, s = x.contiguous(), s.contiguous()
-    y = torch.empty(x.shape, dtype=dtype, device=x.device)
+    y = out if out is not None else torch.empty(x.shape, dtype=dtype, device=x.device)
     rc = L.tg_fp8_weight_dequant(_ref(make_tensor_desc(y)), _ref(make_tensor_desc(x)), _ref(make_tensor_desc(s)),
                                  int(block_size), _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_fp8_weight_dequant")

@@ -1,17 +1,13 @@
-// Deep-pipelined form of the 64x128 per-tensor tile (16 < M <= 64, usually with split-K): three LDS
-// stages of one K step each (3 x 24 KiB, two workgroups per compute unit), loads requested two steps
-// ahead, one barrier per step (four stages measured the same).
-// These launches are weight-streaming: a workgroup runs 8-16 K steps of 8 MFMAs per wave, and with the
-// two stages of fp8_gemm_tile.h (weights one step ahead) every step waited for a full trip to HBM
-// (1.3-2.2 k clocks per step measured, against 0.8 k of load issue and 0.26 k of MFMA).
+// Deep-pipelined form of the 64x128 per-tensor tile (16 < M <= 512 while its tiles fit one round of the chip,
+// usually with split-K): three LDS stages of one K step each (3 x 24 KiB), loads requested up to three steps
+// ahead, one barrier per step, and a software-pipelined step (see the loop).
+// These launches are weight-streaming: a workgroup runs 8-32 K steps of 8 MFMAs per wave, mostly alone on its
+// compute unit.  With the two stages of fp8_gemm_tile.h (weights one step ahead) every step waited for a full trip
+// to HBM (1.3-2.2 k clocks per step measured, against 0.4 k of load issue and 0.26 k of MFMA); with three stages
+// but load issue, fragment reads and MFMAs one after the other inside a step, a step still took ~1 k clocks.
 //
 // Same slab layout, swizzles, fragment addressing, MFMA order per accumulator and epilogue arithmetic
 // as fp8_gemm_tile_kernel<64, 128, 1, 4, false, GROUP_DENSE, SPLIT>: identical results.
-//
-// Step k of a workgroup:   wait until the loads of step k have landed (all but the newest step's worth)
-//                          barrier            (every wave's share of step k is in LDS; everyone is done with step k-1)
-//                          request step k+2 into the stage step k-1 used
-//                          fragments of step k -> MFMAs
 // Steps past the end re-fetch the last one, which keeps the wait counts uniform.
 #pragma once
 
@@ -22,7 +18,7 @@ namespace tg {
 template <bool SPLIT>
 __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    constexpr int BM = 64, BN = 128, WGN = 4, NW = 4, NL = 4, STAGES = 3, AHEAD = STAGES - 1;
+    constexpr int BM = 64, BN = 128, WGN = 4, NW = 4, NL = 4, STAGES = 3;  // (six stages, one workgroup per compute unit: 5-10 % slower)
     constexpr int WTN = BN / WGN;            // 32 columns per wave, all 64 rows
     constexpr int TM = BM / 16, TN = WTN / 16;
     constexpr int RPP = 8 * NL;
@@ -92,35 +88,71 @@ __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmPa
 
     // vmcnt(n): all of this wave's direct loads except the n most recent have landed
     constexpr int PER_STEP = A_IT + B_IT;
-    constexpr int kKeep = (AHEAD - 1) * PER_STEP;  // the steps after the one about to be used may still be in flight
-    constexpr int kWaitStep = 0x0F70 | (kKeep & 15) | ((kKeep >> 4) << 14);
+    constexpr int kPro = (STAGES - 1) * PER_STEP, kLoop = (STAGES - 2) * PER_STEP;  // loads that may stay in flight
+    constexpr int kWaitBut2 = 0x0F70 | (kPro & 15) | ((kPro >> 4) << 14);
+    constexpr int kWaitBut1 = 0x0F70 | (kLoop & 15) | ((kLoop >> 4) << 14);
     constexpr int kWaitAll = 0x0F70;
     constexpr int kWaitLds = 0xC07F;
+#define TG_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-#pragma unroll
-    for (int s = 0; s < AHEAD; ++s) issue(ks + s, s);
-    for (int i = 0; i < nsteps; ++i) {
-        const int stage = i % STAGES;
-        __builtin_amdgcn_s_waitcnt(kWaitStep);
-        __builtin_amdgcn_s_waitcnt(kWaitLds);
-        __builtin_amdgcn_s_barrier();
-        issue(ks + i + AHEAD, (i + AHEAD) % STAGES);
-        const uint8_t* base = lds + stage * STAGE_BYTES;
-        v8i af[TM];
-#pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
-            const uint8_t* a = base + tm * 16 * kKBlock;
-            af[tm] = join(*reinterpret_cast<const v4i*>(a + frag0), *reinterpret_cast<const v4i*>(a + frag1));
-        }
-#pragma unroll
-        for (int tn = 0; tn < TN; ++tn) {
+    // Software-pipelined loop.  The fragments of step i are in registers when iteration i starts (read during iteration
+    // i-1), so iteration i runs its MFMAs while the fragments of step i+1 are read and the loads of step i+3 are issued,
+    // one direct load and one fragment behind each MFMA: with one workgroup per compute unit (these launches rarely have
+    // more) nothing else would hide the LDS latency and the load issue time.  One barrier per step: behind it every
+    // wave's share of step i+1 is visible and stage i is free (everyone holds its fragments).
+    v8i af[2][TM], wf[2][TN];
+    auto read_frag = [&](int f, int set, const uint8_t* base) {  // fragment f of a step: 0..TM-1 activations, then weights
+        if (f < TM) {
+            const uint8_t* a = base + f * 16 * kKBlock;
+            af[set][f] = join(*reinterpret_cast<const v4i*>(a + frag0), *reinterpret_cast<const v4i*>(a + frag1));
+        } else {
+            const int tn = f - TM;
             const uint8_t* b = base + ((tn >> 1) * 32 + (tn & 1) * 4) * kKBlock;
-            const v8i wf = join(*reinterpret_cast<const v4i*>(b + wfrag0), *reinterpret_cast<const v4i*>(b + wfrag1));
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = mfma_e4m3(wf, af[tm], acc[tn][tm]);
+            wf[set][tn] = join(*reinterpret_cast<const v4i*>(b + wfrag0), *reinterpret_cast<const v4i*>(b + wfrag1));
         }
+    };
+    auto issue1 = [&](int q, int kstep, int stage) {  // direct load q of a step (activations first)
+        const int k0 = min(kstep, last) * kKBlock;
+        const uint32_t dst = lds0 + stage * STAGE_BYTES;
+        if (q < A_IT) direct_load_b128(rsrc_a, dst + q * NL * 1024, a_off[q], k0);
+        else direct_load_b128_nt(rsrc_b, dst + BM * kKBlock + (q - A_IT) * NL * 1024, b_off[q - A_IT], k0);
+    };
+#pragma unroll
+    for (int s = 0; s < STAGES; ++s) issue(ks + s, s);
+    __builtin_amdgcn_s_waitcnt(kWaitBut2);  // step 0 has landed
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int f = 0; f < TM + TN; ++f) read_frag(f, 0, lds);
+    auto body = [&](int i, auto cur_tag) {
+        constexpr int CUR = decltype(cur_tag)::value, NXT = CUR ^ 1;
+        const int stage_n = (i + 1) % STAGES, stage_free = i % STAGES;
+        __builtin_amdgcn_s_waitcnt(kWaitBut1);  // step i+1 has landed (steps past the end re-fetch the last one)
+        __builtin_amdgcn_s_waitcnt(kWaitLds);   // my fragments of step i are in registers
+        __builtin_amdgcn_s_barrier();
+        TG_FENCE();
+        const uint8_t* nbase = lds + stage_n * STAGE_BYTES;
+        int j = 0;
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm, ++j) {
+                acc[tn][tm] = mfma_e4m3(wf[CUR][tn], af[CUR][tm], acc[tn][tm]);
+                TG_FENCE();
+                if (j < PER_STEP) issue1(j, ks + i + STAGES, stage_free);
+                if (j < TM + TN) read_frag(j, NXT, nbase);
+                TG_FENCE();
+            }
+    };
+    static_assert(TM * TN >= PER_STEP && TM * TN >= TM + TN, "one load and one fragment behind each MFMA");
+    int i = 0;
+    for (; i + 1 < nsteps; i += 2) {
+        body(i, std::integral_constant<int, 0>{});
+        body(i + 1, std::integral_constant<int, 1>{});
     }
+    if (i < nsteps) body(i, std::integral_constant<int, 0>{});
+#undef TG_FENCE
     __builtin_amdgcn_s_waitcnt(kWaitAll);  // the re-fetches past the end must land before the workgroup's LDS is released
+    __builtin_amdgcn_s_waitcnt(kWaitLds);
 
     // epilogue, straight from the accumulators (row 16*tm + li, eight consecutive columns per lane)
     float scale = p.alpha;
