@@ -9,9 +9,12 @@
 //           max(amax, eps) / 448                                           rule 1, flashinfer
 //           2^ceil(log2(max(that, 1e-10)))                                 rule 2, flashinfer with power-of-two scales
 //   q     = rne_e4m3(clamp(x / scale, -448, 448))
-// Arithmetic of src/tilegym/suites/unsloth/cutile/fp8.py:92-120 and
-// src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:22-145; both divisions are
-// correctly rounded (IEEE) divisions (a plain reciprocal multiply moves values across rounding boundaries).
+// Arithmetic of src/tilegym/suites/unsloth/cutile/fp8.py:92-120, of the column-major kernel of
+// src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:78-145 and of the reference's
+// test oracle for that operator (x / scale); both divisions are correctly rounded (IEEE) divisions.
+// The reference's row-major kernel (per_token_group_quant_8bit.py:57-63) multiplies by 1.0 / scale
+// instead, which can land one e4m3 code away at rounding boundaries: rule 1 with row-major scales
+// follows the test oracle's x / scale here, not that kernel's reciprocal form.
 // The scale of group j of row r is written to scales[r * row_stride + j * col_stride], which covers the
 // row-major layout and the column-major ones of per_token_group_quant_8bit.py:185-204.
 //

@@ -1,9 +1,12 @@
 """FP8 (e4m3fn) quantizer operators: the producers and consumers of the scale layouts the GEMMs use.
 Each is one HIP launch through the C ABI on device tensors (group size 16 / 32 / 64 / 128; bf16 / f16 /
 f32 activations; e4m3 codes).  There is no other path: host tensors and forms the kernels do not cover
-raise.  Every quantizer clamps to +-448 before the cast and divides with IEEE division, as the
-reference's kernels do (src/tilegym/suites/unsloth/cutile/fp8.py:105-116,
-src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:52-66)."""
+raise.  Every quantizer clamps to +-448 before the cast and divides with IEEE division (x / scale),
+as src/tilegym/suites/unsloth/cutile/fp8.py:105-116, the column-major kernel of
+src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:78-145 and the reference's test
+oracle of that operator do.  The reference's row-major kernel (per_token_group_quant_8bit.py:57-63)
+multiplies by 1.0 / scale instead; its codes can differ from x / scale by one e4m3 code at rounding
+boundaries, and the row-major form here follows the oracle's division, not that kernel."""
 
 from __future__ import annotations
 
