@@ -70,7 +70,7 @@ def kernel_symbol(shape):
         return "fp8_gemm_stream_wide_kernel"
     if shape["kernel"] == "tiled" and shape["block_m"] == 64 and shape["block_n"] == 128 and not shape.get("block_scaled", False):
         return "fp8_gemm_tile_deep_kernel"
-    if shape["kernel"] == "tiled" and shape["block_n"] == 32:
+    if shape["kernel"] == "tiled" and (shape["block_n"] == 32 or (shape["block_m"], shape["block_n"]) == (64, 64)):
         return "fp8_gemm_tile_mid_kernel"
     if shape["kernel"] == "tiled" and shape["block_m"] == 256 and shape["split_k"] == 1 and not shape.get("block_scaled", False):
         return "fp8_gemm_tile256_kernel"

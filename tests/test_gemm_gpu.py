@@ -109,34 +109,34 @@ def test_per_tensor_ordered_256(device, M, N, K, waves):
     check(res32, ref32, what=f"256x256 f32 M={M} N={N} K={K}")
 
 
-@pytest.mark.parametrize("bm", [32, 64])
+@pytest.mark.parametrize("bm,bn", [(32, 32), (64, 32), (64, 64)])
 @pytest.mark.parametrize("M,N,K", [(64, 512, 1024), (40, 200, 384), (17, 1000, 2560), (130, 72, 128), (33, 264, 256), (96, 4096, 4096)])
-def test_per_tensor_mid_tiles(device, bm, M, N, K):
-    """The 32-column tiles whose four waves split K inside the workgroup: fewer K steps than waves (K = 128, 256: waves
+def test_per_tensor_mid_tiles(device, bm, bn, M, N, K):
+    """The narrow tiles whose four waves split K inside the workgroup: fewer K steps than waves (K = 128, 256: waves
     without a step), K steps that do not divide by four, ragged M (also across row tiles) and N, N not a multiple of 8;
     bf16 and f32 outputs with alpha and beta; reruns are bit-identical (fixed reduction order)."""
-    g = _g(M + 5 * N + K + bm)
+    g = _g(M + 5 * N + K + bm + bn)
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
     sa, sb = torch.tensor([0.013]), torch.tensor([0.0004])
-    kc = {"KERNEL": "tiled", "BLOCK_M": bm, "BLOCK_N": 32}
+    kc = {"KERNEL": "tiled", "BLOCK_M": bm, "BLOCK_N": bn}
     ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
     out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device), out_dtype=torch.bfloat16, kernel_configs=kc)
     cfg = used("tiled")
-    assert (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["SPLIT_K"]) == (bm, 32, 1)
-    check(out, ref, what=f"mid {bm}x32 M={M} N={N} K={K}")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["SPLIT_K"]) == (bm, bn, 1)
+    check(out, ref, what=f"mid {bm}x{bn} M={M} N={N} K={K}")
     again = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device), out_dtype=torch.bfloat16, kernel_configs=kc)
     assert torch.equal(out, again)
     c0 = torch.randn(M, N, generator=g)
     c = c0.clone().to(device)
     _lib.fp8_gemm(c, a.to(device), b.to(device), sa.to(device), sb.to(device), False, True, 1.5, 0.5, kernel_configs=kc)
     ref32 = 1.5 * R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True, out_dtype=torch.float32) + 0.5 * c0
-    check(c, ref32, what=f"mid {bm}x32 f32 alpha/beta M={M} N={N} K={K}")
+    check(c, ref32, what=f"mid {bm}x{bn} f32 alpha/beta M={M} N={N} K={K}")
 
 
 def test_mid_tiles_are_the_default_for_small_weights(device):
     g = _g(8)
     b = fp8_randn((4096, 4096), g, 0.02)
-    for M, want in ((32, (32, 32)), (64, (32, 32)), (128, (64, 32)), (256, (64, 128))):
+    for M, want in ((32, (32, 32)), (64, (32, 32)), (128, (64, 32)), (256, (64, 64)), (320, (64, 128))):
         a = fp8_randn((M, 4096), g)
         out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
         cfg = used("tiled")

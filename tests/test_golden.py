@@ -96,7 +96,7 @@ def test_oracle_moe_align_fixture():
 
 
 # ----------------------------------------------------------------------------- HIP path (GPU)
-DENSE_KERNELS = [None, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 128}, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 32},
+DENSE_KERNELS = [None, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 128}, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 32}, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 64},
                  {"KERNEL": "tiled", "BLOCK_M": 32, "BLOCK_N": 32}, {"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128},
                  {"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128, "SPLIT_K": 2},
                  {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256}, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "WAVES": 4},

@@ -1,18 +1,22 @@
-// 64 x 32 and 32 x 32 per-tensor tiles whose four waves split K inside the workgroup (16 < M <= 128 against small
-// weights, one launch): C[m,n] = sum_k A[m,k] * B[n,k].
+// 64 x 64, 64 x 32 and 32 x 32 per-tensor tiles whose four waves split K inside the workgroup (16 < M <= 256 against
+// small weights, one launch): C[m,n] = sum_k A[m,k] * B[n,k].
 //
 // These M are weight-streaming problems with too few output tiles to fill the chip: M = 64 against a 4096 x 4096
 // weight is 32 tiles of 64 x 128.  Splitting K across workgroups fills it, but the partial sums then need a second
 // launch that costs more than the GEMM's own roofline time.  Here the tile is narrow (32 weight rows: 128 - 900
 // workgroups on the Llama shapes) and K is split across the four waves of the workgroup instead: every wave owns a
 // contiguous quarter of the K steps and runs its own ring of LDS slabs (BM activation rows + 32 weight rows x 128
-// bytes per stage; three stages of 12 KiB for BM = 64, four of 8 KiB for BM = 32) with direct loads STAGES - 1 steps
+// bytes per stage; two stages of 16 KiB for 64 x 64, three of 12 KiB for 64 x 32, four of 8 KiB for 32 x 32) with direct loads STAGES - 1 steps
 // ahead - no barrier in the loop, a wave only waits for its own loads - and the four partial tiles are added through
 // LDS at the end, in a fixed order.
 // The price is activation traffic: every workgroup reads all K of its activation rows (L2 hits), two bytes (BM = 64)
 // or one (BM = 32) per weight byte, and those bytes take LDS that would otherwise hold weights in flight from HBM.
 // It pays while one round of workgroups covers the problem and the weights are small (measured: 4096 x 4096 and
-// 6144 x 4096 at M <= 128); for larger weights the 64 x 128 tile with split-K across workgroups stays faster.
+// 6144 x 4096 at M <= 128, 4096 x 4096 at M <= 256); for larger weights the 64 x 128 tile with split-K across
+// workgroups stays faster.  Measured and not kept: the same K partition with both operands streamed through a ring of
+// register sets instead of LDS (3 - 8 steps in flight per wave, bit-identical): 20 - 40 % slower at every depth -- a
+// fragment load fetches 64 bytes of 16 rows where a direct load fetches 128 bytes of 8, and these launches are bound
+// by the number of requests the memory path takes, not by the bytes in flight.
 // Slab layout, swizzles and fragment addressing are those of fp8_gemm_tile.h (first column-tile pair).
 #pragma once
 
@@ -20,17 +24,17 @@
 
 namespace tg {
 
-template <int BM, int STAGES>
+template <int BM, int BN, int STAGES>
 __global__ void __launch_bounds__(256, 1) fp8_gemm_tile_mid_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    constexpr int BN = 32, NW = 4, AHEAD = STAGES - 1;
+    constexpr int NW = 4, AHEAD = STAGES - 1;
     constexpr int TM = BM / 16, TN = BN / 16;
-    constexpr int A_IT = BM / 8, B_IT = BN / 8;               // 8 + 4 direct loads per wave and K step
-    constexpr int STAGE_BYTES = (BM + BN) * kKBlock;          // 12 KiB
+    constexpr int A_IT = BM / 8, B_IT = BN / 8;               // BM / 8 + 4 direct loads per wave and K step
+    constexpr int STAGE_BYTES = (BM + BN) * kKBlock;
     constexpr int PER_STEP = A_IT + B_IT;
-    static_assert(TN == 2, "one column-tile pair per wave");
+    static_assert(TN == 2 || TN == 4, "one or two column-tile pairs");
 
-    __shared__ __align__(1024) uint8_t lds[NW * STAGES * STAGE_BYTES];  // 144 KiB; reused for the reduction
+    __shared__ __align__(1024) uint8_t lds[NW * STAGES * STAGE_BYTES];  // 128 - 160 KiB; reused for the reduction
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -92,7 +96,7 @@ __global__ void __launch_bounds__(256, 1) fp8_gemm_tile_mid_kernel(const GemmPar
             v8i af[TM], wf[TN];
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn) {
-                const uint8_t* b = base + (tn & 1) * 4 * kKBlock;
+                const uint8_t* b = base + ((tn >> 1) * 32 + (tn & 1) * 4) * kKBlock;
                 wf[tn] = join(*reinterpret_cast<const v4i*>(b + wfrag0), *reinterpret_cast<const v4i*>(b + wfrag1));
             }
 #pragma unroll
@@ -120,28 +124,32 @@ __global__ void __launch_bounds__(256, 1) fp8_gemm_tile_mid_kernel(const GemmPar
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) red[((wave * TN + tn) * TM + tm) * 64 + lane] = acc[tn][tm];
     __syncthreads();
-    const int tm = wave;  // the first TM waves each finish one row group
-    static_assert(TM <= NW, "one row group per wave in the epilogue");
-    if (tm >= TM) return;
-    v4f s0 = red[((0 * TN + 0) * TM + tm) * 64 + lane], s1 = red[((0 * TN + 1) * TM + tm) * 64 + lane];
-#pragma unroll
-    for (int w = 1; w < NW; ++w) {
-        s0 += red[((w * TN + 0) * TM + tm) * 64 + lane];
-        s1 += red[((w * TN + 1) * TM + tm) * 64 + lane];
-    }
     float scale = p.alpha;
     if (p.As) scale *= p.As[0];
     if (p.Bs) scale *= p.Bs[0];
     const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;
-    const int rt = tm * 16 + li, col = n0 + lg * 8;
-    if (rt >= rows_valid || col >= p.N) return;
-    store8(p.C, p.out_type, m0 + rt, col, p.N, s0 * scale, s1 * scale, p.beta, vec_ok);
+    const int col = n0 + lg * 8;
+    // wave w finishes row groups w, w + 4, ...
+    for (int tm = wave; tm < TM; tm += NW) {
+        const int rt = tm * 16 + li;
+#pragma unroll
+        for (int tp = 0; tp < TN / 2; ++tp) {
+            v4f s0 = red[((0 * TN + 2 * tp) * TM + tm) * 64 + lane], s1 = red[((0 * TN + 2 * tp + 1) * TM + tm) * 64 + lane];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) {
+                s0 += red[((w * TN + 2 * tp) * TM + tm) * 64 + lane];
+                s1 += red[((w * TN + 2 * tp + 1) * TM + tm) * 64 + lane];
+            }
+            const int c = col + tp * 32;
+            if (rt < rows_valid && c < p.N) store8(p.C, p.out_type, m0 + rt, c, p.N, s0 * scale, s1 * scale, p.beta, vec_ok);
+        }
+    }
 #endif
 }
 
-template <int BM, int STAGES>
+template <int BM, int BN, int STAGES>
 inline hipError_t launch_tile_mid(const GemmParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL((fp8_gemm_tile_mid_kernel<BM, STAGES>), dim3((p.N + 31) / 32, (p.M + BM - 1) / BM, 1), dim3(256, 1, 1), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_tile_mid_kernel<BM, BN, STAGES>), dim3((p.N + BN - 1) / BN, (p.M + BM - 1) / BM, 1), dim3(256, 1, 1), 0, stream, p);
     return hipGetLastError();
 }
 

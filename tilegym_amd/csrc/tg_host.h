@@ -24,7 +24,7 @@ hipError_t run_tile_per_tensor(int bm, int bn, bool split, const GemmParams& p, 
 // run_tile_per_tensor(256, 256, false, ...)
 hipError_t run_tile256(const GemmParams& p, int gx, hipStream_t s);
 // 64x32 per-tensor tile, K split across the four waves of a workgroup (one launch; 16 < M <= ~512)
-hipError_t run_tile_mid(int bm, const GemmParams& p, hipStream_t s);
+hipError_t run_tile_mid(int bm, int bn, const GemmParams& p, hipStream_t s);
 // 64x128 per-tensor tile with four LDS stages (loads three K steps ahead): the 16 < M <= 64 form
 hipError_t run_tile_deep(bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
 hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);

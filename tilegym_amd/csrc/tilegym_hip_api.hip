@@ -136,8 +136,11 @@ void remember(const Schedule& s) {
     g_last_cfg[TG_CFG_WAVES] = s.waves;
 }
 
+// Tiles of fp8_gemm_tile_mid_kernel.
+bool is_mid_tile(int bm, int bn) { return ((bm == 64 || bm == 32) && bn == 32) || (bm == 64 && bn == 64); }
+
 bool tile_exists(int bm, int bn, bool block_scaled) {
-    if ((bm == 64 || bm == 32) && bn == 32) return !block_scaled;  // the four waves split K inside the workgroup (per-tensor only)
+    if (is_mid_tile(bm, bn)) return !block_scaled;  // the four waves split K inside the workgroup (per-tensor only)
     if (bm == 128 && bn == 128) return true;
     if (bm == 128 && bn == 256) return true;
     if (bm == 64 && bn == 128) return true;
@@ -252,6 +255,10 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         const bool small_w = !block_scaled && M <= 128 && N * K <= ((int64_t)32 << 20) && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1;
         if (small_w && M <= 64 && tiles(32, 32) <= 256) { bm = 32; bn = 32; }
         else if (small_w && tiles(64, 32) <= 256) { bm = 64; bn = 32; }
+        // 128 < M <= 256: the same scheme at 64 x 64 (half the operand bytes per output of the 32-wide tiles) while one
+        // round covers the problem (4096 x 4096 weight: 15.5 / 15.7 us at M = 192 / 256 against 16.3 / 17.7)
+        else if (!block_scaled && M > 128 && M <= 256 && N * K <= ((int64_t)32 << 20) && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1 &&
+                 tiles(64, 64) <= 256) { bm = 64; bn = 64; }
         else if (M <= 64 || (!block_scaled && tiles(64, 128) <= 256)) { bm = 64; bn = 128; }
         else if (tiles(256, 256) >= 200 && s256 >= s128) { bm = 256; bn = 256; }
         else if (!block_scaled && tiles(128, 256) >= 200 && tiles(256, 256) < 200) { bm = 128; bn = 256; }
@@ -262,7 +269,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     s.bn = bn;
     const int64_t wgs = cdiv(M, bm) * cdiv(N, bn);
     s.split_k = 1;
-    if (bn == 32) return s;  // K is split inside the workgroup: one launch
+    if (is_mid_tile(bm, bn)) return s;  // K is split inside the workgroup: one launch
     if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
     } else if (want_split < 0 && bm == 64 && bn == 128 && !block_scaled) {
@@ -536,11 +543,11 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         int gx = (int)(cdiv(rows, s.bm) * cdiv(N, s.bn));
         const bool split = pc.split_k > 1;
         const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128;
-        const bool mid = s.kernel == 1 && !block_scaled && s.bn == 32;
+        const bool mid = s.kernel == 1 && !block_scaled && is_mid_tile(s.bm, s.bn);
         // hand-ordered K loop for the dense per-tensor 256x256 tile (WAVES = 4 asks for the generic form with four loader waves)
         const bool ordered = s.kernel == 1 && !block_scaled && !split && s.bm == 256 && s.bn == 256 &&
                              cfg_get(cfg, ncfg, TG_CFG_WAVES) != 4;
-        hipError_t e = mid ? tg::run_tile_mid(s.bm, pc, stream)
+        hipError_t e = mid ? tg::run_tile_mid(s.bm, s.bn, pc, stream)
                      : ordered ? tg::run_tile256(pc, gx, stream)
                      : deep ? tg::run_tile_deep(split, pc, gx, pc.split_k, stream)
                      : block_scaled ? tg::run_tile_block_dense(s.bm, s.bn, split, pc, gx, pc.split_k, stream)
