@@ -136,7 +136,7 @@ def test_per_tensor_mid_tiles(device, bm, bn, M, N, K):
 def test_mid_tiles_are_the_default_for_small_weights(device):
     g = _g(8)
     b = fp8_randn((4096, 4096), g, 0.02)
-    for M, want in ((32, (32, 32)), (64, (32, 32)), (128, (64, 32)), (256, (64, 64)), (320, (64, 128))):
+    for M, want in ((32, (32, 32)), (64, (32, 32)), (128, (64, 32)), (192, (64, 64)), (256, (64, 64)), (320, (64, 128))):
         a = fp8_randn((M, 4096), g)
         out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
         cfg = used("tiled")

@@ -248,17 +248,15 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // the three-stage 64x128 kernel (per-tensor) also wins above 64 rows while its tiles fit one round of the
         // chip: 13.3 / 14.5 / 17.8 / 18.1 us against 17.1 / 18.8 / 18.7 / 21.6 for M = 96 / 128 / 256 / 512 at
         // N = K = 4096; with more tiles the larger tiles' operand reuse wins (M = 1024: 32 vs 23 us)
-        // small weights at 16 < M <= 128: narrow tiles whose four waves split K inside the workgroup fill the chip in
-        // one launch, where the 64x128 tile needs split-K and a reduction launch (4096 x 4096 weight: 8.8 / 8.8 / 10.3 us
-        // at M = 32 / 64 / 128 against 10.4 / 12.0 / 14.7; 6144 x 4096: 9.2 / 10.9 against 11.8 / 13.3 at M = 32 / 64).
-        // Beyond one round of workgroups, or when the weights dominate (>= 32 MiB), the activation re-reads cost more.
-        const bool small_w = !block_scaled && M <= 128 && N * K <= ((int64_t)32 << 20) && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1;
+        // small weights at 16 < M <= 256: narrow tiles whose four waves split K inside the workgroup fill the chip in
+        // one launch, where the 64x128 tile needs split-K and a reduction launch (4096 x 4096 weight: 7.9 / 7.9 / 9.8 /
+        // 12.5 us at M = 32 / 64 / 128 / 256 against 10.4 / 12.0 / 14.7 / 17.6; 6144 x 4096: 9.4 / 10.2 / 12.9 against
+        // 11.8 / 13.3 / 16.7 at M = 32 / 64 / 128).  Beyond one round of workgroups, or when the weights dominate
+        // (>= 32 MiB), the activation re-reads cost more.
+        const bool small_w = !block_scaled && M <= 256 && N * K <= ((int64_t)32 << 20) && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1;
         if (small_w && M <= 64 && tiles(32, 32) <= 256) { bm = 32; bn = 32; }
-        else if (small_w && tiles(64, 32) <= 256) { bm = 64; bn = 32; }
-        // 128 < M <= 256: the same scheme at 64 x 64 (half the operand bytes per output of the 32-wide tiles) while one
-        // round covers the problem (4096 x 4096 weight: 15.5 / 15.7 us at M = 192 / 256 against 16.3 / 17.7)
-        else if (!block_scaled && M > 128 && M <= 256 && N * K <= ((int64_t)32 << 20) && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1 &&
-                 tiles(64, 64) <= 256) { bm = 64; bn = 64; }
+        else if (small_w && M <= 128 && tiles(64, 32) <= 256) { bm = 64; bn = 32; }
+        else if (small_w && M > 64 && tiles(64, 64) <= 256) { bm = 64; bn = 64; }
         else if (M <= 64 || (!block_scaled && tiles(64, 128) <= 256)) { bm = 64; bn = 128; }
         else if (tiles(256, 256) >= 200 && s256 >= s128) { bm = 256; bn = 256; }
         else if (!block_scaled && tiles(128, 256) >= 200 && tiles(256, 256) < 200) { bm = 128; bn = 256; }
