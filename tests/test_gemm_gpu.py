@@ -144,6 +144,53 @@ def test_mid_tiles_are_the_default_for_small_weights(device):
         check(out, R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True), what=f"M={M} default")
 
 
+def test_weights_of_2_gib_and_more_run_in_column_chunks(device):
+    """A (N, K) weight of 2 GiB or more cannot be indexed with 32-bit byte offsets: the columns of C are computed in
+    chunks of weight rows on the fast kernels (streaming for M = 8, tiled for M = 40), not on the software-decode
+    fallback.  Checked against the oracle on sampled columns, among them both sides of the chunk boundary and the
+    last column, with per-tensor and with block scales."""
+    K = 16384
+    N = (1 << 31) // K + 520          # 2 GiB + 8.1 MiB of weights; N is a multiple of 8, not of 128
+    chunk = ((1 << 31) - 1) // K // 256 * 256
+    g = _g(77)
+    codes = torch.randint(0, 256, (N, K), dtype=torch.uint8, device=device)
+    codes[(codes & 0x7F) == 0x7F] = 0x38          # no NaN codes
+    codes &= 0xBF                                  # |value| < 2: sums stay well inside bf16's range
+    b_dev = codes.view(torch.float8_e4m3fn)
+    cols = torch.tensor(sorted({0, 1, 127, 128, chunk - 1, chunk, chunk + 1, chunk + 255, N - 129, N - 2, N - 1}
+                               | set(torch.randint(0, N, (64,), generator=g).tolist())))
+    b_cols = b_dev[cols.to(device)].cpu()
+    for M, kernel in ((8, "stream"), (40, "tiled")):
+        a = fp8_randn((M, K), g)
+        sa, sb = torch.tensor([0.02]), torch.tensor([0.01])
+        out = matmul(a.to(device), b_dev, trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device), out_dtype=torch.bfloat16)
+        used(kernel)
+        ref = R.ref_gemm_per_tensor(a, b_cols, sa, sb, trans_b=True)
+        check(out[:, cols.to(device)], ref, what=f"2 GiB weight, per-tensor, M={M}")
+        # block scales: (M, K/128) and (ceil(N/128), K/128)
+        As = torch.rand(M, K // 128, generator=g) * 0.02 + 0.01
+        Bs = torch.rand((N + 127) // 128, K // 128, generator=g) * 0.02 + 0.01
+        out = w8a8_block_fp8_matmul(a.to(device), b_dev, As.to(device), Bs.to(device), [128, 128], torch.bfloat16)
+        used(kernel)
+        a_deq = a.float().view(M, K // 128, 128) * As[:, :, None]
+        b_deq = b_cols.float().view(len(cols), K // 128, 128) * Bs[cols // 128][:, :, None]
+        ref = (a_deq.reshape(M, K).double() @ b_deq.reshape(len(cols), K).double().T).to(torch.bfloat16)
+        check(out[:, cols.to(device)], ref, what=f"2 GiB weight, block scales, M={M}")
+    del codes, b_dev
+
+
+def test_fallback_kernel_takes_more_rows_than_one_grid_dimension_holds(device):
+    """The software-decode kernel walks rows grid-stride: 300 000 rows (above 4 x 65 535) of a K that no fast kernel
+    takes (K % 16 != 0)."""
+    M, N, K = 300_000, 8, 24
+    g = _g(78)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.5, scale_b=0.25, out_dtype=torch.bfloat16)
+    used("fallback")
+    rows = torch.tensor([0, 1, 262139, 262140, 262143, 262144, 299_999] + torch.randint(0, M, (200,), generator=g).tolist())
+    check(out[rows.to(device)], R.ref_gemm_per_tensor(a[rows], b, 0.5, 0.25, trans_b=True), what="fallback, 300000 rows")
+
+
 # ----------------------------------------------------------------------------- skinny
 @pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K,rg,split,waves", [(1000, 512, 1, 1, 4), (4096, 1024, 2, 2, 8), (520, 2064, 4, 4, 16), (256, 128, 1, 1, 16)])

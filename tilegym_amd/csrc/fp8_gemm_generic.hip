@@ -6,11 +6,18 @@
 
 namespace tg {
 
+__device__ void generic_row(const GenericParams& q, int n, int r);
+
 __global__ void __launch_bounds__(256) fp8_gemm_generic_kernel(const GenericParams q) {
     const GemmParams& p = q.g;
     const int n = blockIdx.x * 64 + threadIdx.x;
-    const int r = blockIdx.y * 4 + threadIdx.y;
-    if (n >= p.N || r >= q.rows) return;
+    if (n >= p.N) return;
+    // rows: grid-stride (grid.y is capped at the launch limit)
+    for (int r = blockIdx.y * 4 + threadIdx.y; r < q.rows; r += gridDim.y * 4) generic_row(q, n, r);
+}
+
+__device__ void generic_row(const GenericParams& q, int n, int r) {
+    const GemmParams& p = q.g;
     int arow = r, crow = r, e = 0;
     if (q.group == GROUP_RAGGED) {
         e = -1;
@@ -49,7 +56,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_generic_kernel(const GenericPara
     }
     if (q.group == GROUP_GATHER && p.row_weight) scale *= p.row_weight[crow];
     float v = acc * scale;
-    const int64_t at = (int64_t)crow * p.N + n;
+    const int64_t at = (int64_t)crow * p.ldc + n;
     if (p.out_type == OUT_BF16) {
         __bf16* c = reinterpret_cast<__bf16*>(p.C) + at;
         if (p.beta != 0.f) v += p.beta * (float)(*c);
@@ -71,7 +78,8 @@ __global__ void __launch_bounds__(256) fp8_gemm_generic_kernel(const GenericPara
 
 hipError_t run_generic(const GenericParams& q, hipStream_t s) {
     if (q.rows <= 0 || q.g.N <= 0) return hipSuccess;
-    dim3 grid((q.g.N + 63) / 64, (q.rows + 3) / 4, 1);
+    const int gy = (q.rows + 3) / 4;
+    dim3 grid((q.g.N + 63) / 64, gy < 65535 ? gy : 65535, 1);
     hipLaunchKernelGGL(fp8_gemm_generic_kernel, grid, dim3(64, 4, 1), 0, s, q);
     return hipGetLastError();
 }
@@ -126,7 +134,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmParams p, 
         if (p.As) scale *= p.As[0];
         if (p.Bs) scale *= p.Bs[0];
     }
-    store4(p.C, p.out_type, m, col, p.N, sum * scale, p.beta, vec_ok);
+    store4(p.C, p.out_type, m, col, p.N, p.ldc, sum * scale, p.beta, vec_ok);
 }
 
 hipError_t run_splitk_reduce(const GemmParams& p, bool block_scaled, hipStream_t s) {

@@ -145,7 +145,7 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_skinny_kernel(const GemmPara
 #pragma unroll
             for (int rg = 0; rg < RG; ++rg) {
                 const int col = n_base + rg * 16 + lg * 4;
-                if (col < N) store4(mine, OUT_F32, m, col, N, acc[rg][mt], 0.f, vec_ok);
+                if (col < N) store4(mine, OUT_F32, m, col, N, N, acc[rg][mt], 0.f, vec_ok);
             }
         }
         return;
@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_skinny_kernel(const GemmPara
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg) {
             const int col = n_base + rg * 16 + lg * 4;
-            if (col < N) store4(p.C, p.out_type, m, col, N, acc[rg][mt] * scale, p.beta, vec_ok);
+            if (col < N) store4(p.C, p.out_type, m, col, N, p.ldc, acc[rg][mt] * scale, p.beta, vec_ok);
         }
     }
 }

@@ -217,7 +217,7 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_kernel(const GemmPara
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + li;
-            if (m < M && col < N) store4(mine, OUT_F32, m, col, N, acc[mt], 0.f, vec_ok);
+            if (m < M && col < N) store4(mine, OUT_F32, m, col, N, N, acc[mt], 0.f, vec_ok);
         }
         return;
     }
@@ -229,7 +229,7 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_kernel(const GemmPara
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + li;
-        if (m < M && col < N) store4(p.C, p.out_type, m, col, N, acc[mt] * scale, p.beta, vec_ok);
+        if (m < M && col < N) store4(p.C, p.out_type, m, col, N, p.ldc, acc[mt] * scale, p.beta, vec_ok);
     }
 #endif
 }
@@ -334,7 +334,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmPar
     const int col = n_base + lg * 4, m = li;
     if (m >= M || col >= N) return;
     if (p.split_k > 1) {
-        store4(p.partials + (int64_t)blockIdx.y * M * N, OUT_F32, m, col, N, acc, 0.f, vec_ok);
+        store4(p.partials + (int64_t)blockIdx.y * M * N, OUT_F32, m, col, N, N, acc, 0.f, vec_ok);
         return;
     }
     float scale = p.alpha;
@@ -342,7 +342,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmPar
         if (p.As) scale *= p.As[0];
         if (p.Bs) scale *= p.Bs[0];
     }
-    store4(p.C, p.out_type, m, col, N, acc * scale, p.beta, vec_ok);
+    store4(p.C, p.out_type, m, col, N, p.ldc, acc * scale, p.beta, vec_ok);
 #endif
 }
 

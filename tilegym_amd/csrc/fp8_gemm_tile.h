@@ -142,10 +142,10 @@ __device__ __forceinline__ void ragged_find(const int* indptr, int E, int BM, in
     }
 }
 
-// Write 8 consecutive outputs C[row][col..col+7] = v (+ beta * old), masked against N.
-__device__ __forceinline__ void store8(void* C, int out_type, int64_t row, int col, int N,
+// Write 8 consecutive outputs C[row][col..col+7] = v (+ beta * old), masked against N columns; ld = row stride.
+__device__ __forceinline__ void store8(void* C, int out_type, int64_t row, int col, int N, int ld,
                                        v4f lo, v4f hi, float beta, bool vec_ok) {
-    const int64_t base = row * (int64_t)N + col;
+    const int64_t base = row * (int64_t)ld + col;
     if (vec_ok && col + 7 < N) {
         if (out_type == OUT_F32) {
             v4f* p = reinterpret_cast<v4f*>(reinterpret_cast<float*>(C) + base);
@@ -775,9 +775,9 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
                 const int col = n0 + wn * WTN + tp * 32 + lg * 8;
                 if (dsts[tm] < 0 || col >= p.N) continue;
                 if constexpr (SPLIT)
-                    store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, dsts[tm], col, p.N, acc[2 * tp][tm], acc[2 * tp + 1][tm], 0.f, vec_ok);
+                    store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, dsts[tm], col, p.N, p.N, acc[2 * tp][tm], acc[2 * tp + 1][tm], 0.f, vec_ok);
                 else
-                    store8(p.C, OT, dsts[tm], col, p.N, acc[2 * tp][tm] * rws[tm], acc[2 * tp + 1][tm] * rws[tm], p.beta, vec_ok);
+                    store8(p.C, OT, dsts[tm], col, p.N, p.ldc, acc[2 * tp][tm] * rws[tm], acc[2 * tp + 1][tm] * rws[tm], p.beta, vec_ok);
             }
         }
     };
@@ -809,7 +809,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN, (WGM * WGN == 4 ? 2 : 1)) fp8_
     GemmParams p{};
     p.A = gl.prob[i].A; p.B = gl.prob[i].B; p.C = gl.prob[i].C;
     p.As = gl.prob[i].As; p.Bs = gl.prob[i].Bs;
-    p.M = gl.prob[i].M; p.N = gl.prob[i].N; p.K = gl.prob[i].K;
+    p.M = gl.prob[i].M; p.N = gl.prob[i].N; p.K = gl.prob[i].K; p.ldc = p.N;
     p.kblocks = p.K / kKBlock; p.nblocks = (p.N + 127) / 128;
     p.alpha = gl.alpha; p.beta = 0.f;
     p.out_type = gl.out_type;

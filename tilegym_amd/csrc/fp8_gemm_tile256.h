@@ -190,7 +190,7 @@ __global__ void __launch_bounds__(512, 1) fp8_gemm_tile256_kernel(const GemmPara
             for (int tp = 0; tp < TN / 2; ++tp) {
                 const int col = n0 + wn * WTN + tp * 32 + lg * 8;
                 if (dsts[tm] < 0 || col >= p.N) continue;
-                store8(p.C, OT, dsts[tm], col, p.N, acc[2 * tp][tm] * scale, acc[2 * tp + 1][tm] * scale, p.beta, vec_ok);
+                store8(p.C, OT, dsts[tm], col, p.N, p.ldc, acc[2 * tp][tm] * scale, acc[2 * tp + 1][tm] * scale, p.beta, vec_ok);
             }
         }
     };

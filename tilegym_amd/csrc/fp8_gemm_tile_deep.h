@@ -168,9 +168,9 @@ __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmPa
             const int rt = tm * 16 + li;
             if (rt >= rows_valid || col >= p.N) continue;
             if constexpr (SPLIT)
-                store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, m0 + rt, col, p.N, acc[0][tm], acc[1][tm], 0.f, vec_ok);
+                store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, m0 + rt, col, p.N, p.N, acc[0][tm], acc[1][tm], 0.f, vec_ok);
             else
-                store8(p.C, OT, m0 + rt, col, p.N, acc[0][tm] * scale, acc[1][tm] * scale, p.beta, vec_ok);
+                store8(p.C, OT, m0 + rt, col, p.N, p.ldc, acc[0][tm] * scale, acc[1][tm] * scale, p.beta, vec_ok);
         }
     };
     if (SPLIT || p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});

@@ -154,7 +154,7 @@ __global__ void __launch_bounds__(256, 1) fp8_gemm_tile_mid_kernel(const GemmPar
             s1 += red[((w * TN + 2 * tp + 1) * TM + tm) * 64 + lane];
         }
         const int c = col + tp * 32;
-        if (rt < rows_valid && c < p.N) store8(p.C, p.out_type, m0 + rt, c, p.N, s0 * scale, s1 * scale, p.beta, vec_ok);
+        if (rt < rows_valid && c < p.N) store8(p.C, p.out_type, m0 + rt, c, p.N, p.ldc, s0 * scale, s1 * scale, p.beta, vec_ok);
     }
 #endif
 }

@@ -28,6 +28,7 @@ struct GemmParams {
     const float* As;    // per-tensor: 1 float or null.  block: (M, kblocks)
     const float* Bs;    // per-tensor: 1 float or null.  block: ([E,] nblocks, kblocks)
     int M, N, K;
+    int ldc;               // row stride of C in elements (N, or the full width when the columns are computed in chunks)
     int kblocks, nblocks;  // ceil(K/128), ceil(N/128)
     float alpha, beta;
     int out_type;
@@ -111,10 +112,10 @@ __device__ __forceinline__ int pack_e4m3x4(float a, float b, float c, float d) {
 }
 __device__ __forceinline__ uint8_t f32_to_e4m3(float x) { return (uint8_t)(pack_e4m3x4(x, 0.f, 0.f, 0.f) & 0xFF); }
 
-// Store 4 consecutive outputs C[row][col..col+3] = v (+ beta * old), masked against ncols.
-__device__ __forceinline__ void store4(void* C, int out_type, int64_t row, int col, int N, v4f v,
+// Store 4 consecutive outputs C[row][col..col+3] = v (+ beta * old), masked against N columns; ld = row stride.
+__device__ __forceinline__ void store4(void* C, int out_type, int64_t row, int col, int N, int ld, v4f v,
                                        float beta, bool vec_ok) {
-    int64_t base = row * (int64_t)N + col;
+    int64_t base = row * (int64_t)ld + col;
     if (vec_ok && col + 3 < N) {
         if (out_type == OUT_BF16) {
             bf16x4* p = reinterpret_cast<bf16x4*>(reinterpret_cast<__bf16*>(C) + base);

@@ -81,6 +81,7 @@ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 constexpr int64_t kOffsetLimit = (int64_t)1 << 31;  // kernels index operands with 32-bit byte offsets
+thread_local int64_t g_chunk_ldc = 0;               // row stride of C for the next fp8_gemm_impl call (column chunks), 0 = N
 constexpr int kTargetWaves = 4096;                  // 16 waves on each of 256 CUs
 
 // Switches to the caller's device for the lifetime of a call.
@@ -374,6 +375,10 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
                       int32_t device_id, uint64_t hip_stream) {
     g_err[0] = 0;
     int32_t rc;
+    // (a column chunk of a wider C, handed down by the chunk loop below, is described as (M, chunk) with its real row
+    // stride in g_chunk_ldc)
+    const int64_t chunk_ldc = g_chunk_ldc;
+    g_chunk_ldc = 0;
     if ((rc = check_tensor(a, "a", 2)) || (rc = check_tensor(b, "b", 2)) || (rc = check_tensor(c, "c", 2))) return rc;
     if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN)
         return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7), got %d and %d", a->dtype, b->dtype);
@@ -386,6 +391,36 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         return fail(TG_ERR_INVALID, "c must be (%lld, %lld), got (%lld, %lld)", (long long)M, (long long)N, (long long)c->shape[0], (long long)c->shape[1]);
     if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return fail(TG_ERR_INVALID, "extent exceeds int32");
     const int64_t kblocks = cdiv(K, 128), nblocks = cdiv(N, 128);
+    const int64_t ldc = chunk_ldc ? chunk_ldc : N;
+
+    // ---- weights of 2 GiB and more: the kernels index an operand with 32-bit byte offsets, so the columns of C are
+    // computed in chunks of weight rows that stay below that (same stream, same workspace, one after the other)
+    if (!chunk_ldc && trans_b && !trans_a && N * K >= kOffsetLimit && K > 0 && (K % 16) == 0 && 256 * K < kOffsetLimit &&
+        aligned16(a->ptr) && aligned16(b->ptr) && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0 && M > 0) {
+        const bool b_block = scale_b && numel(scale_b) != 1;
+        const int64_t chunk_n = ((kOffsetLimit - 1) / K) / 256 * 256;
+        for (int64_t n0 = 0; n0 < N; n0 += chunk_n) {
+            const int64_t cn = (N - n0) < chunk_n ? (N - n0) : chunk_n;
+            tg_tensor bs = *b, cs = *c, sbs;
+            bs.ptr = b->ptr + (uint64_t)(n0 * K);
+            bs.shape[0] = cn;
+            cs.ptr = c->ptr + (uint64_t)(n0 * elem_size(c->dtype));
+            cs.shape[1] = cn;
+            cs.strides[0] = cn;  // described as contiguous; the real row stride travels in g_chunk_ldc
+            const tg_tensor* sb = scale_b;
+            if (b_block) {
+                sbs = *scale_b;
+                sbs.ptr = scale_b->ptr + (uint64_t)((n0 / 128) * kblocks * 4);
+                sbs.shape[0] = cdiv(cn, 128);
+                sb = &sbs;
+            }
+            g_chunk_ldc = N;
+            rc = fp8_gemm_impl(&cs, a, &bs, scale_a, sb, trans_a, trans_b, alpha, beta, workspace, static_scratch, cfg, ncfg, device_id, hip_stream);
+            g_chunk_ldc = 0;
+            if (rc) return rc;
+        }
+        return TG_OK;
+    }
 
     // ---- scales
     enum Kind { NONE, TENSOR, BLOCK };
@@ -471,10 +506,11 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
     p.As = scale_a ? reinterpret_cast<const float*>(scale_a->ptr) : nullptr;
     p.Bs = scale_b ? reinterpret_cast<const float*>(scale_b->ptr) : nullptr;
     p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    p.ldc = (int)ldc;
     p.kblocks = (int)kblocks; p.nblocks = (int)nblocks;
     p.alpha = alpha; p.beta = beta;
     p.out_type = out_type;
-    p.vec_store = ((N % 4) == 0 && aligned16(c->ptr)) ? 1 : 0;
+    p.vec_store = ((N % 4) == 0 && aligned16(c->ptr) && (ldc == N || (ldc * elem_size(c->dtype)) % 16 == 0)) ? 1 : 0;
     p.split_k = 1;
     p.ksteps_per_split = (int)kblocks;
     p.E = 1; p.top_k = 1;
@@ -602,7 +638,7 @@ static void fill_grouped(tg::GemmParams& p, const tg_tensor* c, const tg_tensor*
     p.C = reinterpret_cast<void*>(c->ptr);
     p.As = a_scale ? reinterpret_cast<const float*>(a_scale->ptr) : nullptr;
     p.Bs = b_scale ? reinterpret_cast<const float*>(b_scale->ptr) : nullptr;
-    p.M = (int)rows_c; p.N = (int)N; p.K = (int)K;
+    p.M = (int)rows_c; p.N = (int)N; p.K = (int)K; p.ldc = (int)N;
     p.kblocks = (int)cdiv(K, 128); p.nblocks = (int)cdiv(N, 128);
     p.alpha = 1.0f; p.beta = 0.0f;
     p.out_type = out_type;
@@ -799,7 +835,7 @@ int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, 
     p.C = reinterpret_cast<void*>(q->ptr);
     p.As = reinterpret_cast<const float*>(a_scale->ptr);
     p.Bs = reinterpret_cast<const float*>(b_scale->ptr);
-    p.M = (int)num_valid; p.N = (int)N; p.K = (int)K;
+    p.M = (int)num_valid; p.N = (int)N; p.K = (int)K; p.ldc = (int)N;
     p.kblocks = (int)(K / 128); p.nblocks = (int)(N / 128);
     p.alpha = 1.0f; p.beta = 0.0f;
     p.out_type = act_dtype == TG_BF16 ? tg::OUT_BF16 : tg::OUT_F16;
