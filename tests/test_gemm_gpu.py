@@ -179,6 +179,27 @@ def test_weights_of_2_gib_and_more_run_in_column_chunks(device):
     del codes, b_dev
 
 
+@pytest.mark.parametrize("block_size", [[64, 64], [64, 128], [256, 32], [128, 256], [48, 80]])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 256, 256), (33, 200, 328)])
+def test_block_scaled_quantization_blocks_other_than_128(device, block_size, M, N, K):
+    """w8a8_block_fp8_matmul with the reference's block_size=[block_n, block_k] argument
+    (src/tilegym/suites/unsloth/cutile/fp8.py:388-446) for blocks other than 128 x 128, ragged at both edges: these run
+    on the software-decode kernel and must match the oracle like every other form."""
+    bn, bk = block_size
+    g = _g(M + N + K + bn * 3 + bk)
+    A, B = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
+    As = torch.rand(M, -(-K // bk), generator=g) * 0.05 + 0.01
+    Bs = torch.rand(-(-N // bn), -(-K // bk), generator=g) * 0.05 + 0.01
+    ref = R.ref_w8a8_block_fp8_matmul(A, B, As, Bs, block_size, torch.bfloat16)
+    out = w8a8_block_fp8_matmul(A.to(device), B.to(device), As.to(device), Bs.to(device), block_size, torch.bfloat16)
+    used("fallback")
+    check(out, ref, what=f"block_size={block_size} M={M} N={N} K={K}")
+    # the same problem described with 128 x 128 scales has other shapes: the library must refuse the mismatch
+    if (As.shape[1], Bs.shape) != (-(-K // 128), (-(-N // 128), -(-K // 128))):
+        with pytest.raises(RuntimeError):
+            _lib.fp8_gemm(out, A.to(device), B.to(device), As.to(device), Bs.to(device), False, True, 1.0, 0.0, None)
+
+
 def test_fallback_kernel_takes_more_rows_than_one_grid_dimension_holds(device):
     """The software-decode kernel walks rows grid-stride: 300 000 rows (above 4 x 65 535) of a K that no fast kernel
     takes (K % 16 != 0)."""

@@ -174,6 +174,21 @@ def test_block_scaled_oracle_against_loops_and_c(M, N, K):
     assert np.allclose(c, want.numpy(), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("bn,bk", [(64, 64), (256, 32), (48, 80)])
+def test_block_scaled_oracle_with_other_quantization_blocks_against_loops(bn, bk):
+    """block_size=[block_n, block_k] other than 128 x 128 (the reference's general form,
+    tests/suites/unsloth/test_fp8.py:159-191): the vectorised oracle against the element-by-element loop."""
+    g = _g(70 + bn + bk)
+    M, N, K = 5, 150, 200
+    A = (torch.randn(M, K, generator=g) * 0.1).to(FP8)
+    B = (torch.randn(N, K, generator=g) * 0.1).to(FP8)
+    As = torch.rand(M, -(-K // bk), generator=g) + 0.1
+    Bs = torch.rand(-(-N // bn), -(-K // bk), generator=g) + 0.1
+    want = _loop_block_gemm(A, B, As, Bs, bn, bk)
+    got = R.ref_w8a8_block_fp8_matmul(A, B, As, Bs, [bn, bk])
+    assert torch.allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
 def test_block_scaled_invariants():
     g = _g(8)
     M, N, K = 4, 256, 256

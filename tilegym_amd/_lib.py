@@ -21,7 +21,8 @@ DEFAULT_LIB_PATH = os.path.join(_HERE, "libtilegym_hip.so")
 
 TG_MAX_DIMS = 5
 TG_CFG_COUNT = 8
-CFG_SLOTS = {"KERNEL": 0, "BLOCK_M": 1, "BLOCK_N": 2, "SPLIT_K": 3, "ROW_GROUPS": 4, "WAVES": 5}
+CFG_SLOTS = {"KERNEL": 0, "BLOCK_M": 1, "BLOCK_N": 2, "SPLIT_K": 3, "ROW_GROUPS": 4, "WAVES": 5,
+             "QUANT_BLOCK_N": 6, "QUANT_BLOCK_K": 7}
 KERNEL_NAMES = {0: "fallback", 1: "tiled", 2: "skinny", 3: "stream"}
 
 # dtype codes of the ABI (include/tilegym_hip.h)
@@ -154,7 +155,7 @@ def _ref(d: Optional[TgTensor]):
 def make_cfg(kernel_configs: Optional[dict]):
     """``kernel_configs={...}`` (the reference's per-call override, src/tilegym/kernel_utils.py:14-36)
     -> (int32 array, length).  Keys: KERNEL ('fallback'|'tiled'|'skinny' or 0/1/2), BLOCK_M, BLOCK_N,
-    SPLIT_K, ROW_GROUPS; unknown keys (e.g. num_ctas, occupancy) are ignored."""
+    SPLIT_K, ROW_GROUPS, WAVES, QUANT_BLOCK_N, QUANT_BLOCK_K; unknown keys (e.g. num_ctas, occupancy) are ignored."""
     arr = (ctypes.c_int32 * TG_CFG_COUNT)(*([-1] * TG_CFG_COUNT))
     if kernel_configs:
         for key, val in kernel_configs.items():

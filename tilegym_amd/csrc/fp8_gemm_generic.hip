@@ -37,15 +37,18 @@ __device__ void generic_row(const GenericParams& q, int n, int r) {
     const uint8_t* a = p.A + (int64_t)arow * q.a_sm;
     const uint8_t* b = p.B + (int64_t)e * q.b_se + (int64_t)n * q.b_sn;
     float acc = 0.f;
-    for (int kb = 0; kb < p.kblocks; ++kb) {
-        const int k_hi = min((kb + 1) * kKBlock, p.K);
+    // one partial sum per quantization block of K (128 elements unless the caller's blocks differ), scaled, then added
+    const int qbk = q.block_scaled ? q.qbk : kKBlock, qbn = q.block_scaled ? q.qbn : 128;
+    const int nkq = (p.K + qbk - 1) / qbk, nnq = (p.N + qbn - 1) / qbn;
+    for (int kb = 0; kb < nkq; ++kb) {
+        const int k_hi = min((kb + 1) * qbk, p.K);
         float part = 0.f;
-        for (int k = kb * kKBlock; k < k_hi; ++k)
+        for (int k = kb * qbk; k < k_hi; ++k)
             part += e4m3_to_f32(a[(int64_t)k * q.a_sk]) * e4m3_to_f32(b[(int64_t)k * q.b_sk]);
         float s = 1.0f;
         if (q.block_scaled) {
-            if (p.As) s *= p.As[(int64_t)arow * p.kblocks + kb];
-            if (p.Bs) s *= p.Bs[((int64_t)e * p.nblocks + n / 128) * p.kblocks + kb];
+            if (p.As) s *= p.As[(int64_t)arow * nkq + kb];
+            if (p.Bs) s *= p.Bs[((int64_t)e * nnq + n / qbn) * nkq + kb];
         }
         acc += part * s;
     }

@@ -13,6 +13,7 @@ struct GenericParams {
     int64_t b_se;            // element stride between experts
     int group;               // GroupMode
     int block_scaled;        // 0 per-tensor, 1 block
+    int qbn, qbk;            // block-scaled: weight rows and K elements per scale (128 x 128 on the MFMA kernels; any here)
     int rows;                // row slots to visit (M, or the sorted-slot capacity in gather mode)
 };
 

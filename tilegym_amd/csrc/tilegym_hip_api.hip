@@ -392,10 +392,16 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
     if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return fail(TG_ERR_INVALID, "extent exceeds int32");
     const int64_t kblocks = cdiv(K, 128), nblocks = cdiv(N, 128);
     const int64_t ldc = chunk_ldc ? chunk_ldc : N;
+    // quantization blocks: 128 weight rows x 128 K elements unless cfg[] says otherwise
+    int64_t qbn = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_N), qbk = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_K);
+    if (qbn <= 0) qbn = 128;
+    if (qbk <= 0) qbk = 128;
+    const bool std_blocks = qbn == 128 && qbk == 128;
+    const int64_t sk_cols = cdiv(K, qbk), sb_rows = cdiv(N, qbn);
 
     // ---- weights of 2 GiB and more: the kernels index an operand with 32-bit byte offsets, so the columns of C are
     // computed in chunks of weight rows that stay below that (same stream, same workspace, one after the other)
-    if (!chunk_ldc && trans_b && !trans_a && N * K >= kOffsetLimit && K > 0 && (K % 16) == 0 && 256 * K < kOffsetLimit &&
+    if (!chunk_ldc && std_blocks && trans_b && !trans_a && N * K >= kOffsetLimit && K > 0 && (K % 16) == 0 && 256 * K < kOffsetLimit &&
         aligned16(a->ptr) && aligned16(b->ptr) && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0 && M > 0) {
         const bool b_block = scale_b && numel(scale_b) != 1;
         const int64_t chunk_n = ((kOffsetLimit - 1) / K) / 256 * 256;
@@ -422,7 +428,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         return TG_OK;
     }
 
-    // ---- scales
+    // ---- scales (blocks other than 128 x 128 are taken by the fallback kernel only)
     enum Kind { NONE, TENSOR, BLOCK };
     auto kind_of = [&](const tg_tensor* s, const char* name, int64_t rows, int32_t* err) -> Kind {
         *err = TG_OK;
@@ -430,16 +436,16 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         if ((*err = check_tensor(s, name, -1))) return NONE;
         if (s->dtype != TG_F32) { *err = fail(TG_ERR_DTYPE, "%s must be f32", name); return NONE; }
         if (numel(s) == 1) return TENSOR;
-        if (s->ndim == 2 && s->shape[0] == rows && s->shape[1] == kblocks) return BLOCK;
-        *err = fail(TG_ERR_INVALID, "%s: expected 1 element or shape (%lld, %lld)", name, (long long)rows, (long long)kblocks);
+        if (s->ndim == 2 && s->shape[0] == rows && s->shape[1] == sk_cols) return BLOCK;
+        *err = fail(TG_ERR_INVALID, "%s: expected 1 element or shape (%lld, %lld)", name, (long long)rows, (long long)sk_cols);
         return NONE;
     };
     const Kind ka = kind_of(scale_a, "scale_a", M, &rc);
     if (rc) return rc;
-    const Kind kb = kind_of(scale_b, "scale_b", nblocks, &rc);
+    const Kind kb = kind_of(scale_b, "scale_b", sb_rows, &rc);
     if (rc) return rc;
     const bool block_scaled = (ka == BLOCK || kb == BLOCK);
-    if (block_scaled && (ka == TENSOR || kb == TENSOR) && !(M == 1 && kblocks == 1) && !(nblocks == 1 && kblocks == 1))
+    if (block_scaled && (ka == TENSOR || kb == TENSOR) && !(M == 1 && sk_cols == 1) && !(sb_rows == 1 && sk_cols == 1))
         return fail(TG_ERR_INVALID, "scale_a and scale_b must both be per-tensor or both be block scales");
     if (block_scaled && (trans_a || !trans_b))
         return fail(TG_ERR_INVALID, "block scales require a (M,K) and b (N,K) (trans_a=0, trans_b=1)");
@@ -488,7 +494,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
     }
 
     const bool fast_layout = !trans_a && b_is_nk && (K % 16) == 0 && aligned16(a->ptr) &&
-                             aligned16(reinterpret_cast<uint64_t>(Bnt)) && N * K < kOffsetLimit;
+                             aligned16(reinterpret_cast<uint64_t>(Bnt)) && N * K < kOffsetLimit && (!block_scaled || std_blocks);
     Schedule s = choose_dense(M, N, K, block_scaled, fast_layout, cfg, ncfg, ws_free);
     if (static_scratch) {
         // same schedule as tg_fp8_gemm with a full-size workspace, or an error: never a silently smaller split
@@ -525,6 +531,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         q.b_se = 0;
         q.group = tg::GROUP_DENSE;
         q.block_scaled = block_scaled ? 1 : 0;
+        q.qbn = (int)qbn; q.qbk = (int)qbk;
         q.rows = (int)M;
         remember(s);
         if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");
@@ -682,6 +689,7 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
         q.a_sm = K; q.a_sk = 1; q.b_sn = K; q.b_sk = 1; q.b_se = N * K;
         q.group = tg::GROUP_RAGGED;
         q.block_scaled = 1;
+        q.qbn = 128; q.qbk = 128;
         q.rows = (int)total_m;
         remember(s);
         if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");
@@ -767,6 +775,7 @@ int32_t tg_fp8_moe_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor*
         q.a_sm = K; q.a_sk = 1; q.b_sn = K; q.b_sk = 1; q.b_se = N * K;
         q.group = tg::GROUP_GATHER;
         q.block_scaled = 1;
+        q.qbn = 128; q.qbk = 128;
         q.rows = (int)EM;
         remember(s);
         if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");

@@ -104,8 +104,8 @@ def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: Optional[Sequence[int]] = No
     else:
         assert len(block_size) == 2
         block_n, block_k = block_size[0], block_size[1]
-    if (block_n, block_k) != (128, 128):
-        raise NotImplementedError("the hip backend implements 128x128 quantization blocks only")
+    if block_n <= 0 or block_k <= 0:
+        raise ValueError(f"block_size must be positive, got {block_size}")
     _require_fp8(A, B)
     N, K = B.shape
     assert A.shape[-1] == B.shape[-1]
@@ -122,8 +122,11 @@ def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: Optional[Sequence[int]] = No
         return C
     As2 = As.reshape(M, -1).float().contiguous()
     Bs2 = Bs.float().contiguous()
-    _lib.fp8_gemm(C.view(M, N), A.view(M, K), B, As2, Bs2, False, True, 1.0, 0.0,
-                  kwargs.get("kernel_configs"))
+    kc = kwargs.get("kernel_configs")
+    if (block_n, block_k) != (128, 128):
+        # quantization blocks other than 128 x 128 run on the library's software-decode kernel (correct, no MFMA)
+        kc = dict(kc or {}, QUANT_BLOCK_N=block_n, QUANT_BLOCK_K=block_k)
+    _lib.fp8_gemm(C.view(M, N), A.view(M, K), B, As2, Bs2, False, True, 1.0, 0.0, kc)
     return C
 
 
