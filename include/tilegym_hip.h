@@ -60,11 +60,11 @@ typedef struct tg_tensor {
  * (src/tilegym/kernel_utils.py:14-36). */
 enum {
     TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (direct weight streaming), 3 stream (weight streaming through LDS) */
-    TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (32/64/128/256; 32 and 64x32 = in-workgroup K split, per-tensor only) */
-    TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (32/128/256)           */
+    TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (32/64/128/256; 32x32, 64x32 and 64x64 = in-workgroup K split, per-tensor only) */
+    TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (32/64/128/256)        */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
     TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4); stream kernel: LDS buffers per wave (1/2) */
-    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup; tiled 256x256 per-tensor kernel: 4 = the generic form instead of the hand-ordered one */
+    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup; tiled 256x256 per-tensor kernel: 4 = the generic tile kernel instead of the hand-ordered one */
     TG_CFG_QUANT_BLOCK_N = 6, /* block-scaled tg_fp8_gemm: weight rows per scale (default 128) */
     TG_CFG_QUANT_BLOCK_K = 7, /* block-scaled tg_fp8_gemm: K elements per scale (default 128); blocks other than 128 x 128
                                * run on the fallback kernel (no MFMA): the reference's block_size=[bn, bk] argument,

@@ -215,7 +215,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 16, TN = WTN / 16;
     constexpr int NL = NW;                // every wave issues its share of the direct global->LDS loads
-    constexpr int RPP = 8 * NL;           // slab rows filled per pass of the loader waves
+    constexpr int RPP = 8 * NL;           // slab rows filled per pass of the waves
     constexpr int A_IT = BM / RPP, B_IT = BN / RPP;
     static_assert(NW == 4 || NW == 8, "wave grid");
     static_assert(BM % RPP == 0 && BN % RPP == 0 && NL % 2 == 0, "loader shape");
@@ -308,7 +308,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // overlaps the row maps and scale tables fetched below (which the activation loads must wait for).
     const int lrow = lane >> 3;
     // weight slab: its own swizzle (see the fragment addresses below).  Row 8g + lrow with g = i*NL + wave:
-    // NL is even, so bit 3 of the row is the parity of the loader wave.
+    // NL is even, so bit 3 of the row is the parity of the wave.
     const int ljb = (lane & 7) ^ swz_w(((wave & 1) << 3) | lrow);
     // (with NL == NW every wave loads: no test, and so no branch inside the K loop)
     uint32_t b_off[B_IT];
@@ -417,7 +417,7 @@ __device__ __forceinline__ void fp8_gemm_tile_body(const GemmParams& p, const in
     // double-buffered LDS table: one 4-byte direct load covers 8 rows x 8 consecutive K steps, i.e. 8
     // runs of 32 contiguous bytes -- fetching one K step for 64 rows would touch 64 cache lines per
     // instruction, eight times what a slab load does.  Chunk c+1 is requested while chunk c is in use,
-    // one 8-row group per loader wave and K step.  Lane l of the load for row group g lands at float
+    // one 8-row group per wave and K step.  Lane l of the load for row group g lands at float
     // 64*g + l of the chunk's buffer; it fetches row 8g + l/8 at chunk step (l%8 - l/8) % 8, so step s of
     // row r sits at position (s + r) % 8 of the row's eight floats and the 16 rows a fragment's lanes
     // read in one K step spread over the banks.

@@ -3,11 +3,11 @@
 // Same tile, wave grid (4 x 2 waves, 64 x 128 per wave), slab layout, swizzles, fragment addressing,
 // per-accumulator MFMA order and epilogue arithmetic as
 // fp8_gemm_tile_kernel<256, 256, 4, 2, false, GROUP_DENSE, false>: identical results.  What differs is
-// the schedule of one K step.  In the generic kernel four loader waves issue their sixteen direct
-// loads in two bursts of eight; while a wave waits for room in the address path (about 14 clocks per
-// 1 KiB load for the whole compute unit, whoever issues it) it issues no MFMAs, so a loader wave needs
-// load time PLUS its 1024 clocks of MFMA issue per step and the step lasts ~2.6 k clocks instead of
-// the 2048 the matrix pipe needs.  Here
+// the schedule of one K step.  The generic kernel requests the weight slab of the next step in one burst of
+// loads at the top of a step and has two barriers per step.  While a wave waits for room in the address path
+// (about 14 clocks per 1 KiB load for the whole compute unit, whoever issues it) it issues no MFMAs, so a burst
+// puts load time and MFMA time of the issuing waves in series (with four loader waves, as the generic kernel
+// once had, a step lasted ~2.6 k clocks instead of the 2048 the matrix pipe needs).  Here
 //   * all eight waves load (eight 1 KiB loads per wave and step), one load behind every group of
 //     four MFMAs: the address path sees one request per ~32 clocks and never backs up;
 //   * two activation slabs and three weight slabs (160 KiB, all of LDS) let one barrier per step do:
