@@ -200,6 +200,25 @@ def test_block_scaled_quantization_blocks_other_than_128(device, block_size, M, 
             _lib.fp8_gemm(out, A.to(device), B.to(device), As.to(device), Bs.to(device), False, True, 1.0, 0.0, None)
 
 
+@pytest.mark.parametrize("bn,bk", [(64, 64), (128, 64), (256, 32)])
+def test_ragged_quantization_blocks_other_than_128(device, bn, bk):
+    """ragged_block_scaled_bmm derives the quantization block from the scale tensor's shape, as the reference does
+    (src/tilegym/suites/flashinfer/cutile/gemm/ragged_block_scaled_bmm.py:535-537): blocks other than 128 x 128 run on the
+    software-decode kernel and match the oracle, empty experts included."""
+    g = _g(900 + bn + bk)
+    Q, N, K = 5, 256, 384
+    sizes = [37, 0, 130, 1, 64]
+    ptr = torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32)
+    total = int(ptr[-1])
+    a, b = fp8_randn((total, K), g), fp8_randn((Q, N, K), g, 0.5)
+    a_s = torch.rand(total, K // bk, generator=g) * 0.05 + 0.01
+    b_s = torch.rand(Q, N // bn, K // bk, generator=g) * 0.05 + 0.01
+    ref = R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr, block_n=bn, block_k=bk)
+    out = ragged_block_scaled_bmm(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), max(sizes))
+    used("fallback")
+    check(out, ref, what=f"ragged, blocks {bn}x{bk}")
+
+
 def test_fallback_kernel_takes_more_rows_than_one_grid_dimension_holds(device):
     """The software-decode kernel walks rows grid-stride: 300 000 rows (above 4 x 65 535) of a K that no fast kernel
     takes (K % 16 != 0)."""

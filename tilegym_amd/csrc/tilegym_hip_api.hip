@@ -607,7 +607,7 @@ extern "C" {
 // Shared validation of the two grouped entry points.
 static int32_t grouped_common(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
                               const tg_tensor* a_scale, const tg_tensor* b_scale, int64_t* rows_a,
-                              int64_t* E, int64_t* N, int64_t* K, int* out_type) {
+                              int64_t* E, int64_t* N, int64_t* K, int* out_type, int64_t qbn = 128, int64_t qbk = 128) {
     int32_t rc;
     if ((rc = check_tensor(a, "a", 2)) || (rc = check_tensor(b, "b", 3)) || (rc = check_tensor(c, "c", 2))) return rc;
     if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN)
@@ -621,7 +621,7 @@ static int32_t grouped_common(const tg_tensor* c, const tg_tensor* a, const tg_t
     if (b->shape[2] != *K) return fail(TG_ERR_INVALID, "K dimensions must match: %lld != %lld", (long long)*K, (long long)b->shape[2]);
     if (c->shape[1] != *N) return fail(TG_ERR_INVALID, "c must have %lld columns", (long long)*N);
     if (*rows_a > INT32_MAX || *N > INT32_MAX || *K > INT32_MAX || *E > INT32_MAX) return fail(TG_ERR_INVALID, "extent exceeds int32");
-    const int64_t kblocks = cdiv(*K, 128), nblocks = cdiv(*N, 128);
+    const int64_t kblocks = cdiv(*K, qbk), nblocks = cdiv(*N, qbn);  // quantization blocks (128 x 128 unless the caller says otherwise)
     if (a_scale) {
         if ((rc = check_tensor(a_scale, "a_scale", 2))) return rc;
         if (a_scale->dtype != TG_F32) return fail(TG_ERR_DTYPE, "a_scale must be f32");
@@ -663,7 +663,11 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
     g_err[0] = 0;
     int64_t total_m, E, N, K;
     int out_type;
-    int32_t rc = grouped_common(c, a, b, a_scale, b_scale, &total_m, &E, &N, &K, &out_type);
+    // quantization blocks other than 128 x 128 (cfg[] slots) are taken by the fallback kernel
+    int64_t qbn = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_N), qbk = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_K);
+    if (qbn <= 0) qbn = 128;
+    if (qbk <= 0) qbk = 128;
+    int32_t rc = grouped_common(c, a, b, a_scale, b_scale, &total_m, &E, &N, &K, &out_type, qbn, qbk);
     if (rc) return rc;
     if (c->shape[0] != total_m) return fail(TG_ERR_INVALID, "c must have %lld rows", (long long)total_m);
     if ((rc = check_tensor(m_indptr, "m_indptr", 1))) return rc;
@@ -680,7 +684,7 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
     p.m_indptr = reinterpret_cast<const int*>(m_indptr->ptr);
 
     const bool fast = (K % 128) == 0 && K > 0 && K <= 65536 && aligned16(a->ptr) && aligned16(b->ptr) &&
-                      total_m * K < kOffsetLimit && N * K < kOffsetLimit &&
+                      total_m * K < kOffsetLimit && N * K < kOffsetLimit && qbn == 128 && qbk == 128 &&
                       cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
     Schedule s{0, -1, -1, 1, -1, -1, -1};
     if (!fast) {
@@ -689,7 +693,7 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
         q.a_sm = K; q.a_sk = 1; q.b_sn = K; q.b_sk = 1; q.b_se = N * K;
         q.group = tg::GROUP_RAGGED;
         q.block_scaled = 1;
-        q.qbn = 128; q.qbk = 128;
+        q.qbn = (int)qbn; q.qbk = (int)qbk;
         q.rows = (int)total_m;
         remember(s);
         if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");

@@ -149,8 +149,18 @@ def ragged_block_scaled_bmm(a, b, a_scale, b_scale, m_indptr, max_m, max_m_devic
     assert K_A == K_B, f"K dimensions must match: {K_A} != {K_B}"
     assert m_indptr.shape[0] == Q + 1, "m_indptr must have Q+1 elements"
     Q_SB, rnb, rkb = b_scale.shape
-    if K_B // rkb != 128 or math.ceil(N / 128) != rnb:
-        raise NotImplementedError("the hip backend implements 128x128 quantization blocks only")
+    # quantization blocks as the reference derives them (ragged_block_scaled_bmm.py:535-537): K elements per scale from the
+    # scale tensor's shape; likewise the weight rows per scale
+    # (a shape that 128 x 128 blocks explain is read as 128 x 128: ragged edges make the division ambiguous)
+    if math.ceil(N / 128) == rnb and math.ceil(K_B / 128) == rkb:
+        block_n, block_k = 128, 128
+    else:
+        block_k, block_n = K_B // rkb, -(-N // rnb)
+    assert block_k > 0 and math.ceil(K_B / block_k) == rkb and math.ceil(N / block_n) == rnb, "b_scale shape does not tile (N, K)"
+    kc = kwargs.get("kernel_configs")
+    if (block_n, block_k) != (128, 128):
+        # blocks other than 128 x 128 run on the library's software-decode kernel (correct, no MFMA)
+        kc = dict(kc or {}, QUANT_BLOCK_N=block_n, QUANT_BLOCK_K=block_k)
     if a_scale is not None:
         assert a_scale.shape[0] == total_m, "a_scale total_m dimension mismatch"
     assert Q_SB == Q, "b_scale Q dimension mismatch"
@@ -163,7 +173,7 @@ def ragged_block_scaled_bmm(a, b, a_scale, b_scale, m_indptr, max_m, max_m_devic
         else torch.empty((total_m, N), device=a.device, dtype=out_dtype)
     ptr = m_indptr if m_indptr.dtype == torch.int32 else m_indptr.to(torch.int32)
     a_s = None if a_scale is None else a_scale.float()
-    _lib.fp8_ragged_gemm(c, a, b, a_s, b_scale.float(), ptr, kwargs.get("kernel_configs"))
+    _lib.fp8_ragged_gemm(c, a, b, a_s, b_scale.float(), ptr, kc)
     return c
 
 
