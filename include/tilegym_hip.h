@@ -32,7 +32,8 @@ enum {
     TG_I32 = 3,
     TG_I64 = 4,
     TG_F8E5M2 = 5,
-    TG_F8E4M3FN = 7
+    TG_F8E4M3FN = 7,
+    TG_I8 = 8        /* not in the reference's numbering (0-7): the int8 destination of tg_fp8_quant_group */
 };
 
 /* return codes (src/tilegym/ops/cutile_rs/ffi_util.rs:108-122); -1 is reserved as the

@@ -123,8 +123,11 @@ def quantize_per_tensor(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q, scale.reshape(1)
 
 
-def quantize_act_1x128(x: torch.Tensor, block: int = 128, eps: Optional[float] = None, ue8m0: bool = False):
-    """Per-token 1 x ``block`` quantization; returns (q, scales[..., K/block]).
+def quantize_act_1x128(x: torch.Tensor, block: int = 128, eps: Optional[float] = None, ue8m0: bool = False,
+                       dst_dtype: torch.dtype = FP8):
+    """Per-token 1 x ``block`` quantization; returns (q, scales[..., K/block]).  ``dst_dtype=torch.int8``: the
+    integer destination of the flashinfer operator (same test oracle, :52-57): range [-128, 127], scale = amax / 127,
+    the quotient converted by torch's float -> int8 cast (toward zero).
 
     ``eps=None``: the unsloth rule, all-zero block -> scale 1.0
     (tests/suites/unsloth/test_fp8.py:80-97, src/.../unsloth/cutile/fp8.py:105-116).
@@ -132,17 +135,18 @@ def quantize_act_1x128(x: torch.Tensor, block: int = 128, eps: Optional[float] =
     (tests/suites/flashinfer/test_per_token_group_quant_8bit.py:41-68); with ``ue8m0`` the scale is then
     rounded up to a power of two, ``2^ceil(log2(max(|s|, 1e-10)))`` (same file, :61-63)."""
     assert x.shape[-1] % block == 0
+    qmin, qmax = (-128.0, 127.0) if dst_dtype == torch.int8 else (-FP8_MAX, FP8_MAX)
     xb = x.float().reshape(-1, block)
     amax = xb.abs().amax(dim=-1, keepdim=True)
     if eps is None:
         assert not ue8m0
-        s = amax / FP8_MAX
+        s = amax / qmax
         s = torch.where(s == 0, torch.ones_like(s), s)
     else:
-        s = amax.clamp(min=eps) / FP8_MAX
+        s = amax.clamp(min=eps) / qmax
         if ue8m0:
             s = torch.exp2(torch.ceil(torch.log2(torch.maximum(s.abs(), torch.tensor(1e-10)))))
-    q = (xb / s).clamp(-FP8_MAX, FP8_MAX).to(FP8).reshape(x.shape)
+    q = (xb / s).clamp(qmin, qmax).to(dst_dtype).reshape(x.shape)
     return q, s.reshape(*x.shape[:-1], x.shape[-1] // block)
 
 

@@ -125,6 +125,8 @@ def test_quantizer_operators_have_no_host_path():
     with pytest.raises(AssertionError):
         per_token_group_quant_8bit(x, 64, scale_ue8m0=True)            # needs column_major_scales, as in the reference
     with pytest.raises(NotImplementedError):
+        per_token_group_quant_8bit(x, 64, dst_dtype=torch.int16)       # e4m3 and int8 destinations only
+    with pytest.raises(RuntimeError, match="HIP device"):
         per_token_group_quant_8bit(x, 64, dst_dtype=torch.int8)
 
 

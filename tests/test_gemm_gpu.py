@@ -818,7 +818,7 @@ def test_group_quantizer_forms_bit_exact(device, dtype, group, tokens, hidden):
     G = hidden // group
 
     def same(q, s, q_ref, s_ref, what):
-        assert q.dtype == FP8 and s.dtype == torch.float32 and q.shape == x.shape and s.shape == s_ref.shape, what
+        assert q.dtype == q_ref.dtype and s.dtype == torch.float32 and q.shape == x.shape and s.shape == s_ref.shape, what
         assert torch.equal(s.cpu().view(torch.int32), s_ref.view(torch.int32)), f"{what}: scales differ"
         bad = q.cpu().view(torch.uint8) != q_ref.view(torch.uint8)
         assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} codes differ"
@@ -843,6 +843,15 @@ def test_group_quantizer_forms_bit_exact(device, dtype, group, tokens, hidden):
     same(q, s, q_ref3, s_ref3, "act_quant")
     with pytest.raises(AssertionError):
         per_token_group_quant_8bit(xd, group, scale_ue8m0=True)     # needs column_major_scales, as in the reference
+    # int8 destination (the reference's test sweeps dst_dtype over e4m3 and int8, test_per_token_group_quant_8bit.py:73)
+    qi_ref, si_ref = R.quantize_act_1x128(x, group, 1e-10, dst_dtype=torch.int8)
+    q, s = per_token_group_quant_8bit(xd, group, dst_dtype=torch.int8)
+    same(q, s, qi_ref, si_ref, "int8 row-major")
+    q, s = per_token_group_quant_8bit(xd, group, dst_dtype=torch.int8, column_major_scales=True)
+    same(q, s, qi_ref, si_ref, "int8 column-major")
+    qi_ref2, si_ref2 = R.quantize_act_1x128(x, group, 1e-10, ue8m0=True, dst_dtype=torch.int8)
+    q, s = per_token_group_quant_8bit(xd, group, dst_dtype=torch.int8, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    same(q, s, qi_ref2, si_ref2, "int8 power-of-two scales, aligned")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])

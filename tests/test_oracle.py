@@ -160,6 +160,34 @@ def _loop_block_gemm(A, B, As, Bs, bn, bk):
     return A_deq @ B_deq.t()
 
 
+def test_int8_group_quantizer_oracle_hand_vector_and_properties():
+    """dst_dtype=torch.int8 of per_token_group_quant_8bit (tests/suites/flashinfer/test_per_token_group_quant_8bit.py:41-68):
+    a hand-computed group, and what the definition fixes: scale = amax / 127, the largest element maps to +-127 (or
+    +-126 when the fp32 quotient falls one ulp short), truncation toward zero (never away), all-zero groups use eps."""
+    x = torch.zeros(1, 16)
+    x[0, :6] = torch.tensor([12.7, -12.7, 1.0, -0.99, 0.05, 6.36])
+    q, s = R.quantize_act_1x128(x, 16, 1e-10, dst_dtype=torch.int8)
+    assert q.dtype == torch.int8 and abs(float(s) - 0.1) < 1e-7
+    # 12.7/0.1 = 127, 1.0/0.1 = 10 (9.99.. in fp32 -> 9 or 10 by the quotient's rounding), -0.99/0.1 = -9.9 -> -9, 0.05/0.1 -> 0, 63.6 -> 63
+    want = torch.tensor([127, -127, int(torch.tensor(1.0) / s.reshape(())), -9, 0, 63], dtype=torch.int8)
+    assert torch.equal(q[0, :6], want) and int(q[0, 2]) in (9, 10)
+    g = _g(55)
+    y = torch.randn(37, 256, generator=g) * torch.exp(torch.randn(37, 1, generator=g))
+    y[3] = 0.0
+    for group in (16, 64, 128):
+        q, s = R.quantize_act_1x128(y, group, 1e-10, dst_dtype=torch.int8)
+        yb, qb, sb = y.reshape(-1, group), q.reshape(-1, group).float(), s.reshape(-1, 1)
+        amax = yb.abs().amax(dim=1, keepdim=True)
+        assert torch.equal(sb, amax.clamp(min=1e-10) / 127.0)
+        nz = amax.squeeze(1) > 0
+        top = qb.abs().amax(dim=1)[nz]   # amax / (amax / 127) is 127 or one ulp below it in fp32, and the cast truncates
+        assert ((top == 127) | (top == 126)).all() and (top == 127).any()
+        exact = yb.double() / sb.double()
+        assert (qb.abs() <= exact.abs() + 1e-4).all() and ((exact.abs() - qb.abs()) < 1.0 + 1e-4).all()   # toward zero, by less than one step
+        assert torch.equal(torch.sign(qb)[qb != 0], torch.sign(yb)[qb != 0])
+        assert (qb[~nz] == 0).all()
+
+
 @pytest.mark.parametrize("M,N,K", [(3, 130, 256), (5, 256, 384), (2, 100, 200)])
 def test_block_scaled_oracle_against_loops_and_c(M, N, K):
     g = _g(7)

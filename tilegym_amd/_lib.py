@@ -35,6 +35,7 @@ _DTYPE_CODES = {
     torch.float8_e5m2: 5,
     torch.uint8: 6,
     torch.float8_e4m3fn: 7,
+    torch.int8: 8,
 }
 
 _RC_NAMES = {0: "ok", -2: "unsupported dtype", -3: "kernel launch failed", -4: "device init failed",
@@ -349,13 +350,15 @@ def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = F
     return q, scales
 
 
-def fp8_quant_group(x: torch.Tensor, group_size: int, eps: float, rule: int, scales: Optional[torch.Tensor] = None):
-    """(q e4m3fn like x, scales) through tg_fp8_quant_group; rule 0 zero-group -> 1, 1 eps clamp, 2 eps clamp and
+def fp8_quant_group(x: torch.Tensor, group_size: int, eps: float, rule: int, scales: Optional[torch.Tensor] = None,
+                    dst_dtype: torch.dtype = torch.float8_e4m3fn):
+    """(q like x, scales) through tg_fp8_quant_group; q is e4m3fn or, with ``dst_dtype=torch.int8``, int8 (scale =
+    amax / 127, quotient truncated toward zero); rule 0 zero-group -> 1, 1 eps clamp, 2 eps clamp and
     power-of-two scales.  ``scales`` may be a 2-D (rows, K/group_size) f32 tensor with any strides (column-major
     layouts); by default it is allocated row-major with x's leading shape."""
     L = load()
     x = x.contiguous()
-    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    q = torch.empty(x.shape, dtype=dst_dtype, device=x.device)
     if scales is None:
         scales = torch.empty(x.shape[:-1] + (x.shape[-1] // group_size,), dtype=torch.float32, device=x.device)
     rc = L.tg_fp8_quant_group(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),

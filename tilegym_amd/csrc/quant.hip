@@ -54,11 +54,15 @@ enum QuantRule { QUANT_ZERO_TO_ONE = 0, QUANT_EPS = 1, QUANT_EPS_POW2 = 2 };
 
 // LPG lanes per group (group size 8 * LPG).  STRIDED: the scale of group j of row r goes to
 // scales[r * s_row + j * s_col] (groups < 2^31); otherwise to scales[g].
-template <typename T, int LPG, bool STRIDED>
+// I8: the destination is int8 instead of e4m3 (per_token_group_quant_8bit with dst_dtype=torch.int8,
+// tests/suites/flashinfer/test_per_token_group_quant_8bit.py:41-68): scale = amax / 127, q = the quotient clamped to
+// [-128, 127] and converted as a float -> integer cast does (toward zero).
+template <typename T, int LPG, bool STRIDED, bool I8>
 __global__ void __launch_bounds__(256) act_quant_group_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
                                                              float* __restrict__ scales, int64_t groups, float eps,
                                                              int rule, uint32_t groups_per_row, int64_t s_row, int64_t s_col) {
     constexpr int G = kQuantGroupsPerLane, GS = 8 * LPG, PASS = 256 / LPG;
+    constexpr float QMAX = I8 ? 127.0f : 448.0f, QMIN = I8 ? -128.0f : -448.0f;
     const int sub = threadIdx.x & (LPG - 1);
     const int64_t g0 = (int64_t)blockIdx.x * (PASS * G) + (threadIdx.x / LPG);
     v8f_q v[G];
@@ -81,8 +85,8 @@ __global__ void __launch_bounds__(256) act_quant_group_kernel(const T* __restric
 #pragma unroll
         for (int d = 1; d < LPG; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
         float s;
-        if (rule == QUANT_ZERO_TO_ONE) s = amax == 0.f ? 1.0f : amax / 448.0f;
-        else s = fmaxf(amax, eps) / 448.0f;
+        if (rule == QUANT_ZERO_TO_ONE) s = amax == 0.f ? 1.0f : amax / QMAX;
+        else s = fmaxf(amax, eps) / QMAX;
         if (rule == QUANT_EPS_POW2) s = exp2f(ceilf(log2f(fmaxf(fabsf(s), 1e-10f))));
         if (g >= groups) continue;
         const ScaleDivider div(s);
@@ -97,9 +101,17 @@ __global__ void __launch_bounds__(256) act_quant_group_kernel(const T* __restric
         int packed[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
+            float cc[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cc[i] = fminf(fmaxf(c[4 * h + i], QMIN), QMAX);
             int w = 0;
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(fminf(fmaxf(c[4 * h], -448.0f), 448.0f), fminf(fmaxf(c[4 * h + 1], -448.0f), 448.0f), w, false);
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(fminf(fmaxf(c[4 * h + 2], -448.0f), 448.0f), fminf(fmaxf(c[4 * h + 3], -448.0f), 448.0f), w, true);
+            if constexpr (I8) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) w |= ((int)cc[i] & 0xFF) << (8 * i);
+            } else {
+                w = __builtin_amdgcn_cvt_pk_fp8_f32(cc[0], cc[1], w, false);
+                w = __builtin_amdgcn_cvt_pk_fp8_f32(cc[2], cc[3], w, true);
+            }
             packed[h] = w;
         }
         *reinterpret_cast<v2i*>(q + g * GS + sub * 8) = v2i{packed[0], packed[1]};
@@ -221,24 +233,28 @@ __global__ void __launch_bounds__(256) moe_sum_kernel(const T* __restrict__ x, T
 }
 
 template <typename T, int LPG>
-static void launch_act_quant(const T* x, uint8_t* q, float* scales, int64_t groups, float eps, int rule, bool strided,
+static void launch_act_quant(const T* x, uint8_t* q, bool i8, float* scales, int64_t groups, float eps, int rule, bool strided,
                              uint32_t groups_per_row, int64_t s_row, int64_t s_col, hipStream_t s) {
     constexpr int per_wg = (256 / LPG) * kQuantGroupsPerLane;
     const dim3 grid((unsigned)((groups + per_wg - 1) / per_wg)), block(256);
-    if (strided)
-        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, true>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
+    if (strided && i8)
+        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, true, true>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
+    else if (strided)
+        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, true, false>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
+    else if (i8)
+        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, false, true>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
     else
-        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, false>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
+        hipLaunchKernelGGL((act_quant_group_kernel<T, LPG, false, false>), grid, block, 0, s, x, q, scales, groups, eps, rule, groups_per_row, s_row, s_col);
 }
 
 template <typename T>
-static hipError_t dispatch_act_quant(const T* x, uint8_t* q, float* scales, int64_t groups, int group_size, float eps, int rule,
+static hipError_t dispatch_act_quant(const T* x, uint8_t* q, bool i8, float* scales, int64_t groups, int group_size, float eps, int rule,
                                      bool strided, uint32_t groups_per_row, int64_t s_row, int64_t s_col, hipStream_t s) {
     switch (group_size) {
-        case 128: launch_act_quant<T, 16>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
-        case 64: launch_act_quant<T, 8>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
-        case 32: launch_act_quant<T, 4>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
-        case 16: launch_act_quant<T, 2>(x, q, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        case 128: launch_act_quant<T, 16>(x, q, i8, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        case 64: launch_act_quant<T, 8>(x, q, i8, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        case 32: launch_act_quant<T, 4>(x, q, i8, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
+        case 16: launch_act_quant<T, 2>(x, q, i8, scales, groups, eps, rule, strided, groups_per_row, s_row, s_col, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -246,14 +262,14 @@ static hipError_t dispatch_act_quant(const T* x, uint8_t* q, float* scales, int6
 
 // groups of group_size (16, 32, 64, 128) elements; with `strided` the scale of group j of row r (groups_per_row
 // groups in a row) is written to scales[r * s_row + j * s_col], otherwise to scales[r * groups_per_row + j]
-hipError_t run_act_quant_group(const void* x, int x_type, uint8_t* q, float* scales, int64_t groups, int group_size, float eps,
+hipError_t run_act_quant_group(const void* x, int x_type, uint8_t* q, bool q_is_int8, float* scales, int64_t groups, int group_size, float eps,
                                int rule, bool strided, int64_t groups_per_row, int64_t s_row, int64_t s_col, hipStream_t s) {
     if (groups <= 0) return hipSuccess;
     if (strided && (groups > INT32_MAX || groups_per_row <= 0)) return hipErrorInvalidValue;
     const uint32_t gpr = (uint32_t)groups_per_row;
-    if (x_type == OUT_BF16) return dispatch_act_quant((const __bf16*)x, q, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
-    if (x_type == OUT_F16) return dispatch_act_quant((const _Float16*)x, q, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
-    if (x_type == OUT_F32) return dispatch_act_quant((const float*)x, q, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
+    if (x_type == OUT_BF16) return dispatch_act_quant((const __bf16*)x, q, q_is_int8, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
+    if (x_type == OUT_F16) return dispatch_act_quant((const _Float16*)x, q, q_is_int8, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
+    if (x_type == OUT_F32) return dispatch_act_quant((const float*)x, q, q_is_int8, scales, groups, group_size, eps, rule, strided, gpr, s_row, s_col, s);
     return hipErrorInvalidValue;
 }
 

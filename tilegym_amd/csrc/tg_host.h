@@ -46,7 +46,7 @@ hipError_t run_moe_align(const void* ids, int ids_are_i64, int numel, int E, int
 // per-token group e4m3 quantizer (group_size 16/32/64/128); x_type uses the OutType numbering (f32/f16/bf16);
 // rule 0: zero group -> scale 1, 1: amax clamped below by eps, 2: as 1 with the scale rounded up to a power of two;
 // strided: scale of group j of row r at scales[r * s_row + j * s_col]
-hipError_t run_act_quant_group(const void* x, int x_type, uint8_t* q, float* scales, int64_t groups, int group_size, float eps,
+hipError_t run_act_quant_group(const void* x, int x_type, uint8_t* q, bool q_is_int8, float* scales, int64_t groups, int group_size, float eps,
                                int rule, bool strided, int64_t groups_per_row, int64_t s_row, int64_t s_col, hipStream_t s);
 // y (M,N) = float(x) * sc[i / bs][j / bs]; vec needs N % 16 == 0, bs % 16 == 0 and 16-byte aligned x and y
 hipError_t run_weight_dequant(const uint8_t* x, const float* sc, void* y, int y_type, int64_t M, int64_t N, int bs, int64_t s_cols,

@@ -921,7 +921,7 @@ int32_t tg_fp8_quant_group(const tg_tensor* q, const tg_tensor* scales, const tg
     if (scales->ndim < 0 || scales->ndim > TG_MAX_DIMS) return fail(TG_ERR_INVALID, "scales: ndim %d out of range", scales->ndim);
     const int x_type = io_type_of(x->dtype);
     if (x_type < 0) return fail(TG_ERR_DTYPE, "x must be bf16, f16 or f32");
-    if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
+    if (q->dtype != TG_F8E4M3FN && q->dtype != TG_I8) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7) or int8 (8)");
     if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
     if (rule < 0 || rule > 2) return fail(TG_ERR_INVALID, "rule must be 0, 1 or 2");
     if (group_size != 16 && group_size != 32 && group_size != 64 && group_size != 128)
@@ -951,7 +951,7 @@ int32_t tg_fp8_quant_group(const tg_tensor* q, const tg_tensor* scales, const tg
     DeviceGuard guard(device_id);
     if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
     hipError_t e = tg::run_act_quant_group(reinterpret_cast<const void*>(x->ptr), x_type, reinterpret_cast<uint8_t*>(q->ptr),
-                                           reinterpret_cast<float*>(scales->ptr), groups, group_size, eps, rule, strided, gpr,
+                                           q->dtype == TG_I8, reinterpret_cast<float*>(scales->ptr), groups, group_size, eps, rule, strided, gpr,
                                            s_row, s_col, reinterpret_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "quantizer launch failed: %s", hipGetErrorString(e));
     return TG_OK;

@@ -40,9 +40,12 @@ def act_quant(x: torch.Tensor, block_size: int = 128) -> Tuple[torch.Tensor, tor
 
 def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128, eps: float = 1e-10,
                               scale_ue8m0: bool = False, column_major_scales: bool = False,
-                              scale_tma_aligned: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+                              scale_tma_aligned: bool = False,
+                              dst_dtype: torch.dtype = FP8) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per (token, group) quantization with amax clamped below by eps
-    (src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:152-272).
+    (src/tilegym/suites/flashinfer/cutile/per_token_group_quant_8bit.py:152-272); ``dst_dtype`` is
+    float8_e4m3fn or int8 (scale = amax / 127, values clamped to [-128, 127] and converted toward zero, as the
+    float -> int8 cast of the reference's oracle does).
 
     Scale layouts as there (:185-204): row-major ``x.shape[:-1] + (G,)``; ``column_major_scales``: a
     ``(tokens, G)`` tensor with strides ``(1, tokens)``; with ``scale_tma_aligned`` the reference fills a
@@ -53,6 +56,8 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128, eps: float
     assert x.is_contiguous(), "`x` must be contiguous"
     if scale_tma_aligned or scale_ue8m0:
         assert column_major_scales, "scale_tma_aligned or scale_ue8m0 requires column_major_scales=True"
+    if dst_dtype not in (FP8, torch.int8):
+        raise NotImplementedError(f"dst_dtype {dst_dtype} is not implemented (float8_e4m3fn, int8)")
     _require_device(x, "per_token_group_quant_8bit", group_size)
     groups = x.shape[-1] // group_size
     if column_major_scales and x.dim() != 2:
@@ -62,7 +67,7 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128, eps: float
         scales = torch.empty((groups, x.shape[0]), dtype=torch.float32, device=x.device).t()
     elif column_major_scales:
         scales = torch.empty((x.shape[0], groups), dtype=torch.float32, device=x.device)
-    return _lib.fp8_quant_group(x, group_size, eps, 2 if scale_ue8m0 else 1, scales)
+    return _lib.fp8_quant_group(x, group_size, eps, 2 if scale_ue8m0 else 1, scales, dst_dtype)
 
 
 def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128,

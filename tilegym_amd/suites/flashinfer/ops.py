@@ -40,6 +40,6 @@ def per_token_group_quant_8bit(x: torch.Tensor, group_size: int, eps: float = 1e
 @register_impl("flashinfer.per_token_group_quant_8bit", backend="hip")
 def _per_token_group_quant_8bit(x, group_size, eps=1e-10, dst_dtype=torch.float8_e4m3fn,
                                 column_major_scales=False, scale_tma_aligned=False, scale_ue8m0=False):
-    if dst_dtype != torch.float8_e4m3fn:
-        raise NotImplementedError("only float8_e4m3fn is implemented")
-    return _quant.per_token_group_quant_fp8(x, group_size, eps, scale_ue8m0, column_major_scales, scale_tma_aligned)
+    if dst_dtype is None:
+        dst_dtype = torch.float8_e4m3fn
+    return _quant.per_token_group_quant_fp8(x, group_size, eps, scale_ue8m0, column_major_scales, scale_tma_aligned, dst_dtype)
