@@ -219,6 +219,70 @@ def test_ragged_quantization_blocks_other_than_128(device, bn, bk):
     check(out, ref, what=f"ragged, blocks {bn}x{bk}")
 
 
+@pytest.mark.parametrize("block_scaled", [False, True])
+def test_columns_split_where_256_tiles_leave_the_last_round_mostly_empty(device, block_scaled):
+    """M = 1024, N = 16896: 4 x 66 = 264 tiles of 256 x 256 are 1.03 rounds of the chip.  The library computes the 64
+    column tiles that fill one round with 256 x 256 tiles and the remaining 512 columns as a problem of its own
+    (C's row stride stays N).  Same bits as one schedule for everything, and the oracle on sampled rows."""
+    M, N, K = 1024, 16896, 256
+    g = _g(4242 + block_scaled)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
+    if block_scaled:
+        sa = torch.rand(M, K // 128, generator=g) * 0.05 + 0.01
+        sb = torch.rand(N // 128, K // 128, generator=g) * 0.05 + 0.01
+    else:
+        sa, sb = torch.tensor([0.03]), torch.tensor([0.02])
+    ad, bd, sad, sbd = a.to(device), b.to(device), sa.to(device), sb.to(device)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=device)
+    _lib.fp8_gemm(out, ad, bd, sad, sbd, False, True, 1.0, 0.0, None)
+    cfg = _lib.last_config()          # the schedule of the last piece: the 512 remaining columns
+    assert cfg["KERNEL_NAME"] == "tiled" and (cfg["BLOCK_M"], cfg["BLOCK_N"]) != (256, 256), cfg
+    one = torch.empty_like(out)
+    _lib.fp8_gemm(one, ad, bd, sad, sbd, False, True, 1.0, 0.0, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256})
+    assert torch.equal(out, one)
+    rows = _rows_stratified(M, 8, seed=17)
+    if block_scaled:
+        ref = R.ref_w8a8_block_fp8_matmul(a[rows], b, sa[rows], sb, [128, 128], torch.bfloat16)
+    else:
+        ref = R.ref_gemm_per_tensor(a[rows], b, sa, sb, trans_b=True)
+    check(out[rows.to(device)], ref, what=f"column split, block_scaled={block_scaled}")
+    # beta != 0 reads each piece's own part of C
+    c0 = torch.randn(M, N, generator=g).to(torch.bfloat16)
+    c = c0.clone().to(device)
+    if not block_scaled:
+        _lib.fp8_gemm(c, ad, bd, sad, sbd, False, True, 1.0, 1.0, None)
+        ref2 = (R.ref_gemm_per_tensor(a[rows], b, sa, sb, trans_b=True, out_dtype=torch.float32) + c0[rows].float()).to(torch.bfloat16)
+        check(c[rows.to(device)], ref2, what="column split, beta = 1")
+
+
+@pytest.mark.parametrize("block_scaled", [False, True])
+def test_rows_split_where_256_tiles_leave_the_last_round_mostly_empty(device, block_scaled):
+    """M = 5120, N = 4096: 20 x 16 = 320 tiles of 256 x 256; no whole number of column tiles fills a round, sixteen row
+    tiles do: rows 0 .. 4095 run with 256 x 256 tiles, the last 1024 rows as a problem of their own."""
+    M, N, K = 5120, 4096, 128
+    g = _g(4343 + block_scaled)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
+    if block_scaled:
+        sa = torch.rand(M, 1, generator=g) * 0.05 + 0.01
+        sb = torch.rand(N // 128, 1, generator=g) * 0.05 + 0.01
+    else:
+        sa, sb = torch.tensor([0.03]), torch.tensor([0.02])
+    ad, bd, sad, sbd = a.to(device), b.to(device), sa.to(device), sb.to(device)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=device)
+    _lib.fp8_gemm(out, ad, bd, sad, sbd, False, True, 1.0, 0.0, None)
+    cfg = _lib.last_config()
+    assert cfg["KERNEL_NAME"] == "tiled" and (cfg["BLOCK_M"], cfg["BLOCK_N"]) != (256, 256), cfg
+    one = torch.empty_like(out)
+    _lib.fp8_gemm(one, ad, bd, sad, sbd, False, True, 1.0, 0.0, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256})
+    assert torch.equal(out, one)
+    rows = _rows_stratified(M, 4, seed=18)
+    if block_scaled:
+        ref = R.ref_w8a8_block_fp8_matmul(a[rows], b, sa[rows], sb, [128, 128], torch.bfloat16)
+    else:
+        ref = R.ref_gemm_per_tensor(a[rows], b, sa, sb, trans_b=True)
+    check(out[rows.to(device)], ref, what=f"row split, block_scaled={block_scaled}")
+
+
 def test_fallback_kernel_takes_more_rows_than_one_grid_dimension_holds(device):
     """The software-decode kernel walks rows grid-stride: 300 000 rows (above 4 x 65 535) of a K that no fast kernel
     takes (K % 16 != 0)."""
