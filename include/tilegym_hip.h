@@ -213,6 +213,18 @@ int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, i
                                 const tg_tensor* max_expert_count, int32_t device_id, uint64_t hip_stream);
 
 /*
+ * tg_moe_align_block_size and the 1 x 128 activation quantizer (tg_fp8_quant_1x128 with rule 0) as ONE launch: the two
+ * launches in front of the first GEMM of the FP8 MoE layer (the layer of src/tilegym/ops/moe_interface.py:116-321 calls
+ * moe_align_block_size at :246-248; the FP8 GEMM needs its activations quantized 1 x 128 first).  The two share no data.
+ * Arguments and results as for the two entry points; x: bf16 or f16, last dimension a multiple of 128.
+ */
+int32_t tg_moe_align_quant_1x128(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
+                                 const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
+                                 const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,
+                                 const tg_tensor* max_expert_count, const tg_tensor* q, const tg_tensor* scales,
+                                 const tg_tensor* x, int32_t device_id, uint64_t hip_stream);
+
+/*
  * Per-token 1 x 128 FP8 quantizer (the producer of scale_a for the block-scaled GEMMs):
  *   scales[m, kb] = amax(x[m, 128*kb : 128*kb+128]) / 448      (rule 0: an all-zero group gets 1.0;
  *                                                               rule 1: amax is first clamped below by eps)

@@ -820,6 +820,28 @@ def test_moe_align_kernel_matches_oracle(device, T, top_k, E, bs, dtype):
     assert all(torch.equal(a, b) for a, b in zip(got, again))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("ids_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("T,k,E,bs,H", [(4096, 6, 64, 256, 2048), (33, 2, 8, 16, 128), (1, 8, 512, 64, 1024), (700, 4, 20, 128, 384)])
+def test_moe_align_and_quantizer_in_one_launch(device, dtype, ids_dtype, T, k, E, bs, H):
+    """tg_moe_align_quant_1x128: all seven outputs bit for bit those of the two stand-alone launches (and so of the oracle)."""
+    from tilegym_amd.suites.unsloth.ops import act_quant
+
+    g = _g(T * 3 + E + H)
+    ids = torch.randint(0, E, (T, k), generator=g).to(ids_dtype).to(device)
+    x = (torch.randn(T, H, generator=g) * torch.exp(torch.randn(T, 1, generator=g))).to(dtype)
+    x[0, :128] = 0.0
+    xd = x.to(device)
+    want = moe_align_block_size(ids, bs, E)
+    q_want, s_want = act_quant(xd, 128)
+    got = _lib.moe_align_quant_1x128(ids, bs, E, xd)
+    for a_, b_ in zip(got[:5], want):
+        assert torch.equal(a_, b_)
+    assert torch.equal(got[5].view(torch.uint8), q_want.view(torch.uint8)) and torch.equal(got[6], s_want)
+    q_ref, s_ref = R.quantize_act_1x128(x, 128, None)
+    assert torch.equal(got[5].cpu().view(torch.uint8), q_ref.view(torch.uint8)) and torch.equal(got[6].cpu(), s_ref)
+
+
 def test_moe_align_limits(device):
     """More experts than the one-launch kernel takes is an explicit error (no torch-op path); an empty routing
     gives the fill values."""

@@ -110,6 +110,8 @@ def load():
                                              ctypes.c_int32, ctypes.c_uint64]
     L.tg_moe_align_block_size.restype = ctypes.c_int32
     L.tg_moe_align_block_size.argtypes = [P, ctypes.c_int32, ctypes.c_int32, P, P, P, P, P, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_moe_align_quant_1x128.restype = ctypes.c_int32
+    L.tg_moe_align_quant_1x128.argtypes = [P, ctypes.c_int32, ctypes.c_int32, P, P, P, P, P, P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_fp8_quant_1x128.restype = ctypes.c_int32
     L.tg_fp8_quant_1x128.argtypes = [P, P, P, ctypes.c_float, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     L.tg_fp8_quant_group.restype = ctypes.c_int32
@@ -333,6 +335,33 @@ def moe_align_block_size(topk_ids, block_size: int, num_experts: int):
                                    _device_index(ids), _stream_handle(ids))
     check_rc(rc, "tg_moe_align_block_size")
     return sorted_ids, expert_ids, post, cumsum, mx
+
+
+def moe_align_quant_1x128(topk_ids, block_size: int, num_experts: int, x: torch.Tensor):
+    """moe_align_block_size(topk_ids, ...) and the 1 x 128 quantization of ``x`` (bf16 / f16, all-zero group -> scale 1)
+    in one launch (tg_moe_align_quant_1x128).  Returns (sorted_ids, expert_ids, post, cumsum, max_count, q, scales)."""
+    L = load()
+    ids = topk_ids if topk_ids.dtype in (torch.int32, torch.int64) else topk_ids.to(torch.int64)
+    ids = ids.contiguous()
+    x = x.contiguous()
+    dev = ids.device
+    numel = ids.numel()
+    cap = numel + num_experts * (block_size - 1)
+    nblk = -(-cap // block_size)
+    sorted_ids = torch.empty(cap, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(max(nblk, 1), dtype=torch.int32, device=dev)[:nblk]
+    post = torch.empty(1, dtype=torch.int32, device=dev)
+    cumsum = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+    mx = torch.empty(1, dtype=torch.int32, device=dev)
+    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty(x.shape[:-1] + (x.shape[-1] // 128,), dtype=torch.float32, device=x.device)
+    rc = L.tg_moe_align_quant_1x128(_ref(make_tensor_desc(ids)), int(block_size), int(num_experts),
+                                    _ref(make_tensor_desc(sorted_ids)), _ref(make_tensor_desc(expert_ids)),
+                                    _ref(make_tensor_desc(post)), _ref(make_tensor_desc(cumsum)), _ref(make_tensor_desc(mx)),
+                                    _ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+                                    _device_index(ids), _stream_handle(ids))
+    check_rc(rc, "tg_moe_align_quant_1x128")
+    return sorted_ids, expert_ids, post, cumsum, mx, q, scales
 
 
 def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = False, q=None, scales=None):

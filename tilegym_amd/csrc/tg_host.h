@@ -43,6 +43,10 @@ hipError_t run_generic(const GenericParams& p, hipStream_t s);
 // moe_align_block_size in one launch (num_experts <= 512); ids are int32 or int64
 hipError_t run_moe_align(const void* ids, int ids_are_i64, int numel, int E, int block_size, int* sorted_ids, int cap,
                          int* expert_ids, int nblk, int* num_post_pad, int* cumsum, int* max_cnt, hipStream_t s);
+// moe_align_block_size and the 1 x 128 activation quantizer (all-zero group -> scale 1) side by side in one launch
+hipError_t run_moe_align_quant(const void* ids, int ids_are_i64, int numel, int E, int block_size, int* sorted_ids, int cap,
+                               int* expert_ids, int nblk, int* num_post_pad, int* cumsum, int* max_cnt, const void* x,
+                               int x_is_bf16, uint8_t* q, float* scales, int64_t groups, hipStream_t s);
 // per-token group e4m3 quantizer (group_size 16/32/64/128); x_type uses the OutType numbering (f32/f16/bf16);
 // rule 0: zero group -> scale 1, 1: amax clamped below by eps, 2: as 1 with the scale rounded up to a power of two;
 // strided: scale of group j of row r at scales[r * s_row + j * s_col]

@@ -917,11 +917,11 @@ int32_t tg_fp8_moe_gemm_silu_quant(const tg_tensor* q, const tg_tensor* scales, 
     return TG_OK;
 }
 
-int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
+// argument checks of moe_align_block_size (host side only); n = number of (token, slot) pairs, cap = len(sorted_token_ids)
+static int32_t check_align_args(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
                                 const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
                                 const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,
-                                const tg_tensor* max_expert_count, int32_t device_id, uint64_t hip_stream) {
-    g_err[0] = 0;
+                                const tg_tensor* max_expert_count, int64_t* n_out, int64_t* cap_out) {
     int32_t rc;
     if ((rc = check_tensor(topk_ids, "topk_ids", -1)) || (rc = check_tensor(sorted_token_ids, "sorted_token_ids", 1)) ||
         (rc = check_tensor(expert_ids, "expert_ids", 1)) || (rc = check_tensor(num_tokens_post_padded, "num_tokens_post_padded", -1)) ||
@@ -941,6 +941,20 @@ int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, i
     if (numel(expert_ids) < nblk) return fail(TG_ERR_INVALID, "expert_ids must have at least %lld elements", (long long)nblk);
     if (numel(num_tokens_post_padded) < 1 || numel(max_expert_count) < 1) return fail(TG_ERR_INVALID, "scalar outputs need one element");
     if (numel(cumsum) != num_experts + 1) return fail(TG_ERR_INVALID, "cumsum must have num_experts + 1 elements");
+    *n_out = n;
+    *cap_out = cap;
+    return TG_OK;
+}
+
+int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
+                                const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
+                                const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,
+                                const tg_tensor* max_expert_count, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int64_t n, cap;
+    const int32_t rc = check_align_args(topk_ids, block_size, num_experts, sorted_token_ids, expert_ids, num_tokens_post_padded, cumsum,
+                                        max_expert_count, &n, &cap);
+    if (rc) return rc;
     DeviceGuard guard(device_id);
     if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
     hipError_t e = tg::run_moe_align(reinterpret_cast<const void*>(topk_ids->ptr), topk_ids->dtype == TG_I64, (int)n, num_experts,
@@ -949,6 +963,40 @@ int32_t tg_moe_align_block_size(const tg_tensor* topk_ids, int32_t block_size, i
                                      reinterpret_cast<int*>(num_tokens_post_padded->ptr), reinterpret_cast<int*>(cumsum->ptr),
                                      reinterpret_cast<int*>(max_expert_count->ptr), reinterpret_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "moe_align launch failed: %s", hipGetErrorString(e));
+    return TG_OK;
+}
+
+int32_t tg_moe_align_quant_1x128(const tg_tensor* topk_ids, int32_t block_size, int32_t num_experts,
+                                 const tg_tensor* sorted_token_ids, const tg_tensor* expert_ids,
+                                 const tg_tensor* num_tokens_post_padded, const tg_tensor* cumsum,
+                                 const tg_tensor* max_expert_count, const tg_tensor* q, const tg_tensor* scales,
+                                 const tg_tensor* x, int32_t device_id, uint64_t hip_stream) {
+    g_err[0] = 0;
+    int64_t n, cap;
+    int32_t rc = check_align_args(topk_ids, block_size, num_experts, sorted_token_ids, expert_ids, num_tokens_post_padded, cumsum,
+                                  max_expert_count, &n, &cap);
+    if (rc) return rc;
+    if ((rc = check_tensor(x, "x", -1)) || (rc = check_tensor(q, "q", -1)) || (rc = check_tensor(scales, "scales", -1))) return rc;
+    if (x->dtype != TG_BF16 && x->dtype != TG_F16) return fail(TG_ERR_DTYPE, "x must be bf16 or f16");
+    if (q->dtype != TG_F8E4M3FN) return fail(TG_ERR_DTYPE, "q must be float8_e4m3fn (dtype code 7)");
+    if (scales->dtype != TG_F32) return fail(TG_ERR_DTYPE, "scales must be f32");
+    if (x->ndim < 1) return fail(TG_ERR_INVALID, "x needs at least one dimension");
+    const int64_t K = x->shape[x->ndim - 1], nx = numel(x);
+    if (K % 128 != 0) return fail(TG_ERR_INVALID, "the last dimension (%lld) must be a multiple of 128", (long long)K);
+    if (numel(q) != nx) return fail(TG_ERR_INVALID, "q must have the shape of x");
+    const int64_t groups = nx / 128;
+    if (numel(scales) != groups) return fail(TG_ERR_INVALID, "scales must have %lld elements", (long long)groups);
+    if (nx > 0 && (!aligned16(x->ptr) || (q->ptr & 7) != 0)) return fail(TG_ERR_INVALID, "x must be 16-byte and q 8-byte aligned");
+    DeviceGuard guard(device_id);
+    if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+    hipError_t e = tg::run_moe_align_quant(reinterpret_cast<const void*>(topk_ids->ptr), topk_ids->dtype == TG_I64, (int)n, num_experts,
+                                           block_size, reinterpret_cast<int*>(sorted_token_ids->ptr), (int)cap,
+                                           reinterpret_cast<int*>(expert_ids->ptr), (int)numel(expert_ids),
+                                           reinterpret_cast<int*>(num_tokens_post_padded->ptr), reinterpret_cast<int*>(cumsum->ptr),
+                                           reinterpret_cast<int*>(max_expert_count->ptr), reinterpret_cast<const void*>(x->ptr),
+                                           x->dtype == TG_BF16, reinterpret_cast<uint8_t*>(q->ptr), reinterpret_cast<float*>(scales->ptr),
+                                           groups, reinterpret_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "moe_align + quantizer launch failed: %s", hipGetErrorString(e));
     return TG_OK;
 }
 

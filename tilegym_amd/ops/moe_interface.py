@@ -118,9 +118,14 @@ def fused_experts_impl(
             c1 = cache1[:n]
         if cur.dtype == FP8:
             xq, xs = cur, a1_scale[lo:hi]
+            sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids, config["BLOCK_SIZE_M"], E)
+        elif E <= _lib.MOE_ALIGN_MAX_EXPERTS and n > 0:
+            # the alignment of the routing and the 1 x 128 quantization of the activations share no data: one launch
+            sorted_ids, expert_ids, post, _, _, xq, xs = _lib.moe_align_quant_1x128(
+                ids, config["BLOCK_SIZE_M"], E, cur if cur.dtype != torch.float32 else cur.to(out_dtype))
         else:
             xq, xs = quant.act_quant(cur if cur.dtype != torch.float32 else cur.to(out_dtype), 128)
-        sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids, config["BLOCK_SIZE_M"], E)
+            sorted_ids, expert_ids, post, _, _ = moe_align_block_size(ids, config["BLOCK_SIZE_M"], E)
         if fuse_act:
             # GEMM1 with SiLU(gate) * up and the 1x128 re-quantization in its epilogue: same bits as the
             # two steps below, without writing and re-reading the (n * top_k, 2I) intermediate
