@@ -78,13 +78,13 @@ def test_per_tensor_tiled_split_k(device, split):
         assert torch.equal(again, out)
 
 
-# ----------------------------------------------------------------------------- per-tensor, hand-ordered 256x256 tile
-@pytest.mark.parametrize("waves", [-1, 4])
+# ----------------------------------------------------------------------------- per-tensor, persistent hand-ordered 256x256 tile
+@pytest.mark.parametrize("waves", [-1, 8])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 520, 384), (257, 255, 512), (1024, 768, 1280), (40, 1000, 256), (512, 252, 640)])
 def test_per_tensor_ordered_256(device, M, N, K, waves):
-    """The 256x256 tile in its hand-ordered form (default) and in the generic form (WAVES = 4): K = 128 (one step: the
-    prologue's second-step loads re-fetch the first), odd numbers of steps, ragged M and N, N not a multiple of 8 (scalar
-    store path); bf16, f16, f32 outputs and beta; the two forms agree bit for bit."""
+    """The 256x256 tile in its persistent hand-ordered form (default from two K steps up) and in the generic form
+    (WAVES = 8): K = 128 (one step: always the generic form), odd numbers of steps, ragged M and N, N not a multiple of 8
+    (scalar store path); bf16, f16, f32 outputs and beta; the two forms agree bit for bit."""
     g = _g(M + 3 * N + K)
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
     sa, sb = torch.tensor([0.013]), torch.tensor([0.0004])
@@ -96,7 +96,7 @@ def test_per_tensor_ordered_256(device, M, N, K, waves):
     assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (256, 256)
     check(res, ref, what=f"256x256 M={M} N={N} K={K} waves={waves}")
     other = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
-                   out_dtype=torch.bfloat16, kernel_configs=dict(kc, WAVES=4 if waves != 4 else -1))
+                   out_dtype=torch.bfloat16, kernel_configs=dict(kc, WAVES=8 if waves != 8 else -1))
     assert torch.equal(res, other), "ordered and generic 256x256 kernels differ"
     one = torch.tensor([1.0])  # keep the f16 outputs in the normal range
     ref16 = R.ref_gemm_per_tensor(a, b, one, one, trans_b=True, out_dtype=torch.float16)

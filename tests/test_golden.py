@@ -99,7 +99,7 @@ def test_oracle_moe_align_fixture():
 DENSE_KERNELS = [None, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 128}, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 32}, {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 64},
                  {"KERNEL": "tiled", "BLOCK_M": 32, "BLOCK_N": 32}, {"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128},
                  {"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128, "SPLIT_K": 2},
-                 {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256}, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "WAVES": 4},
+                 {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256}, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "WAVES": 8},
                  {"KERNEL": "skinny"}, {"KERNEL": "skinny", "WAVES": 8, "ROW_GROUPS": 2}, {"KERNEL": "stream"},
                  {"KERNEL": "stream", "ROW_GROUPS": 4}, {"KERNEL": "fallback"}]
 

@@ -5,7 +5,20 @@
 
 namespace tg {
 
-hipError_t run_tile256(const GemmParams& p, int gx, hipStream_t s) { return launch_tile256(p, gx, s); }
+// Compute units of the current device: the persistent 256x256 kernel runs one workgroup on each.
+static int compute_units() {
+    static int cached[64];  // by device ordinal; 0 = not asked yet (racing first calls write the same value)
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+hipError_t run_tile256(const GemmParams& p, int gx, hipStream_t s) { return launch_tile256(p, gx, compute_units(), s); }
 hipError_t run_tile_mid(int bm, int bn, const GemmParams& p, hipStream_t s) {
     if (bn == 64) return launch_tile_mid<64, 64, 2>(p, s);
     return bm == 32 ? launch_tile_mid<32, 32, 4>(p, s) : launch_tile_mid<64, 32, 3>(p, s);

@@ -626,9 +626,10 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         const bool split = pc.split_k > 1;
         const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128;
         const bool mid = s.kernel == 1 && !block_scaled && is_mid_tile(s.bm, s.bn);
-        // hand-ordered K loop for the dense per-tensor 256x256 tile (WAVES = 4 asks for the generic tile kernel instead)
-        const bool ordered = s.kernel == 1 && !block_scaled && !split && s.bm == 256 && s.bn == 256 &&
-                             cfg_get(cfg, ncfg, TG_CFG_WAVES) != 4;
+        // persistent kernel with the hand-ordered K loop for the dense per-tensor 256x256 tile, from two K steps up
+        // (WAVES = 8 asks for the generic eight-wave tile kernel instead)
+        const bool ordered = s.kernel == 1 && !block_scaled && !split && s.bm == 256 && s.bn == 256 && kblocks >= 2 &&
+                             cfg_get(cfg, ncfg, TG_CFG_WAVES) != 8;
         hipError_t e = mid ? tg::run_tile_mid(s.bm, s.bn, pc, stream)
                      : ordered ? tg::run_tile256(pc, gx, stream)
                      : deep ? tg::run_tile_deep(split, pc, gx, pc.split_k, stream)
