@@ -109,6 +109,30 @@ def test_per_tensor_ordered_256(device, M, N, K, waves):
     check(res32, ref32, what=f"256x256 f32 M={M} N={N} K={K}")
 
 
+@pytest.mark.parametrize("M,N,K,out_dtype", [(4352, 4352, 384, torch.bfloat16), (4300, 4360, 256, torch.bfloat16),
+                                             (4200, 4507, 640, torch.float16), (2100, 9000, 256, torch.float32)])
+def test_persistent_256_walks_several_tiles_per_workgroup(device, M, N, K, out_dtype):
+    """More 256x256 tiles than the device has compute units: workgroups of the persistent kernel compute two or more
+    tiles, with the operand rings running on from one tile into the next.  Full tiles only; ragged last tile rows and
+    columns (a partial tile in the middle of a workgroup's sequence); N not a multiple of 8 (scalar stores); two K steps
+    (the switch to the next tile's addresses happens in a tile's first step).  Bit-equal to the generic eight-wave
+    kernel, which computes one tile per workgroup, and sampled rows against the oracle."""
+    assert math.ceil(M / 256) * math.ceil(N / 256) > torch.cuda.get_device_properties(device).multi_processor_count
+    g = _g(M + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.021]), torch.tensor([0.0007])
+    kc = {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "SPLIT_K": 1}
+    args = dict(trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device), out_dtype=out_dtype)
+    res = matmul(a.to(device), b.to(device), kernel_configs=kc, **args)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (256, 256)
+    other = matmul(a.to(device), b.to(device), kernel_configs=dict(kc, WAVES=8), **args)
+    assert torch.equal(res, other), "persistent and generic 256x256 kernels differ"
+    rows = torch.cat([torch.arange(0, 4), torch.arange(255, 258), torch.randint(0, M, (24,), generator=g), torch.arange(M - 3, M)])
+    ref = R.ref_gemm_per_tensor(a[rows], b, sa, sb, trans_b=True, out_dtype=out_dtype)
+    check(res[rows.to(device)], ref, what=f"persistent 256x256 M={M} N={N} K={K}")
+
+
 @pytest.mark.parametrize("bm,bn", [(32, 32), (64, 32), (64, 64)])
 @pytest.mark.parametrize("M,N,K", [(64, 512, 1024), (40, 200, 384), (17, 1000, 2560), (130, 72, 128), (33, 264, 256), (96, 4096, 4096)])
 def test_per_tensor_mid_tiles(device, bm, bn, M, N, K):
