@@ -1177,8 +1177,9 @@ def test_fused_moe_fp8_at_the_reference_tests_configurations(device, T, H, I, E,
 def test_launches_replay_from_a_hip_graph(device):
     """Every entry point only enqueues on the caller's stream (no allocation, synchronisation or memset of its
     own), so a caller may capture it: the MoE layer (align, quantizer, both grouped GEMMs with the fused
-    activation epilogue, top-k sum) and a split-K decode GEMM with its workspace are captured once and replayed
-    three times with eager work in between; every replay must reproduce the eager result bit for bit."""
+    activation epilogue, top-k sum), a split-K decode GEMM with its workspace and the persistent 256x256 kernel are
+    captured once and replayed three times with eager work in between; every replay must reproduce the eager result
+    bit for bit."""
     from tilegym_amd.ops import fused_moe
 
     g = _g(33)
@@ -1193,13 +1194,20 @@ def test_launches_replay_from_a_hip_graph(device):
     a = fp8_randn((16, 14336), g).to(device)
     b = fp8_randn((4096, 14336), g, 0.05).to(device)
     one = torch.ones(1, device=device)
+    a2 = fp8_randn((700, 640), g).to(device)
+    b2 = fp8_randn((520, 640), g, 0.05).to(device)
 
     def work():
         out = fused_moe(hidden, w1q, w2q, tw, ids, w1_scale=w1s, w2_scale=w2s)
-        return out, matmul(a, b, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        big = matmul(a2, b2, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16,
+                     kernel_configs={"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256})
+        assert _lib.last_config()["BLOCK_M"] == 256
+        return out, matmul(a, b, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16), big
 
-    eager_moe, eager_mm = work()
-    assert _lib.last_config()["SPLIT_K"] > 1  # the decode GEMM takes the split-K path (workspace + reduction)
+    eager_moe, eager_mm, eager_big = work()
+    assert _lib.last_config()["SPLIT_K"] > 1  # the decode GEMM (the last launch of work()) takes the split-K path (workspace + reduction)
+    assert torch.equal(eager_big, matmul(a2, b2, trans_b=True, scale_a=one, scale_b=one, out_dtype=torch.bfloat16,
+                                         kernel_configs={"KERNEL": "tiled", "BLOCK_M": 128, "BLOCK_N": 128}))
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -1210,16 +1218,18 @@ def test_launches_replay_from_a_hip_graph(device):
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        g_moe, g_mm = work()
+        g_moe, g_mm, g_big = work()
     for rep in range(3):
         g_moe.zero_()
         g_mm.zero_()
+        g_big.zero_()
         hidden.add_(0.0)  # eager work between the replays
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(g_moe, eager_moe), f"MoE layer differs on replay {rep}"
         assert torch.equal(g_mm, eager_mm), f"split-K GEMM differs on replay {rep}"
+        assert torch.equal(g_big, eager_big), f"persistent 256x256 GEMM differs on replay {rep}"
 
 
 def test_graph_workspace_survives_a_larger_eager_gemm(device):
