@@ -245,7 +245,8 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // count fills whole rounds of the chip; a last round that is mostly empty costs more than
         // that, so compare the two by (fraction of the rounds' slots that hold a tile) x (tile rate).
         auto fill = [&](int64_t n, int64_t slots) { return (double)n / (double)(cdiv(n, slots) * slots); };
-        const double s256 = fill(tiles(256, 256), 256) * 1.0, s128 = fill(tiles(128, 128), 512) * 0.83;
+        // (per-tensor: the persistent four-wave 256x256 kernel is another 8 % ahead of its eight-wave form, hence 0.77)
+        const double s256 = fill(tiles(256, 256), 256) * 1.0, s128 = fill(tiles(128, 128), 512) * (block_scaled ? 0.83 : 0.77);
         // the three-stage 64x128 kernel (per-tensor) also wins above 64 rows while its tiles fit one round of the
         // chip: 13.3 / 14.5 / 17.8 / 18.1 us against 17.1 / 18.8 / 18.7 / 21.6 for M = 96 / 128 / 256 / 512 at
         // N = K = 4096; with more tiles the larger tiles' operand reuse wins (M = 1024: 32 vs 23 us)
