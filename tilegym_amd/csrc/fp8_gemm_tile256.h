@@ -52,7 +52,8 @@ __global__ void __launch_bounds__(256, 1) fp8_gemm_tile256_kernel(const GemmPara
     const int K = p.K;
     const int tiles_n = (p.N + BN - 1) / BN, tiles_m = (p.M + BM - 1) / BM;
     // Persistent: workgroup b computes tiles b, b + gridDim.x, b + 2 gridDim.x, ... of the rastered tile sequence
-    // (gridDim.x is a multiple of 8, so a workgroup's tiles all belong to its XCD's range of the sequence).
+    // (with a grid that is a multiple of 8 -- the 256 compute units -- a workgroup's tiles all belong to its XCD's range of
+    // the sequence; any other grid computes the same tiles with less reuse in the L2s).
     const int total = tiles_m * tiles_n, stride = (int)gridDim.x;
     auto origin = [&](int v, int& om0, int& on0) {
         const int pid = xcd_remap(v, total);
