@@ -143,110 +143,110 @@ __global__ void __launch_bounds__(256, 1) fp8_gemm_tile256_kernel(const GemmPara
     // tile (in place of re-fetches past the end), so the next tile's first operands land while this tile's results
     // are converted and stored, and its first step finds them in LDS.
     int sa = 0, sb = 0;  // slabs that hold A(k) and B(k)
-    for (;;) {
-    const int cm0 = m0, cn0 = n0;  // this tile's origin (the offsets move on to the next tile two steps before the end)
-    bool more = false;
-    for (int k = 0; k < nsteps; ++k) {
-        if (k == nsteps - 2) {
-            more = vt + stride < total;
-            if (more) {
-                vt += stride;
-                origin(vt, m0, n0);
-                set_offsets(m0, n0);
+    for (;;) {  // tiles of this workgroup
+        const int cm0 = m0, cn0 = n0;  // this tile's origin (the offsets move on to the next tile two steps before the end)
+        bool more = false;
+        for (int k = 0; k < nsteps; ++k) {
+            if (k == nsteps - 2) {
+                more = vt + stride < total;
+                if (more) {
+                    vt += stride;
+                    origin(vt, m0, n0);
+                    set_offsets(m0, n0);
+                }
             }
-        }
-        int k2 = k + 2;                       // step the requests of this step are for
-        if (k2 >= nsteps) k2 = more ? k2 - nsteps : last;
-        const int sa1 = sa ^ 1;                              // holds/receives A(k+1)
-        const int sb1 = sb == B_STAGES - 1 ? 0 : sb + 1;     // holds B(k+1)
-        const int sb2 = sb1 == B_STAGES - 1 ? 0 : sb1 + 1;   // receives B(k+2)  (free: held B(k-1))
-        const uint8_t* cB = sB + sb * SLAB;
-        TG_FENCE();
-        // column tiles 0 .. 5 in halves of four MFMAs; behind each half of the first four a direct load (B(k+2) goes to
-        // the slab B(k-1) had), behind each first half the weight fragment of the column tile after next
+            int k2 = k + 2;                       // step the requests of this step are for
+            if (k2 >= nsteps) k2 = more ? k2 - nsteps : last;
+            const int sa1 = sa ^ 1;                              // holds/receives A(k+1)
+            const int sb1 = sb == B_STAGES - 1 ? 0 : sb + 1;     // holds B(k+1)
+            const int sb2 = sb1 == B_STAGES - 1 ? 0 : sb1 + 1;   // receives B(k+2)  (free: held B(k-1))
+            const uint8_t* cB = sB + sb * SLAB;
+            TG_FENCE();
+            // column tiles 0 .. 5 in halves of four MFMAs; behind each half of the first four a direct load (B(k+2) goes to
+            // the slab B(k-1) had), behind each first half the weight fragment of the column tile after next
 #pragma unroll
-        for (int tn = 0; tn < 6; ++tn) {
+            for (int tn = 0; tn < 6; ++tn) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+                for (int h = 0; h < 2; ++h) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[tn][4 * h + j] = mfma_e4m3(wf[tn & 3], af[4 * h + j], acc[tn][4 * h + j]);
+                    for (int j = 0; j < 4; ++j) acc[tn][4 * h + j] = mfma_e4m3(wf[tn & 3], af[4 * h + j], acc[tn][4 * h + j]);
+                    TG_FENCE();
+                    if (2 * tn + h < IT) load_b(2 * tn + h, k2, sb2);
+                    if (h == 0) wf[(tn + 2) & 3] = read_w(tn + 2, cB);
+                    TG_FENCE();
+                }
+            }
+            // B(k+1) and A(k+1) have landed (all but the eight requests of B(k+2)); all my reads of B(k) are done
+            __builtin_amdgcn_s_waitcnt(kWaitBut8);
+            __builtin_amdgcn_s_waitcnt(kWaitLds);
+            __builtin_amdgcn_s_barrier();
+            TG_FENCE();
+            // column tiles 6 and 7 by row group: each pair of MFMAs releases one activation fragment, which is refilled from
+            // A(k+1) at once; the first two weight fragments of step k+1 are read first.  A(k)'s slab is free (every wave
+            // read its fragments before this barrier) and receives A(k+2).
+            const uint8_t* nA = sA + sa1 * SLAB;
+            const uint8_t* nB = sB + sb1 * SLAB;
+            wf[0] = read_w(0, nB);
+            wf[1] = read_w(1, nB);
+            TG_FENCE();
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm) {
+                acc[6][tm] = mfma_e4m3(wf[2], af[tm], acc[6][tm]);
+                acc[7][tm] = mfma_e4m3(wf[3], af[tm], acc[7][tm]);
                 TG_FENCE();
-                if (2 * tn + h < IT) load_b(2 * tn + h, k2, sb2);
-                if (h == 0) wf[(tn + 2) & 3] = read_w(tn + 2, cB);
+                af[tm] = read_a(tm, nA);
+                load_a(tm, k2, sa);
                 TG_FENCE();
             }
+            sa = sa1;
+            sb = sb1;
         }
-        // B(k+1) and A(k+1) have landed (all but the eight requests of B(k+2)); all my reads of B(k) are done
-        __builtin_amdgcn_s_waitcnt(kWaitBut8);
-        __builtin_amdgcn_s_waitcnt(kWaitLds);
-        __builtin_amdgcn_s_barrier();
-        TG_FENCE();
-        // column tiles 6 and 7 by row group: each pair of MFMAs releases one activation fragment, which is refilled from
-        // A(k+1) at once; the first two weight fragments of step k+1 are read first.  A(k)'s slab is free (every wave
-        // read its fragments before this barrier) and receives A(k+2).
-        const uint8_t* nA = sA + sa1 * SLAB;
-        const uint8_t* nB = sB + sb1 * SLAB;
-        wf[0] = read_w(0, nB);
-        wf[1] = read_w(1, nB);
-        TG_FENCE();
+        // the fragment reads issued for the step after the last one are never used; keep the compiler from deleting the
+        // loop-carried registers' last assignment in a way that changes the loop body
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) asm volatile("" : : "v"(af[tm]));
+        asm volatile("" : : "v"(wf[0]), "v"(wf[1]));
+
+        // ---- epilogue, straight from the accumulators (as fp8_gemm_tile.h)
+        const int rows_valid = min(BM, p.M - cm0);
+        float scale = p.alpha;
+        if (p.As) scale *= p.As[0];
+        if (p.Bs) scale *= p.Bs[0];
+        const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;
+        int dsts[TM];
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
-            acc[6][tm] = mfma_e4m3(wf[2], af[tm], acc[6][tm]);
-            acc[7][tm] = mfma_e4m3(wf[3], af[tm], acc[7][tm]);
-            TG_FENCE();
-            af[tm] = read_a(tm, nA);
-            load_a(tm, k2, sa);
-            TG_FENCE();
+            const int rt = (tm * WGM + wm) * 16 + li;
+            dsts[tm] = rt < rows_valid ? cm0 + rt : -1;
         }
-        sa = sa1;
-        sb = sb1;
-    }
-    // the fragment reads issued for the step after the last one are never used; keep the compiler from deleting the
-    // loop-carried registers' last assignment in a way that changes the loop body
+        auto emit = [&](auto type_tag) __attribute__((always_inline)) {
+            constexpr int OT = decltype(type_tag)::value;
+            // (one call per row group instead of a loop: the body is too large for the unroller's budget, and a loop that
+            // stays a loop would index the accumulators at run time, i.e. put them in scratch memory)
+            auto rows = [&](auto tm_tag) __attribute__((always_inline)) {
+                constexpr int tm = decltype(tm_tag)::value;
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm) asm volatile("" : : "v"(af[tm]));
-    asm volatile("" : : "v"(wf[0]), "v"(wf[1]));
-
-    // ---- epilogue, straight from the accumulators (as fp8_gemm_tile.h)
-    const int rows_valid = min(BM, p.M - cm0);
-    float scale = p.alpha;
-    if (p.As) scale *= p.As[0];
-    if (p.Bs) scale *= p.Bs[0];
-    const bool vec_ok = p.vec_store != 0 && (p.N % 8) == 0;
-    int dsts[TM];
-#pragma unroll
-    for (int tm = 0; tm < TM; ++tm) {
-        const int rt = (tm * WGM + wm) * 16 + li;
-        dsts[tm] = rt < rows_valid ? cm0 + rt : -1;
-    }
-    auto emit = [&](auto type_tag) __attribute__((always_inline)) {
-        constexpr int OT = decltype(type_tag)::value;
-        // (one call per row group instead of a loop: the body is too large for the unroller's budget, and a loop that
-        // stays a loop would index the accumulators at run time, i.e. put them in scratch memory)
-        auto rows = [&](auto tm_tag) __attribute__((always_inline)) {
-            constexpr int tm = decltype(tm_tag)::value;
-#pragma unroll
-            for (int tp = 0; tp < TN / 2; ++tp) {
-                const int col = cn0 + wn * WTN + tp * 32 + lg * 8;
-                if (dsts[tm] < 0 || col >= p.N) continue;
-                store8(p.C, OT, dsts[tm], col, p.N, p.ldc, acc[2 * tp][tm] * scale, acc[2 * tp + 1][tm] * scale, p.beta, vec_ok);
-            }
+                for (int tp = 0; tp < TN / 2; ++tp) {
+                    const int col = cn0 + wn * WTN + tp * 32 + lg * 8;
+                    if (dsts[tm] < 0 || col >= p.N) continue;
+                    store8(p.C, OT, dsts[tm], col, p.N, p.ldc, acc[2 * tp][tm] * scale, acc[2 * tp + 1][tm] * scale, p.beta, vec_ok);
+                }
+            };
+            rows(std::integral_constant<int, 0>{}); rows(std::integral_constant<int, 1>{});
+            rows(std::integral_constant<int, 2>{}); rows(std::integral_constant<int, 3>{});
+            rows(std::integral_constant<int, 4>{}); rows(std::integral_constant<int, 5>{});
+            rows(std::integral_constant<int, 6>{}); rows(std::integral_constant<int, 7>{});
         };
-        rows(std::integral_constant<int, 0>{}); rows(std::integral_constant<int, 1>{});
-        rows(std::integral_constant<int, 2>{}); rows(std::integral_constant<int, 3>{});
-        rows(std::integral_constant<int, 4>{}); rows(std::integral_constant<int, 5>{});
-        rows(std::integral_constant<int, 6>{}); rows(std::integral_constant<int, 7>{});
-    };
-    if (p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
-    else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
-    else if (p.out_type == OUT_F8) emit(std::integral_constant<int, OUT_F8>{});
-    else emit(std::integral_constant<int, OUT_F16>{});
-    if (!more) break;
+        if (p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
+        else if (p.out_type == OUT_F32) emit(std::integral_constant<int, OUT_F32>{});
+        else if (p.out_type == OUT_F8) emit(std::integral_constant<int, OUT_F8>{});
+        else emit(std::integral_constant<int, OUT_F16>{});
+        if (!more) break;
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
+        for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
-    }  // tiles
+            for (int tm = 0; tm < TM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
 #undef TG_FENCE
     __builtin_amdgcn_s_waitcnt(kWaitAll);  // the re-fetches past the end must land before the workgroup's LDS is released
 #endif
