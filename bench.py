@@ -156,6 +156,32 @@ def _graph_ms(fn, launches, replays, stream):
         return None
 
 
+def _vendor_yardstick(runners, shapes, steps, stream):
+    """The same per-tensor prefill GEMMs through the vendor library (torch._scaled_mm -> hipBLASLt) on the same operand
+    tensors, same process, each after its own load ramp: a yardstick for what this GPU sustains on the shape, not part
+    of the product path and not a baseline of the reference.  Adds `vendor_us` to every prefill shape."""
+    try:
+        total_us = 0.0
+        same = True
+        for r, sh in zip(runners, shapes):
+            sa, sb = r.sa.reshape(()), r.sb.reshape(())
+            fn = lambda i, r=r, sa=sa, sb=sb: torch._scaled_mm(r.a[i % r.copies], r.b[i % r.copies].t(), scale_a=sa, scale_b=sb,  # noqa: E731
+                                                               out_dtype=torch.bfloat16)
+            _ramp(fn)
+            us = _events_ms(fn, steps, stream) * 1e3 / steps
+            sh["vendor_us"] = round(us, 2)
+            total_us += us
+            r(0)
+            torch.cuda.synchronize()
+            same = same and bool(torch.equal(fn(0), r.c[0]))
+        flops = sum(r.case.flops() for r in runners)
+        return {"library": "torch._scaled_mm (hipBLASLt), same operands", "sum_us": round(total_us, 1),
+                "tflops": round(flops / total_us * 1e-6, 1), "outputs_bit_identical_to_ours": same,
+                "ours_sum_us": round(sum(sh["us"] for sh in shapes), 1)}
+    except Exception as exc:  # the yardstick must never break the bench line
+        return {"library": "torch._scaled_mm", "error": f"{type(exc).__name__}: {exc}"[:200]}
+
+
 class DenseRunner:
     """One dense problem with its operands replicated `copies` times for cache-cold rotation."""
 
@@ -278,6 +304,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-vendor", action="store_true", help="skip the vendor-library yardstick of the prefill shapes")
     ap.add_argument("--workload", default="all", choices=["prefill", "decode", "block", "moe", "quant", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time microsecond kernels with plain launches")
@@ -338,6 +365,8 @@ def main():
                          "shape": dom["name"], "us_per_launch": dom["us"]},
         })
         detail["prefill"] = shapes
+        if not args.no_vendor:
+            out["vendor_yardstick"] = _vendor_yardstick(runners, shapes, args.steps, stream)
         del runners
         torch.cuda.empty_cache()
 
