@@ -64,8 +64,11 @@ enum {
     TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (32/64/128/256; 32x32, 64x32 and 64x64 = in-workgroup K split, per-tensor only) */
     TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (32/64/128/256)        */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
-    TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4); stream kernel: LDS buffers per wave (1/2) */
-    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup; tiled 256x256 per-tensor kernel: 8 = the generic eight-wave tile kernel instead of the persistent four-wave one */
+    TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4); stream kernel: LDS buffers per wave (1/2);
+                            * tiled 256x256 block-scaled kernels (dense and ragged): 1 = the persistent form (one workgroup per
+                            * compute unit walks the tiles, three weight slabs in LDS, scales in registers); the ragged GEMM
+                            * chooses it by itself for K <= 1536 */
+    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup; tiled 256x256 kernels: 8 = the generic eight-wave tile kernel (one workgroup per tile) instead of the persistent one */
     TG_CFG_QUANT_BLOCK_N = 6, /* block-scaled tg_fp8_gemm: weight rows per scale (default 128) */
     TG_CFG_QUANT_BLOCK_K = 7, /* block-scaled tg_fp8_gemm: K elements per scale (default 128); blocks other than 128 x 128
                                * run on the fallback kernel (no MFMA): the reference's block_size=[bn, bk] argument,

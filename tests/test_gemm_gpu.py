@@ -617,6 +617,91 @@ def test_block_scaled_tiled_configs_and_edges(device, bm, bn, M, N, K):
     check(out, ref, what=f"block-scaled {bm}x{bn}")
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (300, 520, 1280), (1000, 1000, 384), (2048, 1024, 1408), (768, 256, 768),
+                                   (520, 300, 896), (700, 512, 1024), (256, 512, 5120), (512, 768, 512)])
+def test_block_scaled_persistent_256(device, M, N, K):
+    """The persistent form of the block-scaled 256x256 tile (ROW_GROUPS = 1): three weight slabs, scales in registers in
+    chunks of four K steps.  K steps that are a multiple of four and not (the last chunk holds 2 or 3 steps), a single
+    chunk, ten chunks; ragged M and N; bf16 and f32 outputs.  Against the oracle, and bit for bit against the kernel of
+    one workgroup per tile (WAVES = 8)."""
+    case = W.block_scaled_case(M, N, K, seed=M + N + K)
+    d = case.to(device)
+    kc = {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "SPLIT_K": 1, "ROW_GROUPS": 1}
+    for dtype in (torch.bfloat16, torch.float32):
+        ref = R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, dtype)
+        out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, dtype, kernel_configs=kc)
+        cfg = used("tiled")
+        assert (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["ROW_GROUPS"]) == (256, 256, 1), cfg
+        check(out, ref, what=f"persistent block-scaled M={M} N={N} K={K} {dtype}")
+        other = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, dtype, kernel_configs=dict(kc, ROW_GROUPS=-1, WAVES=8))
+        assert _lib.last_config()["ROW_GROUPS"] != 1
+        assert torch.equal(out, other), "persistent and one-workgroup-per-tile block-scaled kernels differ"
+
+
+def test_block_scaled_persistent_256_refuses_a_single_step_last_chunk(device):
+    """K % 512 == 128 (a last chunk of scales of one step) stays with the kernel of one workgroup per tile, also when the
+    persistent form is asked for."""
+    case = W.block_scaled_case(300, 256, 640, seed=9)
+    d = case.to(device)
+    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16,
+                                kernel_configs={"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "ROW_GROUPS": 1})
+    assert used("tiled")["ROW_GROUPS"] != 1
+    check(out, R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16))
+
+
+def test_block_scaled_persistent_256_walks_several_tiles_per_workgroup(device):
+    """More tiles than compute units: workgroups compute two tiles, the operand rings and the scale chunks run on from one
+    tile into the next (K = 768: the first tile's last chunk is partial); a partial row tile and a partial column tile."""
+    M, N, K = 4300, 4360, 768
+    assert math.ceil(M / 256) * math.ceil(N / 256) > torch.cuda.get_device_properties(device).multi_processor_count
+    case = W.block_scaled_case(M, N, K, seed=4)
+    d = case.to(device)
+    kc = {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "SPLIT_K": 1, "ROW_GROUPS": 1}
+    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs=kc)
+    assert used("tiled")["ROW_GROUPS"] == 1
+    other = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs=dict(kc, ROW_GROUPS=-1, WAVES=8))
+    assert torch.equal(out, other)
+    rows = torch.cat([torch.arange(0, 3), torch.arange(254, 259), torch.randint(0, M, (24,), generator=_g(1)), torch.arange(M - 3, M)])
+    ref = R.ref_w8a8_block_fp8_matmul(case.a[rows], case.b, case.scale_a[rows], case.scale_b, None, torch.bfloat16)
+    check(out[rows.to(device)], ref, what="persistent block-scaled, several tiles per workgroup")
+
+
+@pytest.mark.parametrize("N,K", [(392, 256), (512, 768), (300, 1408), (256, 2048)])
+def test_ragged_persistent_256(device, N, K):
+    """The persistent block-scaled kernel over ragged expert segments (ROW_GROUPS = 1; the default for K <= 1536): empty,
+    tiny, unaligned and multi-tile experts, rows of no segment untouched; against the oracle and bit for bit against the
+    kernel of one workgroup per tile; more than 64 experts."""
+    sizes = [5, 0, 131, 64, 0, 0, 600, 1, 77, 256, 300]
+    a, b, a_s, b_s, ptr = _ragged_inputs(sizes, N, K, 17 + K, total_extra=6)
+    ref = R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr)
+    impl = tilegym_amd.backend._REGISTRY["flashinfer.gemm.ragged_block_scaled_bmm"]["hip"]
+    kc = {"BLOCK_M": 256, "BLOCK_N": 256, "ROW_GROUPS": 1}
+    out = impl(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), max(sizes), kernel_configs=kc, zero_init=True)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["ROW_GROUPS"]) == (256, 256, 1), cfg
+    check(out, ref, what=f"ragged persistent N={N} K={K}")
+    assert torch.equal(out[sum(sizes):].cpu().float(), torch.zeros(6, N))
+    other = impl(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), max(sizes),
+                 kernel_configs={"BLOCK_M": 256, "BLOCK_N": 256, "WAVES": 8}, zero_init=True)
+    assert _lib.last_config()["ROW_GROUPS"] != 1
+    assert torch.equal(out, other), "persistent and one-workgroup-per-tile ragged kernels differ"
+    sizes2 = torch.randint(0, 40, (150,), generator=_g(K)).tolist()
+    a, b, a_s, b_s, ptr = _ragged_inputs(sizes2, 256, K, 5)
+    out = impl(a.to(device), b.to(device), a_s.to(device), b_s.to(device), ptr.to(device), max(sizes2), kernel_configs=kc)
+    check(out, R.ref_ragged_block_scaled_bmm(a, b, a_s, b_s, ptr), what="ragged persistent, 150 experts")
+
+
+def test_ragged_persistent_256_is_the_default_for_short_k(device):
+    a, b, a_s, b_s, ptr = _ragged_inputs([300] * 8, 512, 1408, 3)
+    dev = [t.to(device) for t in (a, b, a_s, b_s, ptr)]
+    ragged_block_scaled_bmm(*dev, 300)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["ROW_GROUPS"]) == (256, 256, 1), cfg
+    a, b, a_s, b_s, ptr = _ragged_inputs([300] * 8, 512, 2048, 3)
+    ragged_block_scaled_bmm(*[t.to(device) for t in (a, b, a_s, b_s, ptr)], 300)
+    assert used("tiled")["ROW_GROUPS"] != 1
+
+
 @pytest.mark.parametrize("M", [1, 16, 40, 64])
 @pytest.mark.parametrize("split", [1, 4])
 @pytest.mark.parametrize("kernel,K", [("skinny", 1024), ("stream", 1024), ("stream", 4224)])

@@ -6,7 +6,7 @@
 namespace tg {
 
 // Compute units of the current device: the persistent 256x256 kernel runs one workgroup on each.
-static int compute_units() {
+int compute_units() {
     static int cached[64];  // by device ordinal; 0 = not asked yet (racing first calls write the same value)
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;

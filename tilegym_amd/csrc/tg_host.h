@@ -28,6 +28,15 @@ hipError_t run_tile256(const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_tile_mid(int bm, int bn, const GemmParams& p, hipStream_t s);
 // 64x128 per-tensor tile with four LDS stages (loads three K steps ahead): the 16 < M <= 64 form
 hipError_t run_tile_deep(bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
+// 256x256 block-scaled tile, persistent (one workgroup per compute unit walks the tiles), dense rows or ragged expert
+// segments: same results as the 256 x 256 forms of run_tile_block_dense / run_tile_block_grouped.  Needs K >= 256,
+// both scale tensors; tiles_bound = an upper bound of the number of tiles
+hipError_t run_bs256(int group, const GemmParams& p, int tiles_bound, hipStream_t s);
+// K steps run_bs256 takes: at least two, and not 4c + 1 (a last chunk of scales of a single step); the weights of all
+// experts together must also stay below 4 GiB
+inline bool bs256_takes_k(int kblocks) { return kblocks >= 2 && kblocks % 4 != 1; }
+// compute units of the current device
+int compute_units();
 hipError_t run_tile_block_dense(int bm, int bn, bool split, const GemmParams& p, int gx, int gy, hipStream_t s);
 hipError_t run_tile_moe_act(int bm, const GemmParams& p, int gx, hipStream_t s);
 hipError_t run_tile_block_grouped(int bm, int bn, int group, const GemmParams& p, int gx, hipStream_t s);
