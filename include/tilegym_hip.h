@@ -73,7 +73,10 @@ enum {
     TG_CFG_QUANT_BLOCK_K = 7, /* block-scaled tg_fp8_gemm: K elements per scale (default 128); blocks other than 128 x 128
                                * run on the fallback kernel (no MFMA): the reference's block_size=[bn, bk] argument,
                                * src/tilegym/suites/unsloth/cutile/fp8.py:388-446 */
-    TG_CFG_COUNT = 8
+    TG_CFG_PIECES = 8,  /* reported by tg_last_config only: 1, or the number of separately scheduled pieces the call ran as
+                         * (column chunks of a weight of 2 GiB and more; the columns or rows that fill whole rounds of the chip
+                         * with 256x256 tiles and the rest): the other slots then describe the first piece.  Ignored in cfg[]. */
+    TG_CFG_COUNT = 9
 };
 
 /*

@@ -200,7 +200,33 @@ def test_weights_of_2_gib_and_more_run_in_column_chunks(device):
         b_deq = b_cols.float().view(len(cols), K // 128, 128) * Bs[cols // 128][:, :, None]
         ref = (a_deq.reshape(M, K).double() @ b_deq.reshape(len(cols), K).double().T).to(torch.bfloat16)
         check(out[:, cols.to(device)], ref, what=f"2 GiB weight, block scales, M={M}")
+        assert _lib.last_config()["PIECES"] == 2
     del codes, b_dev
+
+
+def test_column_piece_with_more_than_one_row_chunk(device):
+    """Both chunkings at once: M = 16384, N = 1280, K = 131072 is 320 tiles of 256 x 256 (1.25 rounds), so columns
+    0 .. 1023 and 1024 .. 1279 run as two pieces of a C that is 1280 wide, and the activations are 2 GiB, so every piece
+    walks its rows in two chunks (32-bit byte offsets).  The second row chunk of a piece must land at row stride 1280, not
+    at the piece's own width: rows either side of the chunk boundary, in both column pieces, against the oracle."""
+    M, N, K = 16384, 1280, 131072
+    g = _g(5)
+    codes = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=device)
+    codes[(codes & 0x7F) == 0x7F] = 0x38
+    codes &= 0xBF
+    a_dev = codes.view(FP8)
+    b = fp8_randn((N, K), g, 0.5)
+    sa, sb = torch.tensor([0.02]), torch.tensor([0.01])
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=device)
+    _lib.fp8_gemm(out, a_dev, b.to(device), sa.to(device), sb.to(device), False, True, 1.0, 0.0, None)
+    cfg = _lib.last_config()
+    assert cfg["KERNEL_NAME"] == "tiled" and cfg["PIECES"] == 2, cfg
+    boundary = ((1 << 31) - 1) // K // 256 * 256     # first row of the second row chunk
+    rows = torch.tensor([0, 1, 255, boundary - 1, boundary, boundary + 1, boundary + 200, M - 1])
+    ref = R.ref_gemm_per_tensor(a_dev[rows.to(device)].cpu(), b, sa, sb, trans_b=True)
+    check(out[rows.to(device)], ref, what="column pieces x row chunks")
+    assert not torch.isnan(out.float()).any()
+    del codes, a_dev, out
 
 
 @pytest.mark.parametrize("block_size", [[64, 64], [64, 128], [256, 32], [128, 256], [48, 80]])
@@ -259,8 +285,8 @@ def test_columns_split_where_256_tiles_leave_the_last_round_mostly_empty(device,
     ad, bd, sad, sbd = a.to(device), b.to(device), sa.to(device), sb.to(device)
     out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=device)
     _lib.fp8_gemm(out, ad, bd, sad, sbd, False, True, 1.0, 0.0, None)
-    cfg = _lib.last_config()          # the schedule of the last piece: the 512 remaining columns
-    assert cfg["KERNEL_NAME"] == "tiled" and (cfg["BLOCK_M"], cfg["BLOCK_N"]) != (256, 256), cfg
+    cfg = _lib.last_config()          # the schedule of the first piece (the columns that fill whole rounds) and the piece count
+    assert cfg["KERNEL_NAME"] == "tiled" and (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["PIECES"]) == (256, 256, 2), cfg
     one = torch.empty_like(out)
     _lib.fp8_gemm(one, ad, bd, sad, sbd, False, True, 1.0, 0.0, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256})
     assert torch.equal(out, one)
@@ -295,7 +321,7 @@ def test_rows_split_where_256_tiles_leave_the_last_round_mostly_empty(device, bl
     out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=device)
     _lib.fp8_gemm(out, ad, bd, sad, sbd, False, True, 1.0, 0.0, None)
     cfg = _lib.last_config()
-    assert cfg["KERNEL_NAME"] == "tiled" and (cfg["BLOCK_M"], cfg["BLOCK_N"]) != (256, 256), cfg
+    assert cfg["KERNEL_NAME"] == "tiled" and (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["PIECES"]) == (256, 256, 2), cfg
     one = torch.empty_like(out)
     _lib.fp8_gemm(one, ad, bd, sad, sbd, False, True, 1.0, 0.0, {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256})
     assert torch.equal(out, one)

@@ -20,9 +20,9 @@ LIB_ENV = "TILEGYM_HIP_LIB"
 DEFAULT_LIB_PATH = os.path.join(_HERE, "libtilegym_hip.so")
 
 TG_MAX_DIMS = 5
-TG_CFG_COUNT = 8
+TG_CFG_COUNT = 9
 CFG_SLOTS = {"KERNEL": 0, "BLOCK_M": 1, "BLOCK_N": 2, "SPLIT_K": 3, "ROW_GROUPS": 4, "WAVES": 5,
-             "QUANT_BLOCK_N": 6, "QUANT_BLOCK_K": 7}
+             "QUANT_BLOCK_N": 6, "QUANT_BLOCK_K": 7, "PIECES": 8}
 KERNEL_NAMES = {0: "fallback", 1: "tiled", 2: "skinny", 3: "stream"}
 
 # dtype codes of the ABI (include/tilegym_hip.h)

@@ -17,7 +17,7 @@ static __device__ __align__(256) unsigned char scratch[TG_STATIC_SCRATCH_BYTES];
 namespace {
 
 thread_local char g_err[512] = "";
-thread_local int32_t g_last_cfg[TG_CFG_COUNT] = {-1, -1, -1, -1, -1, -1, -1, -1};
+thread_local int32_t g_last_cfg[TG_CFG_COUNT] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
 
 int32_t fail(int32_t rc, const char* fmt, ...) {
     va_list ap;
@@ -81,7 +81,6 @@ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 constexpr int64_t kOffsetLimit = (int64_t)1 << 31;  // kernels index operands with 32-bit byte offsets
-thread_local int64_t g_chunk_ldc = 0;               // row stride of C for the next fp8_gemm_impl call (column chunks), 0 = N
 constexpr int kTargetWaves = 4096;                  // 16 waves on each of 256 CUs
 constexpr int64_t kBs256WeightLimit = ((int64_t)1 << 32) - 1;  // the persistent block-scaled kernel addresses all experts' weights with one 32-bit offset
 
@@ -136,7 +135,22 @@ void remember(const Schedule& s) {
     g_last_cfg[TG_CFG_SPLIT_K] = s.split_k;
     g_last_cfg[TG_CFG_ROW_GROUPS] = s.row_groups;
     g_last_cfg[TG_CFG_WAVES] = s.waves;
+    g_last_cfg[TG_CFG_PIECES] = 1;
 }
+
+// A call that ran as several pieces reports the schedule of its first piece and the number of pieces.
+struct PieceRecord {
+    int32_t first[TG_CFG_COUNT];
+    int count = 0;
+    void after_piece() {
+        if (count++ == 0) memcpy(first, g_last_cfg, sizeof(first));
+    }
+    void publish() const {
+        if (count == 0) return;
+        memcpy(g_last_cfg, first, sizeof(first));
+        g_last_cfg[TG_CFG_PIECES] = count;
+    }
+};
 
 // Tiles of fp8_gemm_tile_mid_kernel.
 bool is_mid_tile(int bm, int bn) { return ((bm == 64 || bm == 32) && bn == 32) || (bm == 64 && bn == 64); }
@@ -304,10 +318,12 @@ struct Resolved {
 // Body of tg_fp8_gemm and tg_fp8_gemm_static_scratch.  static_scratch: the workspace is the library's
 // own `scratch` array instead of a caller's buffer, and a problem whose schedule needs more than it holds
 // is rejected instead of run with a smaller split.
+// piece_ldc: 0 for a whole problem; for a piece of a larger problem (a column or row range computed as a call of its own)
+// the row stride of C in elements -- the piece is then described as (M, columns of the piece) and is not split again.
 int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b, const tg_tensor* scale_a,
                       const tg_tensor* scale_b, int32_t trans_a, int32_t trans_b, float alpha, float beta,
                       const tg_tensor* workspace, bool static_scratch, const int32_t* cfg, int32_t ncfg,
-                      int32_t device_id, uint64_t hip_stream);
+                      int32_t device_id, uint64_t hip_stream, int64_t piece_ldc = 0);
 
 }  // namespace
 
@@ -374,13 +390,10 @@ namespace {
 int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b, const tg_tensor* scale_a,
                       const tg_tensor* scale_b, int32_t trans_a, int32_t trans_b, float alpha, float beta,
                       const tg_tensor* workspace, bool static_scratch, const int32_t* cfg, int32_t ncfg,
-                      int32_t device_id, uint64_t hip_stream) {
+                      int32_t device_id, uint64_t hip_stream, int64_t piece_ldc) {
     g_err[0] = 0;
     int32_t rc;
-    // (a column chunk of a wider C, handed down by the chunk loop below, is described as (M, chunk) with its real row
-    // stride in g_chunk_ldc)
-    const int64_t chunk_ldc = g_chunk_ldc;
-    g_chunk_ldc = 0;
+    const int64_t chunk_ldc = piece_ldc;
     if ((rc = check_tensor(a, "a", 2)) || (rc = check_tensor(b, "b", 2)) || (rc = check_tensor(c, "c", 2))) return rc;
     if (a->dtype != TG_F8E4M3FN || b->dtype != TG_F8E4M3FN)
         return fail(TG_ERR_DTYPE, "a and b must be float8_e4m3fn (dtype code 7), got %d and %d", a->dtype, b->dtype);
@@ -429,14 +442,14 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
     if (M == 0 || N == 0) return TG_OK;
 
     // ---- column chunks.  The columns of C (rows of an (N, K) weight) can be computed in pieces, each a call of its own on
-    // the same stream and workspace; the pieces take C's real row stride in g_chunk_ldc.
+    // the same stream and workspace; the pieces take C's real row stride as an argument.
     auto run_columns = [&](int64_t n0, int64_t cn) -> int32_t {
         tg_tensor bs = *b, cs = *c, sbs;
         bs.ptr = b->ptr + (uint64_t)(n0 * K);
         bs.shape[0] = cn;
         cs.ptr = c->ptr + (uint64_t)(n0 * elem_size(c->dtype));
         cs.shape[1] = cn;
-        cs.strides[0] = cn;  // described as contiguous; the real row stride travels in g_chunk_ldc
+        cs.strides[0] = cn;  // described as contiguous; the real row stride is the piece_ldc argument
         const tg_tensor* sb = scale_b;
         if (kb == BLOCK) {
             sbs = *scale_b;
@@ -444,18 +457,19 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
             sbs.shape[0] = cdiv(cn, 128);
             sb = &sbs;
         }
-        g_chunk_ldc = N;
-        const int32_t r = fp8_gemm_impl(&cs, a, &bs, scale_a, sb, trans_a, trans_b, alpha, beta, workspace, static_scratch, cfg, ncfg, device_id, hip_stream);
-        g_chunk_ldc = 0;
-        return r;
+        return fp8_gemm_impl(&cs, a, &bs, scale_a, sb, trans_a, trans_b, alpha, beta, workspace, static_scratch, cfg, ncfg, device_id, hip_stream, N);
     };
     const bool can_chunk = !chunk_ldc && std_blocks && trans_b && !trans_a && K > 0 && (K % 16) == 0 && aligned16(a->ptr) &&
                            aligned16(b->ptr) && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
     // (1) weights of 2 GiB and more: the kernels index an operand with 32-bit byte offsets
     if (can_chunk && N * K >= kOffsetLimit && 256 * K < kOffsetLimit) {
         const int64_t chunk_n = ((kOffsetLimit - 1) / K) / 256 * 256;
-        for (int64_t n0 = 0; n0 < N; n0 += chunk_n)
+        PieceRecord pieces;
+        for (int64_t n0 = 0; n0 < N; n0 += chunk_n) {
             if ((rc = run_columns(n0, (N - n0) < chunk_n ? (N - n0) : chunk_n))) return rc;
+            pieces.after_piece();
+        }
+        pieces.publish();
         return TG_OK;
     }
     // (2) 256 x 256 tiles whose count leaves the last round of the chip mostly empty (4096 x 5120: 320 tiles, 1.25 rounds):
@@ -468,9 +482,14 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
             auto fills = [](int64_t tiles) { return tiles >= 256 && tiles * 100 >= cdiv(tiles, 256) * 256 * 95; };
             const int64_t n1 = ((total / 256) * 256) / tm;   // column tiles that fit the whole rounds
             const int64_t m1 = ((total / 256) * 256) / tn;   // or row tiles
+            PieceRecord pieces;
             if (n1 >= 1 && n1 < tn && fills(tm * n1)) {
                 if ((rc = run_columns(0, n1 * 256))) return rc;
-                return run_columns(n1 * 256, N - n1 * 256);
+                pieces.after_piece();
+                if ((rc = run_columns(n1 * 256, N - n1 * 256))) return rc;
+                pieces.after_piece();
+                pieces.publish();
+                return TG_OK;
             }
             if (m1 >= 1 && m1 < tm && fills(m1 * tn)) {
                 // the same along the rows: the pieces are contiguous row ranges of A, C and the activation scales
@@ -488,11 +507,12 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
                         sas.shape[0] = rows;
                         sa = &sas;
                     }
-                    g_chunk_ldc = N;  // (marks the call as a piece: no further splitting)
-                    rc = fp8_gemm_impl(&cs, &as, b, sa, scale_b, trans_a, trans_b, alpha, beta, workspace, static_scratch, cfg, ncfg, device_id, hip_stream);
-                    g_chunk_ldc = 0;
+                    // (piece_ldc = N marks the call as a piece: no further splitting)
+                    rc = fp8_gemm_impl(&cs, &as, b, sa, scale_b, trans_a, trans_b, alpha, beta, workspace, static_scratch, cfg, ncfg, device_id, hip_stream, N);
                     if (rc) return rc;
+                    pieces.after_piece();
                 }
+                pieces.publish();
                 return TG_OK;
             }
         }
@@ -620,7 +640,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         const int64_t rows = (M - r0) < max_rows ? (M - r0) : max_rows;
         tg::GemmParams pc = p;
         pc.A = p.A + r0 * K;
-        pc.C = reinterpret_cast<uint8_t*>(p.C) + r0 * N * elem_size(c->dtype);
+        pc.C = reinterpret_cast<uint8_t*>(p.C) + r0 * ldc * elem_size(c->dtype);  // (ldc, not N: this call may be a column piece of a wider C)
         if (block_scaled && p.As) pc.As = p.As + r0 * kblocks;
         pc.M = (int)rows;
         if (rows != M && s.split_k > 1) { pc.split_k = 1; pc.ksteps_per_split = (int)kblocks; }
