@@ -1511,19 +1511,27 @@ def test_config2_llama_decode_full(device, proj):
         check(out, ref, what=f"config 2 {proj} M={M}")
 
 
+def check_all_rows(out, ref_rows, M, what, rows_per_pass=2048):
+    """Every row of `out` (on the device) against the oracle, `rows_per_pass` rows at a time: ref_rows(lo, hi) returns the
+    oracle's rows lo .. hi-1.  Bounds the host memory of a full-size comparison."""
+    for lo in range(0, M, rows_per_pass):
+        hi = min(M, lo + rows_per_pass)
+        check(out[lo:hi], ref_rows(lo, hi), what=f"{what} rows {lo}..{hi - 1}")
+
+
 @pytest.mark.parametrize("proj", list(W.LLAMA_SHAPES))
 def test_config3_llama_prefill_sampled_rows(device, proj):
-    """Full-size launch; the oracle is evaluated on ~98 activation rows, three from every 256-row tile and walking
-    through every 16-row group slot of a tile (each output row depends on its own activation row only), and on
-    linearity across the whole output."""
+    """Full-size launch, and the whole output against the oracle: every tile, wave and row-group slot of the persistent
+    kernel's walk (the name is from when rows were sampled).  Plus linearity across the whole output."""
     case = W.llama_prefill_case(proj)
     d = case.to(device)
     out = matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a, scale_b=d.scale_b, out_dtype=torch.bfloat16)
     cfg = used("tiled")
     assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) == (256, 256)
-    rows = _rows_stratified(case.M, 3)
-    ref = R.ref_gemm_per_tensor(case.a[rows], case.b, case.scale_a, case.scale_b, trans_b=True)
-    check(out[rows.to(device)], ref, what=f"config 3 {proj}")
+    b_deq_t = (R.fp8_to_f32(case.b) * case.scale_b).t().contiguous()
+    check_all_rows(out, lambda lo, hi: ((R.fp8_to_f32(case.a[lo:hi]) * case.scale_a) @ b_deq_t).to(torch.bfloat16), case.M,
+                   f"config 3 {proj}")
+    del b_deq_t
     assert torch.isfinite(out.float()).all()
     # doubling a scale doubles every element exactly (bf16, power of two)
     out2 = matmul(d.a, d.b, trans_b=True, scale_a=d.scale_a * 2, scale_b=d.scale_b, out_dtype=torch.bfloat16)
@@ -1536,9 +1544,14 @@ def test_config4_block_scaled_full(device, N, K):
     d = big.to(device)
     out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16)
     used("tiled")
-    rows = _rows_stratified(4096, 4)  # every 256- and 128-row tile, every 16-row group slot
+    # the whole output (the weights are dequantized once)
+    b_deq_t = (R.fp8_to_f32(big.b).view(N // 128, 128, K // 128, 128) * big.scale_b[:, None, :, None]).view(N, K).t().contiguous()
+    check_all_rows(out, lambda lo, hi: ((R.fp8_to_f32(big.a[lo:hi]).view(hi - lo, K // 128, 128) * big.scale_a[lo:hi, :, None])
+                                        .view(hi - lo, K) @ b_deq_t).to(torch.bfloat16), 4096, f"config 4 M=4096 {N}x{K}", 1024)
+    del b_deq_t
+    rows = _rows_stratified(4096, 1)  # and the oracle function itself on a few rows (it dequantizes the same way)
     ref = R.ref_w8a8_block_fp8_matmul(big.a[rows], big.b, big.scale_a[rows], big.scale_b, None, torch.bfloat16)
-    check(out[rows.to(device)], ref, what=f"config 4 M=4096 {N}x{K}")
+    check(out[rows.to(device)], ref, what=f"config 4 M=4096 {N}x{K} (oracle function)")
     out16 = w8a8_block_fp8_matmul(d.a[:16].contiguous(), d.b, d.scale_a[:16].contiguous(), d.scale_b, None, torch.bfloat16)
     used("stream")
     ref16 = R.ref_w8a8_block_fp8_matmul(big.a[:16], big.b, big.scale_a[:16], big.scale_b, None, torch.bfloat16)
@@ -1553,9 +1566,8 @@ def test_config5_moe_grouped_full(device, which):
     assert int(case.m_indptr[-1]) == 4096 * 6 and sizes.min() != sizes.max()  # uneven experts
     out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, int(sizes.max()))
     used("tiled")
-    # per-expert reference GEMMs on a subset of experts (smallest, largest, first, last + 4 others)
-    experts = sorted({0, 63, int(sizes.argmin()), int(sizes.argmax()), 7, 21, 38, 50})
-    for e in experts:
+    # per-expert reference GEMMs, all 64 experts
+    for e in range(case.b.shape[0]):
         lo, hi = int(case.m_indptr[e]), int(case.m_indptr[e + 1])
         ref = R.ref_w8a8_block_fp8_matmul(case.a[lo:hi], case.b[e], case.a_scale[lo:hi], case.b_scale[e], None, torch.bfloat16)
         check(out[lo:hi], ref, what=f"config 5 {which} expert {e}")
