@@ -182,6 +182,56 @@ def _vendor_yardstick(runners, shapes, steps, stream):
         return {"library": "torch._scaled_mm", "error": f"{type(exc).__name__}: {exc}"[:200]}
 
 
+def _read_yardstick_us(runner, steps, stream, use_graph):
+    """A plain read (tg_diag_read: 16 bytes per lane, nothing else) of the same rotated weight copies the GEMM shape
+    streams, timed the same way (graph replay over whole passes of the copies): the floor of any kernel that has to read
+    those bytes once, on this GPU, in this run."""
+    from tilegym_amd import _lib
+    scratch = torch.zeros(4096, dtype=torch.int32, device=runner.b[0].device)
+    fn = lambda i: _lib.diag_read(runner.b[i % runner.copies], scratch)  # noqa: E731
+    for i in range(2):
+        fn(i)
+    torch.cuda.synchronize()
+    per_graph = runner.copies * max(1, -(-8 // runner.copies))
+    replays = max(1, steps // per_graph)
+    ms = _graph_ms(fn, per_graph, replays, stream) if use_graph else None
+    launches = per_graph * replays
+    if ms is None:
+        launches = steps
+        ms = _events_ms(fn, launches, stream)
+    return ms * 1e3 / launches
+
+
+def _eager_us(fn, n, stream):
+    """Per-call time of `n` back-to-back eager calls (no graph): the larger of the host cost of a call through the binding
+    and the kernel time."""
+    for i in range(3):
+        fn(i)
+    torch.cuda.synchronize()
+    return _events_ms(fn, n, stream) * 1e3 / n
+
+
+def _issue_yardstick(device, stream):
+    """tg_diag_mfma: the e4m3 MFMA rate on non-zero register operands with 0 / 4 / 6 scale-and-add FMAs behind every MFMA,
+    eight waves per compute unit on every compute unit: what the matrix pipe sustains here, and what is left of it when
+    it shares the VALU issue port with the block-scaled kernels' four FMAs per MFMA (plus a little more)."""
+    from tilegym_amd import _lib
+    props = torch.cuda.get_device_properties(device)
+    wgs = props.multi_processor_count
+    scratch = torch.empty(wgs * 512, dtype=torch.float32, device=device)
+    iters = 3000
+    out = {}
+    for fmas in (0, 4, 6):
+        fn = lambda i, fmas=fmas: _lib.diag_mfma(fmas, iters, wgs, scratch)  # noqa: E731
+        _ramp(fn, 60.0)
+        us = _events_ms(fn, 5, stream) * 1e3 / 5
+        flops = wgs * 8 * iters * 32 * 65536.0
+        out[f"mfma_plus_{fmas}_fma_tflops"] = round(flops / us * 1e-6, 1)
+    out["note"] = ("register-only loops of the library's tg_diag_mfma, 8 waves per CU, after 60 ms under their own load; "
+                   "a block-scaled K step needs 4 FMAs per MFMA plus its scale, address and conversion work")
+    return out
+
+
 class DenseRunner:
     """One dense problem with its operands replicated `copies` times for cache-cold rotation."""
 
@@ -216,6 +266,21 @@ class RaggedRunner:
     def __call__(self, i):
         j = i % self.copies
         self._lib.fp8_ragged_gemm(self.c, self.a[j], self.b[j], self.d.a_scale, self.d.b_scale, self.d.m_indptr)
+
+
+def _moe_decode_case(base, tokens):
+    """config 5's weights with `tokens` tokens routed over them (top-6 of softmax(N(0,1)) logits), expert-sorted."""
+    from tilegym_amd import workloads as W
+    E, _, K = base.b.shape
+    k = base.extra["top_k"]
+    _, ids = W.moe_routing(tokens, E, k, seed=tokens)
+    flat = ids.reshape(-1).long()
+    counts = torch.bincount(flat, minlength=E)
+    indptr = torch.zeros(E + 1, dtype=torch.int32)
+    indptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+    a = torch.randn(tokens * k, K, generator=torch.Generator().manual_seed(tokens))
+    qa, sa = W._quantize_1x128(a)
+    return W.GroupedCase(f"{base.name}_T{tokens}", qa, base.b, sa, base.b_scale, indptr, dict(base.extra))
 
 
 def _copies_for(nbytes):
@@ -386,7 +451,18 @@ def main():
             for M in W.DECODE_M:
                 case = W.DenseCase(f"c2_decode_{proj}_M{M}", big.a[:M].contiguous(), big.b, big.scale_a, big.scale_b, True, False)
                 r = DenseRunner(case, device, copies=_copies_for(case.algorithmic_bytes()))
-                shapes.append(measure_shape(r, max(args.steps, 64), args.warmup, stream, use_graph=not args.no_graph))
+                sh = measure_shape(r, max(args.steps, 64), args.warmup, stream, use_graph=not args.no_graph)
+                # the floor: a plain read of the same weight copies, same replay (once per projection is enough: M does
+                # not change the weights), and the eager per-call cost through the ctypes binding and through torch.ops
+                if M == W.DECODE_M[0]:
+                    read_us = _read_yardstick_us(r, max(args.steps, 64), stream, use_graph=not args.no_graph)
+                sh["read_yardstick_us"] = round(read_us, 3)
+                sh["eager_us"] = round(_eager_us(r, 200, stream), 2)
+                c0 = r.c[0]
+                op = torch.ops.tilegym_hip.fp8_gemm_out
+                sh["eager_us_torch_op"] = round(_eager_us(lambda i, r=r: op(c0, r.a[i % r.copies], r.b[i % r.copies], r.sa, r.sb,
+                                                                             False, True, 1.0, 0.0), 200, stream), 2)
+                shapes.append(sh)
                 del r
             torch.cuda.empty_cache()
         tot_b = sum(s["bytes"] for s in shapes)
@@ -397,6 +473,11 @@ def main():
         dec = {
             "metric": "FP8 GEMM decode GB/s (algorithmic bytes, cold cache)", "value": round(tot_b / tot_us * 1e-3, 1), "unit": "GB/s",
             "us_per_step": round(tot_us, 2),
+            "hbm_read_yardstick": {
+                "what": "tg_diag_read (plain 16-byte-per-lane read, no LDS, no MFMA) over the same rotated weight copies, same graph replay",
+                "us_M_le_16": round(sum(s["read_yardstick_us"] for s in small), 2),
+                "gemm_us_M_le_16": round(sum(s["us"] for s in small), 2),
+                "frac_hbm_of_the_plain_read": round(sum(s["bytes"] for s in small) / sum(s["read_yardstick_us"] for s in small) * 1e-3 / PEAK_HBM_GBS, 4)},
             "frac_hbm_M_le_16": round(sum(s["bytes"] for s in small) / sum(s["us"] for s in small) * 1e-3 / PEAK_HBM_GBS, 4),
             "roofline": {"bound": "hbm", "achieved": dom["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
                          "traffic": traffic, "traffic_source": traffic_note, "kernel": kernel_symbol(dom) + " per-tensor", "shape": dom["name"], "us_per_launch": dom["us"]},
@@ -421,6 +502,7 @@ def main():
                 del r
             torch.cuda.empty_cache()
         detail["block_scaled"] = shapes
+        out["issue_yardstick"] = _issue_yardstick(device, stream)
     if args.workload in ("moe", "all"):
         shapes = []
         for which in ("gate_up", "down"):
@@ -447,6 +529,49 @@ def main():
         detail["moe_layer"] = [{"name": f"c5_fused_moe_T{T}_E{w1.shape[0]}_top{ids.shape[1]}_H{H}_I{I}", "us": round(us, 2),
                                 "tflops": round(flops / us * 1e-6, 1), "frac_mfma": round(flops / us * 1e-6 / PEAK_FP8_TFLOPS, 4),
                                 "note": "five launches per call, outputs allocated by torch inside the timed region"}]
+        # MoE decode regime: T tokens on config 5's weights (the reference has a swap-AB variant for it,
+        # src/tilegym/suites/flashinfer/cutile/gemm/ragged_block_scaled_bmm.py:189-322).  Bytes = the touched experts'
+        # weights and scales + activations in and out; roofline HBM.  Ragged GEMMs (graph replay) and the whole layer.
+        dec_shapes = []
+        for T_dec in (1, 16, 64):
+            for which in ("gate_up", "down"):
+                gcase = _moe_decode_case(up if which == "gate_up" else down, T_dec)
+                sizes = (gcase.m_indptr[1:] - gcase.m_indptr[:-1])
+                touched = int((sizes > 0).sum())
+                E_, N_, K_ = gcase.b.shape
+                rows = int(gcase.m_indptr[-1])
+                nbytes = touched * (N_ * K_ + (N_ // 128) * (K_ // 128) * 4) + rows * (K_ + (K_ // 128) * 4 + N_ * 2)
+                # no cold-cache rotation over copies of the whole 369 MB weight set: only the touched experts' rows are read,
+                # and they differ per copy anyway (the rotation is over whole weight tensors)
+                r = RaggedRunner(gcase, device, copies=2 if touched * N_ * K_ > (128 << 20) else 4)
+                for i in range(3):
+                    r(i)
+                torch.cuda.synchronize()
+                cfg = _lib.last_config()
+                per_graph = r.copies * 4
+                ms = None if args.no_graph else _graph_ms(r, per_graph, max(1, 64 // per_graph), stream)
+                launches = per_graph * max(1, 64 // per_graph)
+                if ms is None:
+                    launches = 64
+                    ms = _events_ms(r, launches, stream)
+                us = ms * 1e3 / launches
+                dec_shapes.append({"name": f"c5_moe_decode_T{T_dec}_{which}", "kernel": cfg["KERNEL_NAME"], "block_m": cfg["BLOCK_M"],
+                                   "block_n": cfg["BLOCK_N"], "touched_experts": touched, "rows": rows, "us": round(us, 3),
+                                   "gbs": round(nbytes / us * 1e-3, 1), "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
+                                   "eager_us": round(_eager_us(r, 100, stream), 2)})
+                del r
+                torch.cuda.empty_cache()
+            ids_d, tw_d = W.moe_routing(T_dec, w1.shape[0], ids.shape[1], seed=T_dec)[1].to(device), W.moe_routing(T_dec, w1.shape[0], ids.shape[1], seed=T_dec)[0].to(device)
+            hid_d = torch.randn(T_dec, H, device=device).to(torch.bfloat16)
+            fn_d = lambda i: fused_moe(hid_d, w1, w2, tw_d, ids_d, w1_scale=s1, w2_scale=s2)  # noqa: E731
+            us = _eager_us(fn_d, 50, stream)
+            touched = int(torch.unique(ids_d).numel())
+            nbytes = touched * (w1[0].numel() + w2[0].numel() + (s1[0].numel() + s2[0].numel()) * 4) + T_dec * H * 4
+            dec_shapes.append({"name": f"c5_fused_moe_decode_T{T_dec}", "touched_experts": touched, "us": round(us, 2),
+                               "gbs": round(nbytes / us * 1e-3, 1), "frac_hbm": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4),
+                               "note": "eager calls of the whole layer (host cost included), weights hot in the memory-side cache"})
+        detail["moe_decode"] = dec_shapes
+        detail["moe_layer"][0]["eager_us"] = detail["moe_layer"][0]["us"]
         del hidden, w1, w2, s1, s2
         torch.cuda.empty_cache()
 

@@ -294,6 +294,20 @@ const char* tg_last_error(void);
 
 int32_t tg_abi_version(void);
 
+/*
+ * Yardsticks (no counterpart in the reference): kernels that compute nothing useful and exist so that the process that
+ * times the GEMMs can also time, on the same GPU and in the same run, what bounds them.
+ *
+ * tg_diag_read: a plain read of all bytes of x (16-byte aligned; 16 bytes per lane, non-temporal, 2048 workgroups):
+ *   the floor for any kernel that has to read those bytes once.  out: int32, >= 2048 elements (scratch).
+ * tg_diag_mfma: `workgroups` workgroups of eight waves issue iters x 32 e4m3 16x16x128 MFMAs per wave on non-zero register
+ *   operands (65536 FLOP per MFMA and wave), with `fmas` (0, 2, 4, 6 or 8) scale-and-add FMAs behind every MFMA: the
+ *   rate of the matrix pipe, and what is left of it when it shares the issue port with the block-scaled kernels' VALU
+ *   work.  out: f32, >= workgroups * 512 elements (scratch).
+ */
+int32_t tg_diag_read(const tg_tensor* x, const tg_tensor* out, int32_t device_id, uint64_t hip_stream);
+int32_t tg_diag_mfma(int32_t fmas, int32_t iters, int32_t workgroups, const tg_tensor* out, int32_t device_id, uint64_t hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

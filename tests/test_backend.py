@@ -136,3 +136,42 @@ def test_moe_align_has_no_cpu_path():
     ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]]) - 1
     with pytest.raises(RuntimeError, match="device tensors only"):
         moe_align_block_size(ids, 4, 4)  # no CPU path in the product
+
+
+def test_ops_are_registered_with_torchs_dispatcher():
+    """torch.ops.tilegym_hip.* exist after importing the package, carry schemas, infer output shapes without a GPU
+    (fake tensors), and refuse CPU tensors (there is no CPU implementation)."""
+    import torch
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    import tilegym_amd  # noqa: F401
+    from tilegym_amd import torch_ops
+
+    assert torch_ops.registered_ops() == [f"tilegym_hip::{n}" for n in torch_ops.OP_NAMES]
+    schema = str(torch.ops.tilegym_hip.fp8_gemm.default._schema)
+    assert "Tensor? scale_a" in schema and "ScalarType out_dtype" in schema and schema.endswith("-> Tensor")
+    assert "Tensor(a0!) c" in str(torch.ops.tilegym_hip.fp8_gemm_out.default._schema)
+    fp8 = torch.float8_e4m3fn
+    with FakeTensorMode():
+        a = torch.empty(8, 256, dtype=fp8, device="cuda")
+        b = torch.empty(512, 256, dtype=fp8, device="cuda")
+        c = torch.ops.tilegym_hip.fp8_gemm(a, b, None, None, False, True, 1.0, torch.bfloat16)
+        assert tuple(c.shape) == (8, 512) and c.dtype == torch.bfloat16
+        c = torch.ops.tilegym_hip.fp8_gemm(a.t(), b.t(), None, None, True, False, 1.0, torch.float32)
+        assert tuple(c.shape) == (8, 512) and c.dtype == torch.float32
+        w = torch.empty(4, 384, 256, dtype=fp8, device="cuda")
+        r = torch.ops.tilegym_hip.fp8_ragged_gemm(a, w, None, torch.empty(4, 3, 2, device="cuda"),
+                                                  torch.empty(5, dtype=torch.int32, device="cuda"), torch.bfloat16)
+        assert tuple(r.shape) == (8, 384)
+        q, s = torch.ops.tilegym_hip.fp8_quant_1x128(torch.empty(4, 3, 256, dtype=torch.bfloat16, device="cuda"))
+        assert q.dtype == fp8 and tuple(q.shape) == (4, 3, 256) and tuple(s.shape) == (4, 3, 2)
+    x = torch.zeros(8, 256).to(fp8)
+    import pytest
+    with pytest.raises(NotImplementedError):
+        torch.ops.tilegym_hip.fp8_gemm(x, x, None, None, False, True, 1.0, torch.bfloat16)
+
+
+def test_release_workspaces_empties_the_cache():
+    from tilegym_amd import _lib
+    _lib._workspaces[(0, 0, False)] = [__import__("torch").empty(1024, dtype=__import__("torch").uint8)]
+    assert _lib.release_workspaces() == 1024 and not _lib._workspaces

@@ -1487,6 +1487,35 @@ def _rows_stratified(M, per_tile, seed=0, tile=256):
     return torch.tensor(sorted(set(rows)))
 
 
+def test_ops_through_torchs_dispatcher(device):
+    """torch.ops.tilegym_hip.*: same bits as the direct calls; traceable by torch.compile (aot_eager: the graph is captured
+    through the fake implementations and run through the dispatcher)."""
+    g = _g(8)
+    M, N, K = 40, 520, 1024
+    a, b = fp8_randn((M, K), g).to(device), fp8_randn((N, K), g, 0.02).to(device)
+    sa, sb = torch.tensor([0.02], device=device), torch.tensor([0.01], device=device)
+    direct = matmul(a, b, trans_b=True, scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+    via = torch.ops.tilegym_hip.fp8_gemm(a, b, sa, sb, False, True, 1.0, torch.bfloat16)
+    assert torch.equal(direct, via)
+    c = torch.ones(M, N, dtype=torch.bfloat16, device=device)
+    torch.ops.tilegym_hip.fp8_gemm_out(c, a, b, sa, sb, False, True, 1.0, 1.0)
+    expect = gemm_alpha_beta(a, b, torch.ones(M, N, dtype=torch.bfloat16, device=device), alpha=0.02 * 0.01, beta=1.0)
+    check(c, expect.cpu(), what="fp8_gemm_out, beta = 1")
+
+    @torch.compile(backend="aot_eager", fullgraph=True)
+    def f(a, b, sa, sb):
+        return torch.ops.tilegym_hip.fp8_gemm(a, b, sa, sb, False, True, 1.0, torch.bfloat16).float() * 2
+
+    assert torch.equal(f(a, b, sa, sb), direct.float() * 2)
+    ra, rb, ras, rbs, ptr = _ragged_inputs([100, 0, 300], 256, 512, 3)
+    dev = [t.to(device) for t in (ra, rb, ras, rbs, ptr)]
+    assert torch.equal(torch.ops.tilegym_hip.fp8_ragged_gemm(*dev, torch.bfloat16), ragged_block_scaled_bmm(*dev, 300))
+    x = torch.randn(33, 384, generator=g).to(torch.bfloat16).to(device)
+    q, s = torch.ops.tilegym_hip.fp8_quant_1x128(x)
+    q2, s2 = _lib.fp8_quant_1x128(x, 0.0, False)
+    assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+
+
 def test_config1_full(device):
     for trans_b in (True, False):
         case = W.config1(trans_b=trans_b)

@@ -6,7 +6,8 @@ Import paths mirror the reference package (src/tilegym/__init__.py:34-49):
 ``tilegym_amd.suites.unsloth.ops.w8a8_block_fp8_matmul``,
 ``tilegym_amd.suites.flashinfer.ops.{ragged_block_scaled_bmm,gemm_alpha_beta}``,
 ``tilegym_amd.set_backend`` / ``is_backend_available``.  ``install_as_tilegym()`` makes the same
-modules importable under the name ``tilegym``.
+modules importable under the name ``tilegym``.  Importing the package also registers the GEMM entry points with
+torch's dispatcher as ``torch.ops.tilegym_hip.*`` (``tilegym_amd.torch_ops``).
 """
 
 from __future__ import annotations
@@ -18,6 +19,7 @@ __version__ = "0.1.0"
 from .backend import (dispatch, get_available_backends, get_current_backend,  # noqa: F401
                       get_registry_info, is_backend_available, register_impl, set_backend)
 from . import ops, suites  # noqa: F401,E402
+from . import torch_ops  # noqa: F401,E402  (registers torch.ops.tilegym_hip.*)
 
 
 def install_as_tilegym() -> None:

@@ -126,6 +126,10 @@ def load():
     L.tg_fp8_group_gemm.restype = ctypes.c_int32
     L.tg_fp8_group_gemm.argtypes = [PP, PP, PP, PP, PP, ctypes.c_int32, ctypes.c_int32, P, I32P, ctypes.c_int32,
                                     ctypes.c_int32, ctypes.c_uint64]
+    L.tg_diag_read.restype = ctypes.c_int32
+    L.tg_diag_read.argtypes = [P, P, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_diag_mfma.restype = ctypes.c_int32
+    L.tg_diag_mfma.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, P, ctypes.c_int32, ctypes.c_uint64]
     if L.tg_abi_version() != 1:
         raise RuntimeError(f"libtilegym_hip.so ABI version {L.tg_abi_version()} != 1")
     _lib = L
@@ -214,6 +218,15 @@ def workspace_for(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     ws = torch.empty(size, dtype=torch.uint8, device=device)
     held.append(ws)
     return ws
+
+
+def release_workspaces() -> int:
+    """Drop every scratch buffer held for the GEMM calls and return the number of bytes released.  Only for callers who
+    know that no HIP graph captured from these calls will be replayed again (a graph keeps writing to the buffer it was
+    captured with) and that no call is in flight; the next call allocates afresh."""
+    freed = sum(t.numel() for held in _workspaces.values() for t in held)
+    _workspaces.clear()
+    return freed
 
 
 def workspace_bytes(M: int, N: int, K: int, trans_b: bool, cfg, ncfg) -> int:
@@ -460,3 +473,17 @@ def fp8_group_gemm(cs, As, Bs, scales_a=None, scales_b=None, trans_b=True, kerne
     del k1, k2, k3, k4, k5
     check_rc(rc, "tg_fp8_group_gemm")
 
+
+
+# ---------------------------------------------------------------------------- yardsticks
+def diag_read(x: torch.Tensor, scratch: torch.Tensor) -> None:
+    """tg_diag_read: enqueue a plain read of all bytes of x (scratch: int32, >= 2048 elements)."""
+    rc = load().tg_diag_read(_ref(make_tensor_desc(x)), _ref(make_tensor_desc(scratch)), _device_index(x), _stream_handle(x))
+    check_rc(rc, "tg_diag_read")
+
+
+def diag_mfma(fmas: int, iters: int, workgroups: int, scratch: torch.Tensor) -> None:
+    """tg_diag_mfma: enqueue the MFMA (+ scale-and-add FMA) issue-rate kernel (scratch: f32, >= workgroups * 512)."""
+    rc = load().tg_diag_mfma(int(fmas), int(iters), int(workgroups), _ref(make_tensor_desc(scratch)), _device_index(scratch),
+                             _stream_handle(scratch))
+    check_rc(rc, "tg_diag_mfma")
