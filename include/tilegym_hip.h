@@ -68,7 +68,7 @@ enum {
                             * tiled 256x256 block-scaled kernels (dense and ragged): 1 = the persistent form (one workgroup per
                             * compute unit walks the tiles, three weight slabs in LDS, scales in registers); the ragged GEMM
                             * chooses it by itself for K <= 1536 */
-    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup; tiled 256x256 kernels: 8 = the generic eight-wave tile kernel (one workgroup per tile) instead of the persistent one */
+    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup, and with ROW_GROUPS = 4 (the wide form) 1 = one 1 KiB piece per wave in flight instead of two half pieces; tiled 256x256 kernels: 8 = the generic eight-wave tile kernel (one workgroup per tile) instead of the persistent one */
     TG_CFG_QUANT_BLOCK_N = 6, /* block-scaled tg_fp8_gemm: weight rows per scale (default 128) */
     TG_CFG_QUANT_BLOCK_K = 7, /* block-scaled tg_fp8_gemm: K elements per scale (default 128); blocks other than 128 x 128
                                * run on the fallback kernel (no MFMA): the reference's block_size=[bn, bk] argument,
@@ -298,14 +298,16 @@ int32_t tg_abi_version(void);
  * Yardsticks (no counterpart in the reference): kernels that compute nothing useful and exist so that the process that
  * times the GEMMs can also time, on the same GPU and in the same run, what bounds them.
  *
- * tg_diag_read: a plain read of all bytes of x (16-byte aligned; 16 bytes per lane, non-temporal, 2048 workgroups):
- *   the floor for any kernel that has to read those bytes once.  out: int32, >= 2048 elements (scratch).
+ * tg_diag_read: a plain read of all bytes of x (16-byte aligned; 16 bytes per lane, non-temporal, grid-stride over
+ *   `workgroups` workgroups of 256 threads with `loads_in_flight` (1, 2, 4 or 8) loads per lane in flight; 0 = 2048 and 4):
+ *   the floor for any kernel that has to read those bytes once.  out: int32, >= workgroups elements (scratch).
  * tg_diag_mfma: `workgroups` workgroups of eight waves issue iters x 32 e4m3 16x16x128 MFMAs per wave on non-zero register
  *   operands (65536 FLOP per MFMA and wave), with `fmas` (0, 2, 4, 6 or 8) scale-and-add FMAs behind every MFMA: the
  *   rate of the matrix pipe, and what is left of it when it shares the issue port with the block-scaled kernels' VALU
  *   work.  out: f32, >= workgroups * 512 elements (scratch).
  */
-int32_t tg_diag_read(const tg_tensor* x, const tg_tensor* out, int32_t device_id, uint64_t hip_stream);
+int32_t tg_diag_read(const tg_tensor* x, const tg_tensor* out, int32_t workgroups, int32_t loads_in_flight, int32_t device_id,
+                     uint64_t hip_stream);
 int32_t tg_diag_mfma(int32_t fmas, int32_t iters, int32_t workgroups, const tg_tensor* out, int32_t device_id, uint64_t hip_stream);
 
 #ifdef __cplusplus

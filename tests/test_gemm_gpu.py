@@ -391,43 +391,82 @@ def test_per_tensor_stream_eight_waves(device, M, N, K):
     check(out, ref, what=f"stream 8 waves M={M} N={N} K={K}")
 
 
-def test_stream_eight_waves_is_the_default_for_long_k_few_rows(device):
+def test_stream_eight_waves_is_the_default_for_long_k_one_or_two_rows(device):
     g = _g(5)
-    a, b = fp8_randn((4, 14336), g), fp8_randn((4096, 14336), g, 0.02)
+    a, b = fp8_randn((2, 14336), g), fp8_randn((4096, 14336), g, 0.02)
     ref = R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True)
     out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
     cfg = used("stream")
     assert cfg["WAVES"] == 8 and cfg["SPLIT_K"] == 1, cfg
-    check(out, ref, what="down projection, M=4")
+    check(out, ref, what="down projection, M=2")
 
 
+@pytest.mark.parametrize("M", [4, 16])
+def test_stream_wide_with_one_workgroup_per_compute_unit_is_the_default_for_long_k(device, M):
+    """4096 x 14336: 64 row blocks, four K splits = 256 workgroups."""
+    g = _g(6 + M)
+    a, b = fp8_randn((M, 14336), g), fp8_randn((4096, 14336), g, 0.02)
+    ref = R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
+    cfg = used("stream")
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == 4 and cfg["WAVES"] == 4, cfg
+    check(out, ref, what=f"down projection, M={M}")
+
+
+def _wide_form(K, in_flight):
+    """WAVES as tg_last_config reports it for the wide form: 4 = two half pieces per wave in flight (K % 512 == 0 only),
+    1 = one 1 KiB piece."""
+    return 4 if in_flight == 2 and K % 512 == 0 else 1
+
+
+@pytest.mark.parametrize("in_flight", [2, 1])
 @pytest.mark.parametrize("M", [1, 3, 8, 16])
 @pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 1), (264, 2064, 1), (128, 16384, 4), (72, 512, 1), (4096, 3072, 2)])
-def test_per_tensor_stream_wide(device, M, N, K, split):
+def test_per_tensor_stream_wide(device, M, N, K, split, in_flight):
     """64 weight rows per workgroup with the activation piece shared through LDS: ragged N (also inside a
-    workgroup's 64 rows), K tails inside a 1 KiB piece, split-K, every M up to 16."""
+    workgroup's 64 rows), K tails inside a 1 KiB piece, split-K, every M up to 16; both forms of the piece pipeline."""
     g = _g(M * 13 + N + K)
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
     sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
     ref = R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True)
+    kc = {"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split}
+    if in_flight == 1:
+        kc["WAVES"] = 1
     out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
-                 out_dtype=torch.bfloat16, kernel_configs={"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split})
+                 out_dtype=torch.bfloat16, kernel_configs=kc)
     cfg = used("stream")
-    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split and cfg["WAVES"] == _wide_form(K, in_flight), cfg
     check(out, ref, what=f"stream wide M={M} N={N} K={K} split={split}")
 
 
+@pytest.mark.parametrize("in_flight", [2, 1])
 @pytest.mark.parametrize("M", [1, 7, 16])
-@pytest.mark.parametrize("N,K,split", [(640, 1024, 1), (264, 2304, 1), (1152, 5120, 2), (128, 12288, 6)])
-def test_block_scaled_stream_wide(device, M, N, K, split):
+@pytest.mark.parametrize("N,K,split", [(640, 1024, 1), (264, 2304, 1), (1152, 5120, 2), (128, 12288, 6), (1000, 512, 1)])
+def test_block_scaled_stream_wide(device, M, N, K, split, in_flight):
     case = W.block_scaled_case(M, N, K, seed=M + N)
     ref = R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16)
     d = case.to(device)
-    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16,
-                                kernel_configs={"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split})
+    kc = {"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split}
+    if in_flight == 1:
+        kc["WAVES"] = 1
+    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs=kc)
     cfg = used("stream")
-    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split and cfg["WAVES"] == _wide_form(K, in_flight), cfg
     check(out, ref, what=f"block-scaled stream wide M={M} N={N} K={K} split={split}")
+
+
+def test_stream_wide_staggered_start_adds_the_same_products(device):
+    """The two-piece form starts every workgroup at another K piece and wraps around; with integer-valued operands the
+    sums are exact in fp32, so the rotated order must give the bits of the in-order form."""
+    g = _g(77)
+    M, N, K = 16, 1024, 8192
+    a = torch.randint(-2, 3, (M, K), generator=g).float().to(torch.float8_e4m3fn)
+    b = torch.randint(-2, 3, (N, K), generator=g).float().to(torch.float8_e4m3fn)
+    outs = []
+    for kc in ({"KERNEL": "stream", "ROW_GROUPS": 4}, {"KERNEL": "stream", "ROW_GROUPS": 4, "WAVES": 1}):
+        outs.append(matmul(a.to(device), b.to(device), trans_b=True, out_dtype=torch.float32, kernel_configs=kc))
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(outs[0].cpu(), a.float() @ b.float().t())
 
 
 def test_decode_auto_schedule_and_determinism(device):

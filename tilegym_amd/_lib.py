@@ -127,7 +127,7 @@ def load():
     L.tg_fp8_group_gemm.argtypes = [PP, PP, PP, PP, PP, ctypes.c_int32, ctypes.c_int32, P, I32P, ctypes.c_int32,
                                     ctypes.c_int32, ctypes.c_uint64]
     L.tg_diag_read.restype = ctypes.c_int32
-    L.tg_diag_read.argtypes = [P, P, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_diag_read.argtypes = [P, P, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     L.tg_diag_mfma.restype = ctypes.c_int32
     L.tg_diag_mfma.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, P, ctypes.c_int32, ctypes.c_uint64]
     if L.tg_abi_version() != 1:
@@ -476,9 +476,11 @@ def fp8_group_gemm(cs, As, Bs, scales_a=None, scales_b=None, trans_b=True, kerne
 
 
 # ---------------------------------------------------------------------------- yardsticks
-def diag_read(x: torch.Tensor, scratch: torch.Tensor) -> None:
-    """tg_diag_read: enqueue a plain read of all bytes of x (scratch: int32, >= 2048 elements)."""
-    rc = load().tg_diag_read(_ref(make_tensor_desc(x)), _ref(make_tensor_desc(scratch)), _device_index(x), _stream_handle(x))
+def diag_read(x: torch.Tensor, scratch: torch.Tensor, workgroups: int = 0, loads_in_flight: int = 0) -> None:
+    """tg_diag_read: enqueue a plain read of all bytes of x (scratch: int32, >= workgroups elements; 0 = the defaults,
+    2048 workgroups and 4 loads per lane in flight)."""
+    rc = load().tg_diag_read(_ref(make_tensor_desc(x)), _ref(make_tensor_desc(scratch)), int(workgroups), int(loads_in_flight),
+                             _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_diag_read")
 
 

@@ -11,14 +11,17 @@
 
 namespace {
 
+template <int UNROLL>
 __global__ void __launch_bounds__(256) diag_read_kernel(const v4i* __restrict__ src, int64_t n16, int* out) {
     const int64_t stride = (int64_t)gridDim.x * 256;
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     v4i acc = {0, 0, 0, 0};
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        const v4i a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + stride);
-        const v4i c = __builtin_nontemporal_load(src + i + 2 * stride), d = __builtin_nontemporal_load(src + i + 3 * stride);
-        acc ^= a ^ b ^ c ^ d;
+    for (; i + (UNROLL - 1) * stride < n16; i += UNROLL * stride) {
+        v4i t[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) t[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) acc ^= t[u];
     }
     for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
     const int v = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
@@ -64,7 +67,8 @@ __global__ void __launch_bounds__(512, 1) diag_mfma_kernel(float* out, int iters
 
 extern "C" {
 
-int32_t tg_diag_read(const tg_tensor* x, const tg_tensor* out, int32_t device_id, uint64_t hip_stream) {
+int32_t tg_diag_read(const tg_tensor* x, const tg_tensor* out, int32_t workgroups, int32_t loads_in_flight, int32_t device_id,
+                     uint64_t hip_stream) {
     if (!x || !out || !x->ptr || !out->ptr) return TG_ERR_NULL;
     int64_t bytes = 1;
     for (int i = 0; i < x->ndim; ++i) bytes *= x->shape[i];
@@ -76,12 +80,24 @@ int32_t tg_diag_read(const tg_tensor* x, const tg_tensor* out, int32_t device_id
     }
     int64_t slots = 1;
     for (int i = 0; i < out->ndim; ++i) slots *= out->shape[i];
-    if ((x->ptr & 15) != 0 || out->dtype != TG_I32 || slots < 2048) return TG_ERR_INVALID;
+    if (workgroups <= 0) workgroups = 2048;
+    if (loads_in_flight <= 0) loads_in_flight = 4;
+    if ((x->ptr & 15) != 0 || out->dtype != TG_I32 || workgroups > 65536 || slots < workgroups ||
+        (loads_in_flight != 1 && loads_in_flight != 2 && loads_in_flight != 4 && loads_in_flight != 8))
+        return TG_ERR_INVALID;
     int prev = -1;
     if (hipGetDevice(&prev) != hipSuccess) return TG_ERR_DEVICE;
     if (prev != device_id && hipSetDevice(device_id) != hipSuccess) return TG_ERR_DEVICE;
-    hipLaunchKernelGGL(diag_read_kernel, dim3(2048), dim3(256), 0, reinterpret_cast<hipStream_t>(hip_stream),
-                       reinterpret_cast<const v4i*>(x->ptr), bytes / 16, reinterpret_cast<int*>(out->ptr));
+    hipStream_t s = reinterpret_cast<hipStream_t>(hip_stream);
+    const v4i* src = reinterpret_cast<const v4i*>(x->ptr);
+    int* o = reinterpret_cast<int*>(out->ptr);
+    const dim3 g(workgroups), b(256);
+    switch (loads_in_flight) {
+        case 1: hipLaunchKernelGGL(diag_read_kernel<1>, g, b, 0, s, src, bytes / 16, o); break;
+        case 2: hipLaunchKernelGGL(diag_read_kernel<2>, g, b, 0, s, src, bytes / 16, o); break;
+        case 4: hipLaunchKernelGGL(diag_read_kernel<4>, g, b, 0, s, src, bytes / 16, o); break;
+        default: hipLaunchKernelGGL(diag_read_kernel<8>, g, b, 0, s, src, bytes / 16, o); break;
+    }
     const hipError_t e = hipGetLastError();
     if (prev != device_id) (void)hipSetDevice(prev);
     return e == hipSuccess ? TG_OK : TG_ERR_LAUNCH;

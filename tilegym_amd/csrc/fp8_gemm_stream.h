@@ -354,6 +354,161 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_kernel(const GemmPar
 #endif
 }
 
+// One float at a wave-uniform address: a scalar load.
+__device__ __forceinline__ float stream_uniform_f32(const float* p) {
+    return *(const __attribute__((address_space(4))) float*)(uintptr_t)p;
+}
+
+// The wide variant with two half-size buffers per wave: pieces of 512 bytes of K (four K steps), piece c+1 in flight
+// while piece c is multiplied, piece c+2 requested as soon as piece c's fragments are in registers.  A load instruction
+// covers two rows x 512 bytes (lanes 0 - 31 one row, lanes 32 - 63 the next).  Needs K % 512 == 0: every wave issues a
+// fixed number of loads per piece (eight for its weight rows, one or two for its share of the activation rows, one for
+// the activations' block scales), which the vmcnt waits count.
+// Workgroup b starts at piece b % (pieces) of its K range and wraps around: with all workgroups at the same K offset of
+// rows that lie a power of two apart (K = 4096, 8192) the requests of one moment fall on few memory channels
+// (28672 x 4096 at M = 1: 22.1 us in step, 20.6 us staggered; 8192 x 8192: 17.1 and 15.7).  The sum over K is the same
+// set of products added in a rotated order.
+// NW waves per workgroup (16 NW weight rows).  Measured with 4 .. 8: four is the fastest everywhere (28672 x 4096:
+// 22.1 / 26.0 / 29.3 / 24.6 / 25.4 us for 4 / 5 / 6 / 7 / 8 waves, although seven waves make exactly one workgroup per
+// compute unit), so only four is built.
+template <bool BLOCKSCALE, int NW>
+__global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_wide_db_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    static_assert(NW >= 4 && NW <= 8, "the eight activation loads of a piece are dealt over the waves, one or two each");
+    constexpr int PIECE = 512;                 // bytes of K per piece and row
+    constexpr int BUF = 16 * PIECE;            // 8 KiB
+    constexpr int SPC = PIECE / kKBlock;       // 4 K steps per piece
+    __shared__ __align__(1024) uint8_t sW[NW * 2 * BUF];
+    __shared__ __align__(1024) uint8_t sA[2 * BUF];
+    // block scales: every wave's own copy of the piece's 16 rows x 4 steps of activation scales, fetched by one more direct
+    // load of the piece so that it is counted by the same vmcnt wait.  (An ordinary load here would make the compiler wait
+    // for vmcnt(0) before its first use, i.e. for the next piece's loads as well: no overlap left.)
+    __shared__ __align__(16) float sS[BLOCKSCALE ? NW * 2 * 64 : 4];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int K = p.K, N = p.N, M = p.M;
+    const int n_base = blockIdx.x * (16 * NW) + wave * 16;
+    const int npieces = K / PIECE;
+    int c_begin = 0, c_end = npieces;
+    if (p.split_k > 1) {  // ksteps_per_split counts 1 KiB of K: two pieces
+        c_begin = blockIdx.y * p.ksteps_per_split * 2;
+        c_end = min(c_begin + p.ksteps_per_split * 2, npieces);
+    }
+    const v4i rsrc_b = make_rsrc(p.B), rsrc_a = make_rsrc(p.A);
+    const uint32_t my_lds = lds_address(sW) + wave * 2 * BUF, a_lds = lds_address(sA);
+    const uint8_t* my_buf = sW + wave * 2 * BUF;
+    const int rows_a = min(M, 16);
+
+    // lane l of a load: row 2i + l/32, LDS position l%32 of the row's 32 chunks, which holds logical chunk (l%32) ^ row
+    const int half = lane >> 5, pos = lane & 31;
+    uint32_t w_off[8], a_off[2];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = 2 * i + half;
+        w_off[i] = (uint32_t)min(n_base + r, N - 1) * (uint32_t)K + (uint32_t)((pos ^ r) << 4);
+    }
+    // the activation piece is eight loads of two rows: wave w issues load w and, if there is one, load w + NW
+    const bool two_a = wave + NW < 8;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int r = 2 * (wave + i * NW) + half;
+        a_off[i] = (uint32_t)min(r, rows_a - 1) * (uint32_t)K + (uint32_t)((pos ^ (r & 15)) << 4);  // (rows past M: a copy of the last row, never stored)
+    }
+    // lane l of the scale load: activation row l / 4, K step l % 4 of the piece
+    const bool has_as = BLOCKSCALE && p.As != nullptr;
+    const float* bs_ptr = BLOCKSCALE && p.Bs ? p.Bs + (int64_t)min(n_base / 128, p.nblocks - 1) * p.kblocks : nullptr;
+    const v4i rsrc_as = make_rsrc(p.As);
+    const uint32_t s_lds = lds_address(sS) + (BLOCKSCALE ? wave * 512 : 0);
+    const uint32_t as_off = ((uint32_t)min(lane >> 2, rows_a - 1) * (uint32_t)p.kblocks + (lane & 3)) * 4u;
+    auto issue = [&](int c, int buf) {
+        const int k0 = c * PIECE;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) direct_load_b128_nt(rsrc_b, my_lds + buf * BUF + i * 1024, w_off[i], k0);
+        direct_load_b128(rsrc_a, a_lds + buf * BUF + wave * 1024, a_off[0], k0);
+        if (two_a) direct_load_b128(rsrc_a, a_lds + buf * BUF + (wave + NW) * 1024, a_off[1], k0);
+        if constexpr (BLOCKSCALE)
+            if (has_as) direct_load_b32(rsrc_as, s_lds + buf * 256, as_off, c * (SPC * 4));
+    };
+
+    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+    // loads of one piece per wave: 8 + (1 or 2) + (block scales of the activations: 1)
+    const int per_piece = 9 + (two_a ? 1 : 0) + (has_as ? 1 : 0);
+    constexpr int kWaitBut9 = 0x0F70 | 9, kWaitBut10 = 0x0F70 | 10, kWaitBut11 = 0x0F70 | 11, kWaitAll = 0x0F70;
+    constexpr int kWaitLds = 0xC07F;
+    const int n_pieces = max(c_end - c_begin, 0);
+    const int rot = n_pieces > 0 ? (int)(blockIdx.x % (unsigned)n_pieces) : 0;  // staggered start, see above
+    auto piece = [&](int i) { const int c = c_begin + i + rot; return c >= c_end ? c - n_pieces : c; };
+    if (0 < n_pieces) issue(piece(0), 0);
+    if (1 < n_pieces) issue(piece(1), 1);
+    for (int it = 0; it < n_pieces; ++it) {
+        const int c = piece(it);
+        const int buf = it & 1;
+        float psc[BLOCKSCALE ? SPC : 1];
+        if constexpr (BLOCKSCALE) {  // the weight scales are the same in every lane: scalar loads, not counted by vmcnt
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) psc[s] = bs_ptr ? stream_uniform_f32(bs_ptr + c * SPC + s) : 1.0f;
+        }
+        // my loads of piece c have landed (those of piece c+1 may be in flight) ...
+        if (it + 1 >= n_pieces) __builtin_amdgcn_s_waitcnt(kWaitAll);
+        else if (per_piece == 9) __builtin_amdgcn_s_waitcnt(kWaitBut9);
+        else if (per_piece == 10) __builtin_amdgcn_s_waitcnt(kWaitBut10);
+        else __builtin_amdgcn_s_waitcnt(kWaitBut11);
+        __builtin_amdgcn_s_barrier();  // ... and so has every other wave's share of the activation piece
+        const uint8_t* wb = my_buf + buf * BUF + li * PIECE;
+        const uint8_t* ab = sA + buf * BUF + li * PIECE;
+        v8i wf[SPC], af[SPC];
+#pragma unroll
+        for (int s = 0; s < SPC; ++s) {
+            const int j0 = ((s * 8 + lg) ^ li) << 4, j1 = ((s * 8 + 4 + lg) ^ li) << 4;
+            wf[s] = join(*reinterpret_cast<const v4i*>(wb + j0), *reinterpret_cast<const v4i*>(wb + j1));
+            af[s] = join(*reinterpret_cast<const v4i*>(ab + j0), *reinterpret_cast<const v4i*>(ab + j1));
+        }
+        v4f as4 = v4f{1.f, 1.f, 1.f, 1.f};
+        if constexpr (BLOCKSCALE)
+            if (has_as) as4 = *reinterpret_cast<const v4f*>(sS + wave * 128 + buf * 64 + li * 4);
+        __builtin_amdgcn_s_waitcnt(kWaitLds);
+#pragma unroll
+        for (int s = 0; s < SPC; ++s) asm volatile("" : "+v"(wf[s]), "+v"(af[s]));
+        if constexpr (BLOCKSCALE) {
+            asm volatile("" : "+v"(as4));
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) psc[s] = as4[s] * psc[s];
+        }
+        __builtin_amdgcn_s_barrier();  // every wave holds its fragments: this buffer may be refilled
+        if (it + 2 < n_pieces) issue(piece(it + 2), buf);
+#pragma unroll
+        for (int s = 0; s < SPC; ++s) {
+            if constexpr (BLOCKSCALE) acc += mfma_e4m3(wf[s], af[s], v4f{0.f, 0.f, 0.f, 0.f}) * psc[s];
+            else acc = mfma_e4m3(wf[s], af[s], acc);
+        }
+    }
+    const bool vec_ok = p.vec_store != 0;
+    const int col = n_base + lg * 4, m = li;
+    const bool mine = m < M && col < N;
+    if (p.split_k > 1) {
+        if (mine) store4(p.partials + (int64_t)blockIdx.y * M * N, OUT_F32, m, col, N, N, acc, 0.f, vec_ok);
+        return;
+    }
+    if (!mine) return;
+    float scale = p.alpha;
+    if constexpr (!BLOCKSCALE) {
+        if (p.As) scale *= p.As[0];
+        if (p.Bs) scale *= p.Bs[0];
+    }
+    store4(p.C, p.out_type, m, col, N, p.ldc, acc * scale, p.beta, vec_ok);
+#endif
+}
+
+// grid_x = ceil(N / (16 * NW))
+template <bool BLOCKSCALE, int NW>
+inline hipError_t launch_stream_wide_db(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
+    if (p.K % 512 != 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((fp8_gemm_stream_wide_db_kernel<BLOCKSCALE, NW>), dim3(grid_x, grid_y, 1), dim3(64 * NW, 1, 1), 0, stream, p);
+    return hipGetLastError();
+}
+
 template <bool BLOCKSCALE>
 inline hipError_t launch_stream_wide(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
     hipLaunchKernelGGL(fp8_gemm_stream_wide_kernel<BLOCKSCALE>, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);

@@ -203,28 +203,42 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         s.waves = 4;
         const int64_t pieces = cdiv(K, 1024), wgs = cdiv(N, 16);
         s.split_k = 1;
-        // wide variant (64 weight rows per workgroup, activations shared through LDS): enough row
-        // blocks to fill the chip without a second pass; ROW_GROUPS = 4 asks for it explicitly
+        // wide variant (64 weight rows per workgroup, activations shared through LDS); ROW_GROUPS = 4 asks for it
         const int want_rg = cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS);
         const int64_t wide_wgs = cdiv(N, 64);
-        // without a second pass when the row blocks alone fill the chip; otherwise K is split over ~448
-        // workgroups, which pays a reduction pass (~3 us): measured to win from ~50 MB of weights on
-        // (4096 x 14336, 12288 x 5120, 5120 x 12288) and to lose on 4096 x 4096 and 6144 x 4096
-        int64_t wide_split = cdiv(448, wide_wgs);
+        // Split-K of the wide form.  A workgroup works through its pieces one memory round trip (~1.5 us) after the other
+        // and the reduction launch costs ~3 us: from 136 row blocks on no split pays (12288 x 5120: 12.2 us unsplit, 14.6
+        // with two splits; 10240 x 8192: 17.5 against 20.2); below, the workgroups should number about 256, one per
+        // compute unit (4096 x 14336, 64 row blocks, M = 1: 22.3 / 16.0 / 13.0 / 14.2 us with 1 / 2 / 4 / 7 splits;
+        // 6144 x 8192, 96 row blocks: 14.7 / 12.2 / 12.9 with 1 / 2 / 4) -- counts between one and two per compute unit
+        // leave some compute units with twice the work of the others.
+        int64_t wide_split = wide_wgs >= 136 ? 1 : 256 / wide_wgs;
         if (wide_split > pieces) wide_split = pieces;
-        const bool wide_auto = N >= 16384 || (N * K >= ((int64_t)48 << 20) && wide_wgs * wide_split >= 320);
-        // long K over few weight rows (at most ~one 16-row workgroup per compute unit): eight waves split K inside the
-        // workgroup, one launch, no partial sums (4096 x 14336: 12.4 / 14.3 us at M = 1 / 8 against 14.1 / 14.8 for the
-        // wide form with split-K and its reduction; at M = 16 every wave's own activation loads make it lose, 17.0 vs 15.4)
+        if (wide_split > 16) wide_split = 16;
+        if (wide_wgs >= 112 && pieces < 6) wide_split = 1;  // (8192 x 3072 at M = 16: 7.9 us unsplit, 9.5 with two splits)
+        // The wide form wins from 136 row blocks on (11008 x 4096 at M = 16: 11.1 us against 14.3 for the narrow form), and
+        // with fewer once the weight is large enough that the reduction launch is paid back: ~32 MB, ~24 MB at more than
+        // eight rows where every narrow workgroup's own activation loads weigh more (6144 x 4096 at M = 16: 9.3 against
+        // 9.6; 1536 x 24576: 10.4 - 11.9 against 13.5 - 19.4).  One to four rows over 96 - 135 row blocks stay narrow: its
+        // 384 - 540 workgroups fill the chip without a reduction (8192 x 8192 at M = 1: 13.6 against 15.7).
+        const bool wide_auto = N >= 16384 || (wide_wgs >= 136 && K >= 2048) ||
+                               (N * K >= ((int64_t)(M > 8 || pieces >= 12 ? 24 : 32) << 20) && wide_wgs * wide_split >= 176 && !(M <= 4 && wide_wgs >= 96));
+        // long K over one 16-row workgroup per compute unit, one or two activation rows: eight waves split K inside the
+        // workgroup, one launch, no partial sums (4096 x 14336: 12.6 us at M = 1 against 13.0 for the wide form with four
+        // splits; at M = 8 it is 14.4 against 13.4, and with fewer or more workgroups than compute units it loses by
+        // 20 - 35 %: 5120 x 12288, 2048 x 32768)
         const int want_waves = cfg_get(cfg, ncfg, TG_CFG_WAVES);
-        if (want_rg != 4 && want_split <= 1 && ((want_waves == 8 && M <= 16) || (want_waves < 0 && want_rg < 0 && M <= 8 && pieces >= 8 && wgs <= 320))) {
+        if (want_rg != 4 && want_split <= 1 && ((want_waves == 8 && M <= 16) || (want_waves < 0 && want_rg < 0 && M <= 2 && pieces >= 8 && wgs >= 224 && wgs <= 256))) {
             s.waves = 8;
             return s;
         }
         if (M <= 16 && (want_rg == 4 || (want_rg < 0 && wide_auto))) {
             s.row_groups = 4;
+            // K % 512 == 0: the form with two half pieces per wave in flight (reported as WAVES = 4); else, or with
+            // WAVES = 1, one 1 KiB piece per wave (reported as WAVES = 1)
+            s.waves = (K % 512) != 0 || want_waves == 1 ? 1 : 4;
             if (want_split > 1) s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, want_split);
-            else if (want_split < 0 && wide_wgs < 384 && wide_split > 1)
+            else if (want_split < 0 && wide_split > 1)
                 s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, (int)wide_split);
             return s;
         }
@@ -617,7 +631,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         // one workgroup, except for long K where they tie
         if (nbuf != 1 && nbuf != 2) nbuf = (per_wave >= 3 && s.mt == 1 && !block_scaled) ? 2 : 1;
         if (s.mt != 1 || s.waves == 8) nbuf = 1;
-        hipError_t e = s.row_groups == 4 ? tg::run_stream_wide(block_scaled, p, (int)cdiv(N, 64), s.split_k, stream)
+        hipError_t e = s.row_groups == 4 ? tg::run_stream_wide(block_scaled, p, s.split_k, stream, s.waves == 4)
                                          : tg::run_stream(s.mt, nbuf, s.waves, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "stream kernel launch failed: %s", hipGetErrorString(e));
         if (s.split_k > 1 && tg::run_splitk_reduce(p, block_scaled, stream) != hipSuccess)
