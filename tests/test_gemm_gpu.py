@@ -1443,7 +1443,7 @@ def test_config5_fused_experts_full_size(device):
     fused_moe; the oracle is evaluated on 24 sampled tokens (a token's output depends on its own row only)."""
     from tilegym_amd.ops import fused_moe
 
-    up, down = W.moe_grouped_case("gate_up"), W.moe_grouped_case("down")
+    up, down = _moe_base("gate_up"), _moe_base("down")
     ids, tw = up.extra["topk_ids"], up.extra["topk_weights"]
     T, H = ids.shape[0], up.b.shape[2]
     hidden = torch.randn(T, H, generator=_g(9)).to(torch.bfloat16)
@@ -1460,6 +1460,98 @@ def test_config5_fused_experts_full_size(device):
     again = fused_moe(hidden.to(device), up.b.to(device), down.b.to(device), tw.to(device), ids.to(device),
                       w1_scale=up.b_scale.to(device), w2_scale=down.b_scale.to(device))
     assert torch.equal(out, again)
+
+
+_MOE_BASE = {}
+
+
+def _moe_base(which):
+    """config 5's full-size grouped case, built once per test process (64 experts' weights are quantized on the CPU)."""
+    if which not in _MOE_BASE:
+        _MOE_BASE[which] = W.moe_grouped_case(which)
+    return _MOE_BASE[which]
+
+
+@pytest.mark.parametrize("T", [1, 16, 64])
+@pytest.mark.parametrize("which", ["gate_up", "down"])
+def test_config5_moe_decode_regime(device, which, T):
+    """The full-size expert weights (64 x 2816 x 2048 and 64 x 2048 x 1408) with 1 / 16 / 64 tokens routed over them: most
+    experts receive no row, the others one to a dozen.  Whole output against per-expert oracle GEMMs; rows of experts
+    that received nothing do not exist, and the result does not depend on what the output buffer held."""
+    case = W.moe_decode_case(_moe_base(which), T)
+    sizes = case.m_indptr[1:] - case.m_indptr[:-1]
+    assert int(case.m_indptr[-1]) == T * 6 and int((sizes == 0).sum()) >= 64 - 6 * T
+    d = case.to(device)
+    out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, int(sizes.max()))
+    for e in range(case.b.shape[0]):
+        lo, hi = int(case.m_indptr[e]), int(case.m_indptr[e + 1])
+        if hi > lo:
+            ref = R.ref_w8a8_block_fp8_matmul(case.a[lo:hi], case.b[e], case.a_scale[lo:hi], case.b_scale[e], None, torch.bfloat16)
+            check(out[lo:hi], ref, what=f"config 5 {which} T={T} expert {e}")
+    again = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, int(sizes.max()))
+    assert torch.equal(out, again)
+
+
+@pytest.mark.parametrize("T", [1, 16, 64])
+def test_config5_fused_experts_decode_regime(device, T):
+    """The whole layer at 1 / 16 / 64 tokens over the full-size weights, every token against the oracle."""
+    from tilegym_amd.ops import fused_moe
+
+    up, down = _moe_base("gate_up"), _moe_base("down")
+    tw, ids = W.moe_routing(T, up.b.shape[0], up.extra["top_k"], seed=T)
+    H = up.b.shape[2]
+    hidden = torch.randn(T, H, generator=_g(90 + T)).to(torch.bfloat16)
+    out = fused_moe(hidden.to(device), up.b.to(device), down.b.to(device), tw.to(device), ids.to(device),
+                    w1_scale=up.b_scale.to(device), w2_scale=down.b_scale.to(device))
+    assert out.shape == (T, H) and torch.isfinite(out.float()).all()
+    ref = R.ref_fused_experts_fp8(hidden, up.b, down.b, up.b_scale, down.b_scale, tw, ids)
+    ok, rep = R.compare_to_oracle(out, ref, RTOL, ATOL)
+    assert rep["matched"] >= 0.999 and rep["max_rel_to_sigma"] <= 0.1, rep
+
+
+def test_prepared_call_cache_follows_the_tensors(device):
+    """The binding keeps the prepared arguments of a call by the identity of its tensors.  The same objects again: same
+    result; an operand given new storage, a resized output, fresh outputs whose Python ids repeat, a dead weight whose id
+    is taken over by another tensor: each described afresh, never the stale pointer."""
+    from tilegym_amd import _lib
+
+    g = _g(123)
+    M, N, K = 8, 512, 1024
+    a1, a2 = fp8_randn((M, K), g).to(device), fp8_randn((M, K), g).to(device)
+    b1, b2 = fp8_randn((N, K), g, 0.02).to(device), fp8_randn((N, K), g, 0.02).to(device)
+    sa, sb = torch.tensor([0.5], device=device), torch.tensor([0.25], device=device)
+
+    def ref(a, b):
+        return ((a.float() * 0.5) @ (b.float() * 0.25).t()).to(torch.bfloat16)
+
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+    for _ in range(3):
+        _lib.fp8_gemm(c, a1, b1, sa, sb)
+        check(c, ref(a1, b1).cpu(), what="same objects")
+    a = a1.clone()
+    _lib.fp8_gemm(c, a, b1, sa, sb)
+    _lib.fp8_gemm(c, a, b1, sa, sb)
+    a.data = a2.clone()                      # same object, new storage
+    _lib.fp8_gemm(c, a, b1, sa, sb)
+    check(c, ref(a2, b1).cpu(), what="operand with new storage")
+    for i in range(6):                       # fresh outputs: ids repeat, every one must be written
+        out = torch.zeros(M, N, dtype=torch.bfloat16, device=device)
+        _lib.fp8_gemm(out, a1, b2 if i % 2 else b1, sa, sb)
+        check(out, ref(a1, b2 if i % 2 else b1).cpu(), what=f"fresh output {i}")
+        del out
+    w = b1.clone()
+    _lib.fp8_gemm(c, a1, w, sa, sb)
+    del w
+    w = b2.clone()                           # likely the dead weight's id and address
+    _lib.fp8_gemm(c, a1, w, sa, sb)
+    check(c, ref(a1, b2).cpu(), what="weight object replaced")
+    c2 = torch.empty(2 * M, N, dtype=torch.bfloat16, device=device)
+    a_big = torch.cat([a1, a2])
+    _lib.fp8_gemm(c2, a_big, b1, sa, sb)
+    check(c2, ref(a_big, b1).cpu(), what="other M")
+    _lib.release_call_caches()
+    _lib.fp8_gemm(c, a1, b1, sa, sb)
+    check(c, ref(a1, b1).cpu(), what="after release_call_caches")
 
 
 # ----------------------------------------------------------------------------- group_gemm (list form)
@@ -1628,7 +1720,7 @@ def test_config4_block_scaled_full(device, N, K):
 
 @pytest.mark.parametrize("which", ["gate_up", "down"])
 def test_config5_moe_grouped_full(device, which):
-    case = W.moe_grouped_case(which)
+    case = _moe_base(which)
     d = case.to(device)
     sizes = (case.m_indptr[1:] - case.m_indptr[:-1])
     assert int(case.m_indptr[-1]) == 4096 * 6 and sizes.min() != sizes.max()  # uneven experts

@@ -10,6 +10,7 @@ The descriptor / return-code conventions follow the reference's own C-ABI preced
 from __future__ import annotations
 
 import ctypes
+import weakref
 import os
 from typing import Dict, Optional, Sequence, Tuple
 
@@ -201,17 +202,27 @@ _workspaces: Dict[Tuple[int, int, bool], list] = {}
 _WS_MIN_BYTES = 1 << 20
 
 
-def workspace_for(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+def _raw_stream(index: int) -> int:
+    """Handle of torch's current stream on device `index` (what ``torch.cuda.current_stream(d).cuda_stream`` returns,
+    without building a Stream object: this is on the path of every call)."""
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
+def workspace_for(device: torch.device, nbytes: int, index: Optional[int] = None, stream: Optional[int] = None) -> Optional[torch.Tensor]:
     """Scratch buffer for the current stream of ``device`` (grown on demand, never freed).  One live buffer
     per (device, stream): calls on one stream are ordered, so they can share it.  Calls made while the
     stream is being captured get buffers of their own (allocated from the capturing graph's pool and kept
     alive here too), so eager calls and graph replays never share scratch memory."""
     if nbytes <= 0:
         return None
-    stream = torch.cuda.current_stream(device)
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    key = (index, stream.cuda_stream, bool(torch.cuda.is_current_stream_capturing()))
-    held = _workspaces.setdefault(key, [])
+    if index is None:
+        index = device.index if device.index is not None else torch.cuda.current_device()
+    if stream is None:
+        stream = _raw_stream(index)
+    key = (index, stream, torch.cuda.is_current_stream_capturing())
+    held = _workspaces.get(key)
+    if held is None:
+        held = _workspaces.setdefault(key, [])
     if held and held[-1].numel() >= nbytes:
         return held[-1]
     size = max(int(nbytes), _WS_MIN_BYTES, 2 * held[-1].numel() if held else 0)
@@ -241,13 +252,116 @@ def _device_index(t: torch.Tensor) -> int:
 
 
 def _stream_handle(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    index = t.device.index
+    return _raw_stream(index if index is not None else torch.cuda.current_device())
 
 
 # ---------------------------------------------------------------------------- raw calls
+# tg_fp8_gemm is called with the same weights, and often with the same activation and output buffers, over and over by
+# a decode loop, and building six descriptors, the cfg array and the workspace size costs more host time (~15 us) than a
+# small decode kernel runs (6 - 20 us).  Two caches take most of that away:
+#   * per call: the prepared arguments of a call whose five tensors are the very objects of an earlier call, keyed by
+#     their identities.  A hit is checked on every use (weak references to the tensors, their data pointers and shapes),
+#     so a tensor that was freed, resized or given new storage is described afresh; a key whose entry keeps failing that
+#     check (Python hands the address of a freed tensor object to the next one, so fresh outputs repeat ids) is marked
+#     volatile and no longer kept;
+#   * per weight: the descriptors of b and scale_b, keyed and checked the same way, for calls whose activations and
+#     outputs are fresh tensors every time; and the workspace size per (M, N, K, trans_b).
+_gemm_calls: Dict[tuple, object] = {}
+_weight_descs: Dict[int, tuple] = {}
+_ws_bytes: Dict[tuple, int] = {}
+_CACHE_MAX = 4096
+_VOLATILE = object()
+_default_cfg = None
+
+
+def _same(ref, ptr, t) -> bool:
+    return (t is None) if ref is None else (ref() is t and t.data_ptr() == ptr)
+
+
+def _weight_desc(t):
+    """Descriptor of a long-lived tensor (None -> None), cached by identity."""
+    if t is None:
+        return None
+    hit = _weight_descs.get(id(t))
+    if hit is not None and hit[0]() is t and t.data_ptr() == hit[1] and t.shape == hit[2]:
+        return hit[3]
+    d = make_tensor_desc(t)
+    if len(_weight_descs) >= _CACHE_MAX:
+        _weight_descs.clear()
+    _weight_descs[id(t)] = (weakref.ref(t), t.data_ptr(), t.shape, d)
+    return d
+
+
+def _gemm_constants(a, b, trans_a, trans_b, use_workspace):
+    global _default_cfg
+    if _default_cfg is None:
+        _default_cfg = make_cfg(None)
+    cfg, ncfg = _default_cfg
+    M = a.shape[1] if trans_a else a.shape[0]
+    K = a.shape[0] if trans_a else a.shape[1]
+    N = b.shape[0] if trans_b else b.shape[1]
+    ws_bytes = 0
+    if use_workspace and M > 0 and N > 0 and K > 0:
+        ws_bytes = _ws_bytes.get((M, N, K, trans_b))
+        if ws_bytes is None:
+            if len(_ws_bytes) >= _CACHE_MAX:
+                _ws_bytes.clear()
+            ws_bytes = _ws_bytes[(M, N, K, trans_b)] = workspace_bytes(M, N, K, trans_b, cfg, ncfg)
+    return cfg, ncfg, ws_bytes
+
+
+def _prepared_gemm(c, a, b, scale_a, scale_b, trans_a, trans_b, use_workspace):
+    """(argument references, cfg, ncfg, device index, workspace bytes, device, keep-alive) of a call without kernel_configs."""
+    key = (id(c), id(a), id(b), id(scale_a), id(scale_b), trans_a, trans_b, use_workspace)
+    hit = _gemm_calls.get(key)
+    if hit is not None and hit is not _VOLATILE:
+        refs, ptrs, shapes = hit[0], hit[1], hit[2]
+        if (_same(refs[0], ptrs[0], c) and _same(refs[1], ptrs[1], a) and _same(refs[2], ptrs[2], b)
+                and _same(refs[3], ptrs[3], scale_a) and _same(refs[4], ptrs[4], scale_b)
+                and c.shape == shapes[0] and a.shape == shapes[1] and b.shape == shapes[2]):
+            return hit[3]
+        hit[4][0] += 1
+    dev = _device_index(a)
+    cfg, ncfg, ws_bytes = _gemm_constants(a, b, trans_a, trans_b, use_workspace)
+    if hit is _VOLATILE or (hit is not None and hit[4][0] >= 2):
+        _gemm_calls[key] = _VOLATILE
+        descs = (make_tensor_desc(c), make_tensor_desc(a), _weight_desc(b), make_tensor_desc(scale_a), _weight_desc(scale_b))
+        return tuple(_ref(d) for d in descs), cfg, ncfg, dev, ws_bytes, a.device, descs
+    tensors = (c, a, b, scale_a, scale_b)
+    descs = (make_tensor_desc(c), make_tensor_desc(a), _weight_desc(b), make_tensor_desc(scale_a), _weight_desc(scale_b))
+    prepared = (tuple(_ref(d) for d in descs), cfg, ncfg, dev, ws_bytes, a.device, descs)
+    if len(_gemm_calls) >= _CACHE_MAX:
+        _gemm_calls.clear()
+    _gemm_calls[key] = (tuple(None if t is None else weakref.ref(t) for t in tensors),
+                        tuple(0 if t is None else t.data_ptr() for t in tensors), (c.shape, a.shape, b.shape), prepared,
+                        hit[4] if hit is not None else [0])
+    return prepared
+
+
+def release_call_caches() -> None:
+    """Forget every prepared call and cached descriptor (they hold no tensor alive; this only frees the bookkeeping)."""
+    _gemm_calls.clear()
+    _weight_descs.clear()
+    _ws_bytes.clear()
+
+
 def fp8_gemm(c, a, b, scale_a=None, scale_b=None, trans_a=False, trans_b=True, alpha=1.0, beta=0.0,
              kernel_configs=None, use_workspace=True) -> None:
-    L = load()
+    L = _lib if _lib is not None else load()
+    if kernel_configs is None:
+        refs, cfg, ncfg, dev, ws_bytes, device, _ = _prepared_gemm(c, a, b, scale_a, scale_b, bool(trans_a), bool(trans_b),
+                                                                   bool(use_workspace))
+        stream = _raw_stream(dev)
+        dws = None
+        if ws_bytes > 0:
+            dws = _ref(_weight_desc(workspace_for(device, ws_bytes, dev, stream)))
+        rc = L.tg_fp8_gemm(refs[0], refs[1], refs[2], refs[3], refs[4], 1 if trans_a else 0, 1 if trans_b else 0,
+                           alpha if type(alpha) is float else float(alpha), beta if type(beta) is float else float(beta),
+                           dws, cfg, ncfg, dev, stream)
+        if rc != 0:
+            check_rc(rc, "tg_fp8_gemm")
+        return
     dev = _device_index(a)
     cfg, ncfg = make_cfg(kernel_configs)
     M = a.shape[1] if trans_a else a.shape[0]

@@ -210,3 +210,20 @@ def moe_grouped_case(which: str = "gate_up", seed: int = 0, tokens: Optional[int
         qb[e], sb[e] = q, s
     return GroupedCase(f"c5_moe_{which}", qa, qb, sa, sb, indptr,
                        {"topk_ids": ids, "topk_weights": tw, "order": order, "top_k": k})
+
+
+def moe_decode_case(base: GroupedCase, tokens: int) -> GroupedCase:
+    """The weights of a full-size grouped case with only `tokens` tokens routed over them (top-k of softmax(N(0,1))
+    logits, seed = tokens), expert-sorted: the decode regime of the same layer, where most experts receive no row."""
+    E, _, K = base.b.shape
+    k = base.extra["top_k"]
+    tw, ids = moe_routing(tokens, E, k, seed=tokens)
+    flat = ids.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=E)
+    indptr = torch.zeros(E + 1, dtype=torch.int32)
+    indptr[1:] = torch.cumsum(counts, 0).to(torch.int32)
+    a = torch.randn(tokens * k, K, generator=_gen(tokens))
+    qa, sa = _quantize_1x128(a)
+    return GroupedCase(f"{base.name}_T{tokens}", qa, base.b, sa, base.b_scale, indptr,
+                       {"topk_ids": ids, "topk_weights": tw, "order": order, "top_k": k})
