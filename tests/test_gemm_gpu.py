@@ -455,6 +455,42 @@ def test_block_scaled_stream_wide(device, M, N, K, split, in_flight):
     check(out, ref, what=f"block-scaled stream wide M={M} N={N} K={K} split={split}")
 
 
+@pytest.mark.parametrize("M", [17, 24, 32])
+@pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 2), (72, 512, 1), (4096, 3072, 3)])
+def test_stream_wide_two_row_tiles(device, M, N, K, split):
+    """17 .. 32 activation rows: two tiles of 16 in the wide form's activation piece (per-tensor and block-scaled)."""
+    g = _g(M * 7 + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
+    kc = {"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split}
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs=kc)
+    cfg = used("stream")
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split and cfg["WAVES"] == 4, cfg
+    check(out, R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True), what=f"stream wide, two row tiles M={M} N={N} K={K}")
+    case = W.block_scaled_case(M, N, K, seed=M + N)
+    d = case.to(device)
+    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs=kc)
+    cfg = used("stream")
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == split, cfg
+    check(out, R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16),
+          what=f"block-scaled stream wide, two row tiles M={M} N={N} K={K}")
+
+
+def test_stream_wide_is_the_default_for_32_rows_over_a_large_weight(device):
+    """4096 x 14336 (58 MB) at M = 32 streams; 6144 x 4096 (25 MB) stays with the tile kernels."""
+    g = _g(41)
+    a, b = fp8_randn((32, 14336), g), fp8_randn((4096, 14336), g, 0.02)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
+    cfg = used("stream")
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == 4, cfg
+    check(out, R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True), what="down projection, M=32")
+    a, b = fp8_randn((32, 4096), g), fp8_randn((6144, 4096), g, 0.02)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
+    used("tiled")
+    check(out, R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True), what="qkv projection, M=32")
+
+
 def test_stream_wide_staggered_start_adds_the_same_products(device):
     """The two-piece form starts every workgroup at another K piece and wraps around; with integer-valued operands the
     sums are exact in fp32, so the rotated order must give the bits of the in-order form."""

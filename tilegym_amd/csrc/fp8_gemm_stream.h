@@ -362,28 +362,32 @@ __device__ __forceinline__ float stream_uniform_f32(const float* p) {
 // The wide variant with two half-size buffers per wave: pieces of 512 bytes of K (four K steps), piece c+1 in flight
 // while piece c is multiplied, piece c+2 requested as soon as piece c's fragments are in registers.  A load instruction
 // covers two rows x 512 bytes (lanes 0 - 31 one row, lanes 32 - 63 the next).  Needs K % 512 == 0: every wave issues a
-// fixed number of loads per piece (eight for its weight rows, one or two for its share of the activation rows, one for
-// the activations' block scales), which the vmcnt waits count.
+// fixed number of loads per piece (eight for its weight rows, two per 16 activation rows for its share of those, one per
+// 16 activation rows for their block scales), which the vmcnt waits count.
 // Workgroup b starts at piece b % (pieces) of its K range and wraps around: with all workgroups at the same K offset of
 // rows that lie a power of two apart (K = 4096, 8192) the requests of one moment fall on few memory channels
 // (28672 x 4096 at M = 1: 22.1 us in step, 20.6 us staggered; 8192 x 8192: 17.1 and 15.7).  The sum over K is the same
 // set of products added in a rotated order.
-// NW waves per workgroup (16 NW weight rows).  Measured with 4 .. 8: four is the fastest everywhere (28672 x 4096:
+// Four waves per workgroup (64 weight rows).  Measured with 4 .. 8: four is the fastest everywhere (28672 x 4096:
 // 22.1 / 26.0 / 29.3 / 24.6 / 25.4 us for 4 / 5 / 6 / 7 / 8 waves, although seven waves make exactly one workgroup per
-// compute unit), so only four is built.
-template <bool BLOCKSCALE, int NW>
-__global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_wide_db_kernel(const GemmParams p) {
+// compute unit).
+// MT tiles of 16 activation rows (M <= 16 MT): the activation piece in LDS grows to 16 MT rows, every wave multiplies
+// its weight fragments with all of them.  Built for MT = 1 and 2; MT = 4 works and is slower than the tile kernels.
+template <bool BLOCKSCALE, int MT>
+__global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    static_assert(NW >= 4 && NW <= 8, "the eight activation loads of a piece are dealt over the waves, one or two each");
+    constexpr int NW = 4;
     constexpr int PIECE = 512;                 // bytes of K per piece and row
-    constexpr int BUF = 16 * PIECE;            // 8 KiB
+    constexpr int BUF = 16 * PIECE;            // 8 KiB: a wave's 16 weight rows
+    constexpr int ABUF = MT * BUF;             // the activation piece
     constexpr int SPC = PIECE / kKBlock;       // 4 K steps per piece
+    constexpr int A_LOADS = 2 * MT;            // per wave and piece: the piece is 8 MT loads of two rows, dealt over four waves
     __shared__ __align__(1024) uint8_t sW[NW * 2 * BUF];
-    __shared__ __align__(1024) uint8_t sA[2 * BUF];
-    // block scales: every wave's own copy of the piece's 16 rows x 4 steps of activation scales, fetched by one more direct
-    // load of the piece so that it is counted by the same vmcnt wait.  (An ordinary load here would make the compiler wait
-    // for vmcnt(0) before its first use, i.e. for the next piece's loads as well: no overlap left.)
-    __shared__ __align__(16) float sS[BLOCKSCALE ? NW * 2 * 64 : 4];
+    __shared__ __align__(1024) uint8_t sA[2 * ABUF];
+    // block scales: every wave's own copy of the piece's 16 MT rows x 4 steps of activation scales, fetched by MT more direct
+    // loads of the piece so that they are counted by the same vmcnt wait.  (An ordinary load here would make the compiler
+    // wait for vmcnt(0) before its first use, i.e. for the next piece's loads as well: no overlap left.)
+    __shared__ __align__(16) float sS[BLOCKSCALE ? NW * 2 * MT * 64 : 4];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -399,44 +403,52 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_wide_db_kernel(const 
     const v4i rsrc_b = make_rsrc(p.B), rsrc_a = make_rsrc(p.A);
     const uint32_t my_lds = lds_address(sW) + wave * 2 * BUF, a_lds = lds_address(sA);
     const uint8_t* my_buf = sW + wave * 2 * BUF;
-    const int rows_a = min(M, 16);
+    const int rows_a = min(M, 16 * MT);
 
-    // lane l of a load: row 2i + l/32, LDS position l%32 of the row's 32 chunks, which holds logical chunk (l%32) ^ row
+    // lane l of a load: row 2i + l/32, LDS position l%32 of the row's 32 chunks, which holds logical chunk (l%32) ^ (row % 16)
     const int half = lane >> 5, pos = lane & 31;
-    uint32_t w_off[8], a_off[2];
+    uint32_t w_off[8], a_off[A_LOADS];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int r = 2 * i + half;
         w_off[i] = (uint32_t)min(n_base + r, N - 1) * (uint32_t)K + (uint32_t)((pos ^ r) << 4);
     }
-    // the activation piece is eight loads of two rows: wave w issues load w and, if there is one, load w + NW
-    const bool two_a = wave + NW < 8;
+    // wave w issues loads w, w + 4, w + 8, ... of the activation piece
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < A_LOADS; ++i) {
         const int r = 2 * (wave + i * NW) + half;
         a_off[i] = (uint32_t)min(r, rows_a - 1) * (uint32_t)K + (uint32_t)((pos ^ (r & 15)) << 4);  // (rows past M: a copy of the last row, never stored)
     }
-    // lane l of the scale load: activation row l / 4, K step l % 4 of the piece
+    // lane l of scale load mt: activation row 16 mt + l / 4, K step l % 4 of the piece
     const bool has_as = BLOCKSCALE && p.As != nullptr;
     const float* bs_ptr = BLOCKSCALE && p.Bs ? p.Bs + (int64_t)min(n_base / 128, p.nblocks - 1) * p.kblocks : nullptr;
     const v4i rsrc_as = make_rsrc(p.As);
-    const uint32_t s_lds = lds_address(sS) + (BLOCKSCALE ? wave * 512 : 0);
-    const uint32_t as_off = ((uint32_t)min(lane >> 2, rows_a - 1) * (uint32_t)p.kblocks + (lane & 3)) * 4u;
+    const uint32_t s_lds = lds_address(sS) + (BLOCKSCALE ? wave * (2 * MT * 256) : 0);
+    uint32_t as_off[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) as_off[mt] = ((uint32_t)min(mt * 16 + (lane >> 2), rows_a - 1) * (uint32_t)p.kblocks + (lane & 3)) * 4u;
     auto issue = [&](int c, int buf) {
         const int k0 = c * PIECE;
 #pragma unroll
         for (int i = 0; i < 8; ++i) direct_load_b128_nt(rsrc_b, my_lds + buf * BUF + i * 1024, w_off[i], k0);
-        direct_load_b128(rsrc_a, a_lds + buf * BUF + wave * 1024, a_off[0], k0);
-        if (two_a) direct_load_b128(rsrc_a, a_lds + buf * BUF + (wave + NW) * 1024, a_off[1], k0);
-        if constexpr (BLOCKSCALE)
-            if (has_as) direct_load_b32(rsrc_as, s_lds + buf * 256, as_off, c * (SPC * 4));
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) direct_load_b128(rsrc_a, a_lds + buf * ABUF + (wave + i * NW) * 1024, a_off[i], k0);
+        if constexpr (BLOCKSCALE) {
+            if (has_as) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) direct_load_b32(rsrc_as, s_lds + (buf * MT + mt) * 256, as_off[mt], c * (SPC * 4));
+            }
+        }
     };
 
-    v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
-    // loads of one piece per wave: 8 + (1 or 2) + (block scales of the activations: 1)
-    const int per_piece = 9 + (two_a ? 1 : 0) + (has_as ? 1 : 0);
-    constexpr int kWaitBut9 = 0x0F70 | 9, kWaitBut10 = 0x0F70 | 10, kWaitBut11 = 0x0F70 | 11, kWaitAll = 0x0F70;
-    constexpr int kWaitLds = 0xC07F;
+    v4f acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+    // all but the loads of one piece: 8 + 2 MT, and MT more with block scales of the activations
+    constexpr int kPlain = 8 + A_LOADS, kScaled = 8 + A_LOADS + MT;
+    constexpr int kWaitButPlain = 0x0F70 | (kPlain & 15) | ((kPlain >> 4) << 14);
+    constexpr int kWaitButScaled = 0x0F70 | (kScaled & 15) | ((kScaled >> 4) << 14);
+    constexpr int kWaitAll = 0x0F70, kWaitLds = 0xC07F;
     const int n_pieces = max(c_end - c_begin, 0);
     const int rot = n_pieces > 0 ? (int)(blockIdx.x % (unsigned)n_pieces) : 0;  // staggered start, see above
     auto piece = [&](int i) { const int c = c_begin + i + rot; return c >= c_end ? c - n_pieces : c; };
@@ -445,67 +457,78 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_wide_db_kernel(const 
     for (int it = 0; it < n_pieces; ++it) {
         const int c = piece(it);
         const int buf = it & 1;
-        float psc[BLOCKSCALE ? SPC : 1];
+        float bsc[BLOCKSCALE ? SPC : 1];
         if constexpr (BLOCKSCALE) {  // the weight scales are the same in every lane: scalar loads, not counted by vmcnt
 #pragma unroll
-            for (int s = 0; s < SPC; ++s) psc[s] = bs_ptr ? stream_uniform_f32(bs_ptr + c * SPC + s) : 1.0f;
+            for (int s = 0; s < SPC; ++s) bsc[s] = bs_ptr ? stream_uniform_f32(bs_ptr + c * SPC + s) : 1.0f;
         }
         // my loads of piece c have landed (those of piece c+1 may be in flight) ...
         if (it + 1 >= n_pieces) __builtin_amdgcn_s_waitcnt(kWaitAll);
-        else if (per_piece == 9) __builtin_amdgcn_s_waitcnt(kWaitBut9);
-        else if (per_piece == 10) __builtin_amdgcn_s_waitcnt(kWaitBut10);
-        else __builtin_amdgcn_s_waitcnt(kWaitBut11);
+        else if (has_as) __builtin_amdgcn_s_waitcnt(kWaitButScaled);
+        else __builtin_amdgcn_s_waitcnt(kWaitButPlain);
         __builtin_amdgcn_s_barrier();  // ... and so has every other wave's share of the activation piece
         const uint8_t* wb = my_buf + buf * BUF + li * PIECE;
-        const uint8_t* ab = sA + buf * BUF + li * PIECE;
-        v8i wf[SPC], af[SPC];
+        const uint8_t* ab = sA + buf * ABUF + li * PIECE;
+        v8i wf[SPC], af[MT][SPC];
 #pragma unroll
         for (int s = 0; s < SPC; ++s) {
             const int j0 = ((s * 8 + lg) ^ li) << 4, j1 = ((s * 8 + 4 + lg) ^ li) << 4;
             wf[s] = join(*reinterpret_cast<const v4i*>(wb + j0), *reinterpret_cast<const v4i*>(wb + j1));
-            af[s] = join(*reinterpret_cast<const v4i*>(ab + j0), *reinterpret_cast<const v4i*>(ab + j1));
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                af[mt][s] = join(*reinterpret_cast<const v4i*>(ab + mt * BUF + j0), *reinterpret_cast<const v4i*>(ab + mt * BUF + j1));
         }
-        v4f as4 = v4f{1.f, 1.f, 1.f, 1.f};
-        if constexpr (BLOCKSCALE)
-            if (has_as) as4 = *reinterpret_cast<const v4f*>(sS + wave * 128 + buf * 64 + li * 4);
+        v4f as4[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            as4[mt] = v4f{1.f, 1.f, 1.f, 1.f};
+            if constexpr (BLOCKSCALE)
+                if (has_as) as4[mt] = *reinterpret_cast<const v4f*>(sS + wave * (2 * MT * 64) + (buf * MT + mt) * 64 + li * 4);
+        }
         __builtin_amdgcn_s_waitcnt(kWaitLds);
 #pragma unroll
-        for (int s = 0; s < SPC; ++s) asm volatile("" : "+v"(wf[s]), "+v"(af[s]));
-        if constexpr (BLOCKSCALE) {
-            asm volatile("" : "+v"(as4));
+        for (int s = 0; s < SPC; ++s) {
+            asm volatile("" : "+v"(wf[s]));
 #pragma unroll
-            for (int s = 0; s < SPC; ++s) psc[s] = as4[s] * psc[s];
+            for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(af[mt][s]));
+        }
+        if constexpr (BLOCKSCALE) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(as4[mt]));
         }
         __builtin_amdgcn_s_barrier();  // every wave holds its fragments: this buffer may be refilled
         if (it + 2 < n_pieces) issue(piece(it + 2), buf);
 #pragma unroll
         for (int s = 0; s < SPC; ++s) {
-            if constexpr (BLOCKSCALE) acc += mfma_e4m3(wf[s], af[s], v4f{0.f, 0.f, 0.f, 0.f}) * psc[s];
-            else acc = mfma_e4m3(wf[s], af[s], acc);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                if constexpr (BLOCKSCALE) acc[mt] += mfma_e4m3(wf[s], af[mt][s], v4f{0.f, 0.f, 0.f, 0.f}) * (as4[mt][s] * bsc[s]);
+                else acc[mt] = mfma_e4m3(wf[s], af[mt][s], acc[mt]);
+            }
         }
     }
     const bool vec_ok = p.vec_store != 0;
-    const int col = n_base + lg * 4, m = li;
-    const bool mine = m < M && col < N;
-    if (p.split_k > 1) {
-        if (mine) store4(p.partials + (int64_t)blockIdx.y * M * N, OUT_F32, m, col, N, N, acc, 0.f, vec_ok);
-        return;
-    }
-    if (!mine) return;
+    const int col = n_base + lg * 4;
     float scale = p.alpha;
     if constexpr (!BLOCKSCALE) {
         if (p.As) scale *= p.As[0];
         if (p.Bs) scale *= p.Bs[0];
     }
-    store4(p.C, p.out_type, m, col, N, p.ldc, acc * scale, p.beta, vec_ok);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + li;
+        if (m >= M || col >= N) continue;
+        if (p.split_k > 1) store4(p.partials + (int64_t)blockIdx.y * M * N, OUT_F32, m, col, N, N, acc[mt], 0.f, vec_ok);
+        else store4(p.C, p.out_type, m, col, N, p.ldc, acc[mt] * scale, p.beta, vec_ok);
+    }
 #endif
 }
 
-// grid_x = ceil(N / (16 * NW))
-template <bool BLOCKSCALE, int NW>
+// grid_x = ceil(N / 64); M <= 16 MT
+template <bool BLOCKSCALE, int MT>
 inline hipError_t launch_stream_wide_db(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
-    if (p.K % 512 != 0) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((fp8_gemm_stream_wide_db_kernel<BLOCKSCALE, NW>), dim3(grid_x, grid_y, 1), dim3(64 * NW, 1, 1), 0, stream, p);
+    if (p.K % 512 != 0 || p.M > 16 * MT) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((fp8_gemm_stream_wide_db_kernel<BLOCKSCALE, MT>), dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
     return hipGetLastError();
 }
 

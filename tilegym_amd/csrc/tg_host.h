@@ -46,7 +46,8 @@ hipError_t run_skinny(int mt, int rg, int nw, bool blockscale, const GemmParams&
 hipError_t run_stream(int mt, int nbuf, int waves, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
 // 64 weight rows per workgroup, activation piece shared through LDS: M <= 16
 // two_buffers (needs K % 512 == 0): two 512-byte-per-row pieces per wave in flight, staggered over K; else one 1 KiB piece
-hipError_t run_stream_wide(bool blockscale, const GemmParams& p, int gy, hipStream_t s, bool two_buffers);
+// mt = 1, 2: tiles of 16 activation rows (M <= 16 mt; two only with two_buffers)
+hipError_t run_stream_wide(bool blockscale, const GemmParams& p, int gy, hipStream_t s, bool two_buffers, int mt);
 // C <- epilogue(sum_z partials[z]) for the split-K schedules (fixed z order: bit-reproducible)
 hipError_t run_splitk_reduce(const GemmParams& p, bool block_scaled, hipStream_t s);
 hipError_t run_generic(const GenericParams& p, hipStream_t s);
