@@ -364,6 +364,9 @@ def main():
     ap.add_argument("--workload", default="all", choices=["prefill", "decode", "block", "moe", "quant", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time microsecond kernels with plain launches")
+    ap.add_argument("--no-yardsticks", action="store_true",
+                    help="skip the plain-read and MFMA-issue yardsticks, the eager per-call costs and the MoE decode regime "
+                         "(profiler runs: only the GEMM launches of the workload)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run a plain elementwise copy of known size (256 MiB read + 256 MiB written, 3 launches): "
                          "the yardstick that hardware traffic counters are scaled by when this command runs under a profiler")
@@ -445,6 +448,10 @@ def main():
                 sh = measure_shape(r, max(args.steps, 64), args.warmup, stream, use_graph=not args.no_graph)
                 # the floor: a plain read of the same weight copies, same replay (once per projection is enough: M does
                 # not change the weights), and the eager per-call cost through the ctypes binding and through torch.ops
+                if args.no_yardsticks:
+                    shapes.append(sh)
+                    del r
+                    continue
                 if M == W.DECODE_M[0]:
                     read_us = _read_yardstick_us(r, max(args.steps, 64), stream, use_graph=not args.no_graph)
                 sh["read_yardstick_us"] = round(read_us, 3)
@@ -470,7 +477,7 @@ def main():
         dec = {
             "metric": "FP8 GEMM decode GB/s (algorithmic bytes, cold cache)", "value": round(tot_b / tot_us * 1e-3, 1), "unit": "GB/s",
             "us_per_step": round(tot_us, 2),
-            "hbm_read_yardstick": {
+            "hbm_read_yardstick": None if args.no_yardsticks else {
                 "what": "tg_diag_read (plain 16-byte-per-lane read, no LDS, no MFMA; the fastest of three launch shapes) over the same rotated weight copies, same graph replay",
                 "us_M_le_16": round(sum(s["read_yardstick_us"] for s in small), 2),
                 "gemm_us_M_le_16": round(sum(s["us"] for s in small), 2),
@@ -499,7 +506,8 @@ def main():
                 del r
             torch.cuda.empty_cache()
         detail["block_scaled"] = shapes
-        out["issue_yardstick"] = _issue_yardstick(device, stream)
+        if not args.no_yardsticks:
+            out["issue_yardstick"] = _issue_yardstick(device, stream)
     if args.workload in ("moe", "all"):
         shapes = []
         for which in ("gate_up", "down"):
@@ -530,7 +538,7 @@ def main():
         # src/tilegym/suites/flashinfer/cutile/gemm/ragged_block_scaled_bmm.py:189-322).  Bytes = the touched experts'
         # weights and scales + activations in and out; roofline HBM.  Ragged GEMMs (graph replay) and the whole layer.
         dec_shapes = []
-        for T_dec in (1, 16, 64):
+        for T_dec in (() if args.no_yardsticks else (1, 16, 64)):
             for which in ("gate_up", "down"):
                 gcase = W.moe_decode_case(up if which == "gate_up" else down, T_dec)
                 sizes = (gcase.m_indptr[1:] - gcase.m_indptr[:-1])
