@@ -185,6 +185,17 @@ def _as_scalar(s) -> torch.Tensor:
     return torch.tensor(float(s), dtype=torch.float32)
 
 
+def cast_output(acc: torch.Tensor, out_dtype, saturate: bool = True) -> torch.Tensor:
+    """The one stated rule for a GEMM's output cast.  16- and 32-bit types: torch's cast (nearest even).  e4m3: nearest
+    even after clamping to +-448 when ``saturate`` (what the HIP epilogues do); ``saturate=False`` is torch's plain cast,
+    which gives NaN from about 465 up -- what the reference gets when it casts an fp32 result with ``.to(float8_e4m3fn)``
+    (src/tilegym/ops/cutile/matmul.py:446).  The reference's own tests keep results in range, where the two agree; beyond
+    the range parity with the reference is unpinned."""
+    if out_dtype == FP8 and saturate:
+        return acc.float().clamp(-FP8_MAX, FP8_MAX).to(FP8)
+    return acc.to(out_dtype)
+
+
 def ref_gemm_per_tensor(a, b, scale_a=None, scale_b=None, trans_a=False, trans_b=False,
                         out_dtype=torch.bfloat16) -> torch.Tensor:
     """(dequant(a) @ dequant(b)) in fp32 -> out_dtype.
@@ -199,7 +210,7 @@ def ref_gemm_per_tensor(a, b, scale_a=None, scale_b=None, trans_a=False, trans_b
         bf = bf.t()
     af = af * _as_scalar(scale_a)
     bf = bf * _as_scalar(scale_b)
-    return (af @ bf).to(out_dtype)
+    return cast_output(af @ bf, out_dtype)
 
 
 def ref_gemm_alpha_beta(a, b, c, trans_a=False, trans_b=True, alpha=1.0, beta=0.0) -> torch.Tensor:
@@ -208,7 +219,7 @@ def ref_gemm_alpha_beta(a, b, c, trans_a=False, trans_b=True, alpha=1.0, beta=0.
     (the reference *test* multiplies in bf16, test_flashinfer_gemm_alpha_beta.py:17-22;
     the kernel accumulates in fp32, which is what is restated here)."""
     acc = ref_gemm_per_tensor(a, b, None, None, trans_a, trans_b, out_dtype=torch.float32)
-    return (alpha * acc + beta * c.float()).to(c.dtype)
+    return cast_output(alpha * acc + beta * c.float(), c.dtype)
 
 
 def expand_block_scales(As: torch.Tensor, Bs: torch.Tensor, N: int, K: int,
@@ -269,7 +280,7 @@ def ref_group_gemm(group_A: List[torch.Tensor], group_B: List[torch.Tensor], tra
         sb = None if scales_b is None else scales_b[i]
         od = out_dtype or A.dtype
         acc = ref_gemm_per_tensor(A, B, sa, sb, False, transpose_b, out_dtype=torch.float32)
-        outs.append(acc.to(od))
+        outs.append(cast_output(acc, od))
     return outs
 
 

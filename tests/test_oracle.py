@@ -405,3 +405,17 @@ def test_compare_to_oracle_flags_errors():
     assert not ok and rep["matched"] < 1.0
     nan = ref.clone(); nan[0, 0] = float("nan")
     assert not R.compare_to_oracle(nan, ref)[0]
+
+
+def test_output_cast_rule_saturates_e4m3_and_leaves_wider_types_to_torch():
+    x = torch.tensor([0.0, 1.0, -447.9, 448.0, 464.0, 465.0, 1e4, -1e9, float("inf")])
+    sat = R.cast_output(x, R.FP8).float()
+    assert torch.equal(sat, torch.tensor([0.0, 1.0, -448.0, 448.0, 448.0, 448.0, 448.0, -448.0, 448.0]))
+    plain = R.cast_output(x, R.FP8, saturate=False).float()
+    assert torch.equal(plain[:5], sat[:5]) and torch.isnan(plain[5:]).all()
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        assert torch.equal(R.cast_output(x[:7], dt), x[:7].to(dt))
+    # in range the two rules are the same function: all 256 codes round-trip
+    codes = torch.arange(256, dtype=torch.uint8).view(R.FP8).float()
+    finite = codes[~torch.isnan(codes)]
+    assert torch.equal(R.cast_output(finite, R.FP8).float(), finite)
