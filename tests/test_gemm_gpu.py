@@ -1508,6 +1508,37 @@ def _moe_base(which):
     return _MOE_BASE[which]
 
 
+@pytest.mark.parametrize("T,E,H,I,k,which", [(3, 8, 512, 256, 2, "gate_up"), (3, 8, 512, 384, 2, "down"), (40, 8, 1024, 128, 2, "gate_up"),
+                                             (5, 4, 2048, 1408, 2, "down"), (1, 6, 640, 128, 3, "down"), (2, 5, 128, 200, 1, "gate_up")])
+def test_ragged_stream_form(device, T, E, H, I, k, which):
+    """The streaming ragged kernel (one grid row per expert) forced at several row counts: empty experts, experts with more
+    than 16 rows (several passes over their weights), K of 1 .. 3 steps past a multiple of 512 (the short last piece), N that
+    is no multiple of 64, against per-expert oracle GEMMs; untouched rows of the output do not exist."""
+    base = W.moe_grouped_case(which, tokens=max(T, 8), experts=E, hidden=H, inter=I, top_k=k)
+    case = W.moe_decode_case(base, T)
+    d = case.to(device)
+    out = torch.full((case.a.shape[0], case.b.shape[1]), 7.0, dtype=torch.bfloat16, device=device)
+    _lib.fp8_ragged_gemm(out, d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, {"KERNEL": "stream"})
+    cfg = used("stream")
+    assert cfg["ROW_GROUPS"] == 4, cfg
+    for e in range(E):
+        lo, hi = int(case.m_indptr[e]), int(case.m_indptr[e + 1])
+        if hi > lo:
+            ref = R.ref_w8a8_block_fp8_matmul(case.a[lo:hi], case.b[e], case.a_scale[lo:hi], case.b_scale[e], None, torch.bfloat16)
+            check(out[lo:hi], ref, what=f"ragged stream {which} T={T} expert {e}")
+
+
+def test_ragged_stream_form_is_the_default_for_one_token(device):
+    case = W.moe_decode_case(_moe_base("down"), 1)
+    d = case.to(device)
+    out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, 1)
+    used("stream")
+    case = W.moe_decode_case(_moe_base("down"), 16)
+    d = case.to(device)
+    out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, 16)
+    used("tiled")
+
+
 @pytest.mark.parametrize("T", [1, 16, 64])
 @pytest.mark.parametrize("which", ["gate_up", "down"])
 def test_config5_moe_decode_regime(device, which, T):

@@ -532,6 +532,124 @@ inline hipError_t launch_stream_wide_db(const GemmParams& p, int grid_x, int gri
     return hipGetLastError();
 }
 
+// Ragged (expert-grouped) block-scaled GEMM for a handful of rows per expert: the decode regime of a MoE layer, where most
+// experts receive no row and the others one to a dozen.  The wide two-piece form above, one grid row per expert:
+// workgroup (x, e) streams weight rows 64 x .. 64 x + 63 of expert e once per 16 rows that m_indptr gives that expert and
+// leaves at once when it has none.  K % 128 == 0: the last piece of a K that is no multiple of 512 has one to three K
+// steps; its loads are redirected to the piece's first step where they would pass the end of a row, and its MFMAs stop
+// at the valid steps.  N * K < 2^31 per expert (32-bit offsets inside an expert's weight), total rows * K < 2^32.
+__global__ void __launch_bounds__(256) fp8_gemm_stream_ragged_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int NW = 4, PIECE = 512, BUF = 16 * PIECE, SPC = PIECE / kKBlock;
+    __shared__ __align__(1024) uint8_t sW[NW * 2 * BUF];
+    __shared__ __align__(1024) uint8_t sA[2 * BUF];
+    __shared__ __align__(16) float sS[NW * 2 * 64];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int K = p.K, N = p.N;
+    const int e = blockIdx.y;
+    const int row_lo = __builtin_amdgcn_readfirstlane(p.m_indptr[e]), row_hi = __builtin_amdgcn_readfirstlane(p.m_indptr[e + 1]);
+    if (row_hi <= row_lo) return;
+    const int n_base = blockIdx.x * (16 * NW) + wave * 16;
+    const int npieces = (K + PIECE - 1) / PIECE;
+    const int tail_steps = (K % PIECE) / kKBlock;  // 0: every piece is whole
+    const v4i rsrc_b = make_rsrc(p.B + (int64_t)e * N * K), rsrc_a = make_rsrc(p.A), rsrc_as = make_rsrc(p.As);
+    const float* bs_ptr = p.Bs + ((int64_t)e * p.nblocks + min(n_base / 128, p.nblocks - 1)) * p.kblocks;
+    const uint32_t my_lds = lds_address(sW) + wave * 2 * BUF, a_lds = lds_address(sA), s_lds = lds_address(sS) + wave * 512;
+    const uint8_t* my_buf = sW + wave * 2 * BUF;
+
+    // lane l of a load: row 2i + l/32, LDS position l%32 of the row's 32 chunks, which holds logical chunk (l%32) ^ row
+    const int half = lane >> 5, pos = lane & 31;
+    uint32_t w_off[8], w_tail[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = 2 * i + half, chunk = pos ^ r;
+        const uint32_t row = (uint32_t)min(n_base + r, N - 1) * (uint32_t)K;
+        w_off[i] = row + (uint32_t)(chunk << 4);
+        w_tail[i] = row + (uint32_t)((chunk < tail_steps * 8 ? chunk : 0) << 4);
+    }
+    constexpr int kWaitBut11 = 0x0F70 | 11, kWaitAll = 0x0F70, kWaitLds = 0xC07F;
+    const int rot = (int)(blockIdx.x % (unsigned)npieces);  // staggered start over K, as in the dense form
+    auto piece = [&](int i) { const int c = i + rot; return c >= npieces ? c - npieces : c; };
+    const bool vec_ok = p.vec_store != 0;
+    const int col = n_base + lg * 4;
+
+    for (int row0 = row_lo; row0 < row_hi; row0 += 16) {
+        const int rows_a = min(16, row_hi - row0);
+        uint32_t a_off[2], a_tail[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int r = 2 * (wave + i * NW) + half, chunk = pos ^ r;
+            const uint32_t row = (uint32_t)(row0 + min(r, rows_a - 1)) * (uint32_t)K;  // (rows past the tile: a copy of its last row, never stored)
+            a_off[i] = row + (uint32_t)(chunk << 4);
+            a_tail[i] = row + (uint32_t)((chunk < tail_steps * 8 ? chunk : 0) << 4);
+        }
+        // lane l of the scale load: activation row l / 4, K step l % 4 of the piece
+        const uint32_t as_row = (uint32_t)(row0 + min(lane >> 2, rows_a - 1)) * (uint32_t)p.kblocks;
+        const uint32_t as_off = (as_row + (lane & 3)) * 4u, as_tail = (as_row + ((lane & 3) < tail_steps ? (lane & 3) : 0)) * 4u;
+        auto issue = [&](int c, int buf) {
+            const int k0 = c * PIECE;
+            if (tail_steps != 0 && c == npieces - 1) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) direct_load_b128_nt(rsrc_b, my_lds + buf * BUF + i * 1024, w_tail[i], k0);
+                direct_load_b128(rsrc_a, a_lds + buf * BUF + wave * 1024, a_tail[0], k0);
+                direct_load_b128(rsrc_a, a_lds + buf * BUF + (wave + NW) * 1024, a_tail[1], k0);
+                direct_load_b32(rsrc_as, s_lds + buf * 256, as_tail, c * (SPC * 4));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) direct_load_b128_nt(rsrc_b, my_lds + buf * BUF + i * 1024, w_off[i], k0);
+                direct_load_b128(rsrc_a, a_lds + buf * BUF + wave * 1024, a_off[0], k0);
+                direct_load_b128(rsrc_a, a_lds + buf * BUF + (wave + NW) * 1024, a_off[1], k0);
+                direct_load_b32(rsrc_as, s_lds + buf * 256, as_off, c * (SPC * 4));
+            }
+        };
+        v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+        issue(piece(0), 0);
+        if (1 < npieces) issue(piece(1), 1);
+        for (int it = 0; it < npieces; ++it) {
+            const int c = piece(it);
+            const int buf = it & 1;
+            const int steps = (tail_steps != 0 && c == npieces - 1) ? tail_steps : SPC;
+            float bsc[SPC];
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) bsc[s] = stream_uniform_f32(bs_ptr + min(c * SPC + s, p.kblocks - 1));
+            if (it + 1 >= npieces) __builtin_amdgcn_s_waitcnt(kWaitAll);
+            else __builtin_amdgcn_s_waitcnt(kWaitBut11);
+            __builtin_amdgcn_s_barrier();
+            const uint8_t* wb = my_buf + buf * BUF + li * PIECE;
+            const uint8_t* ab = sA + buf * BUF + li * PIECE;
+            v8i wf[SPC], af[SPC];
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) {
+                const int j0 = ((s * 8 + lg) ^ li) << 4, j1 = ((s * 8 + 4 + lg) ^ li) << 4;
+                wf[s] = join(*reinterpret_cast<const v4i*>(wb + j0), *reinterpret_cast<const v4i*>(wb + j1));
+                af[s] = join(*reinterpret_cast<const v4i*>(ab + j0), *reinterpret_cast<const v4i*>(ab + j1));
+            }
+            v4f as4 = *reinterpret_cast<const v4f*>(sS + wave * 128 + buf * 64 + li * 4);
+            __builtin_amdgcn_s_waitcnt(kWaitLds);
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) asm volatile("" : "+v"(wf[s]), "+v"(af[s]));
+            asm volatile("" : "+v"(as4));
+            __builtin_amdgcn_s_barrier();  // every wave holds its fragments: this buffer may be refilled
+            if (it + 2 < npieces) issue(piece(it + 2), buf);
+#pragma unroll
+            for (int s = 0; s < SPC; ++s)
+                if (s < steps) acc += mfma_e4m3(wf[s], af[s], v4f{0.f, 0.f, 0.f, 0.f}) * (as4[s] * bsc[s]);
+        }
+        if (li < rows_a && col < N) store4(p.C, p.out_type, row0 + li, col, N, p.ldc, acc * p.alpha, p.beta, vec_ok);
+    }
+#endif
+}
+
+// one grid row per expert; needs both scale tensors, K % 128 == 0, N * K < 2^31
+inline hipError_t launch_stream_ragged(const GemmParams& p, hipStream_t stream) {
+    if (p.K % kKBlock != 0 || p.K <= 0 || !p.As || !p.Bs || !p.m_indptr || (int64_t)p.N * p.K >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fp8_gemm_stream_ragged_kernel, dim3((p.N + 63) / 64, p.E, 1), dim3(256, 1, 1), 0, stream, p);
+    return hipGetLastError();
+}
+
 template <bool BLOCKSCALE>
 inline hipError_t launch_stream_wide(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
     hipLaunchKernelGGL(fp8_gemm_stream_wide_kernel<BLOCKSCALE>, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);

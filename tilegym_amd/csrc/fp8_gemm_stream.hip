@@ -16,6 +16,8 @@ hipError_t run_stream(int mt, int nbuf, int waves, bool bs, const GemmParams& p,
     return hipErrorInvalidConfiguration;
 }
 
+hipError_t run_stream_ragged(const GemmParams& p, hipStream_t s) { return launch_stream_ragged(p, s); }
+
 hipError_t run_stream_wide(bool bs, const GemmParams& p, int gy, hipStream_t s, bool two_buffers, int mt) {
     const int gx = (p.N + 63) / 64;
     if (two_buffers && p.K % 512 == 0) {

@@ -82,6 +82,9 @@ inline bool aligned16(uint64_t p) { return (p & 15) == 0; }
 
 constexpr int64_t kOffsetLimit = (int64_t)1 << 31;  // kernels index operands with 32-bit byte offsets
 constexpr int kTargetWaves = 4096;                  // 16 waves on each of 256 CUs
+// ragged GEMM: up to this many rows in all take the streaming form (config 5's weights, 64 experts: 6 rows 11.9 / 7.1 us
+// against 16.6 / 12.5 for the 64x128 tiles; 24 rows 26.0 / 16.1 against 23.0 / 16.1; 96 rows 60.6 / 35.5 against 59.9 / 32.8)
+constexpr int64_t kRaggedStreamRows = 8;
 constexpr int64_t kBs256WeightLimit = ((int64_t)1 << 32) - 1;  // the persistent block-scaled kernel addresses all experts' weights with one 32-bit offset
 
 // Switches to the caller's device for the lifetime of a call.
@@ -794,6 +797,18 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
         q.rows = (int)total_m;
         remember(s);
         if (tg::run_generic(q, stream) != hipSuccess) return fail(TG_ERR_LAUNCH, "fallback kernel launch failed");
+        return TG_OK;
+    }
+    // One or two tokens' rows over many experts (the batch-1 decode step of a MoE layer): the streaming form, one grid row
+    // per expert, reads the weights of the experts that have rows once per 16 rows and nothing of the others.
+    // KERNEL = stream asks for it at any row count, KERNEL = tiled for the tile kernels below.
+    const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
+    const bool stream_ok = p.As && p.Bs && N * K < ((int64_t)1 << 31) && E <= 65535;
+    if (stream_ok && (want_kernel == 3 || (want_kernel < 0 && total_m <= kRaggedStreamRows))) {
+        s.kernel = 3; s.row_groups = 4; s.waves = 4;
+        remember(s);
+        const hipError_t e = tg::run_stream_ragged(p, stream);
+        if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "ragged stream kernel launch failed: %s", hipGetErrorString(e));
         return TG_OK;
     }
     int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
