@@ -414,14 +414,15 @@ def test_stream_wide_with_one_workgroup_per_compute_unit_is_the_default_for_long
 
 
 def _wide_form(K, in_flight):
-    """WAVES as tg_last_config reports it for the wide form: 4 = two half pieces per wave in flight (K % 512 == 0 only),
+    """WAVES as tg_last_config reports it for the wide form: 4 = two half pieces per wave in flight (K % 128 == 0 only),
     1 = one 1 KiB piece."""
-    return 4 if in_flight == 2 and K % 512 == 0 else 1
+    return 4 if in_flight == 2 and K % 128 == 0 else 1
 
 
 @pytest.mark.parametrize("in_flight", [2, 1])
 @pytest.mark.parametrize("M", [1, 3, 8, 16])
-@pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 1), (264, 2064, 1), (128, 16384, 4), (72, 512, 1), (4096, 3072, 2)])
+@pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 1), (264, 2064, 1), (128, 16384, 4), (72, 512, 1), (4096, 3072, 2),
+                                       (200, 1408, 1), (136, 128, 1), (520, 2432, 2), (264, 11008, 3)])
 def test_per_tensor_stream_wide(device, M, N, K, split, in_flight):
     """64 weight rows per workgroup with the activation piece shared through LDS: ragged N (also inside a
     workgroup's 64 rows), K tails inside a 1 KiB piece, split-K, every M up to 16; both forms of the piece pipeline."""
@@ -441,7 +442,8 @@ def test_per_tensor_stream_wide(device, M, N, K, split, in_flight):
 
 @pytest.mark.parametrize("in_flight", [2, 1])
 @pytest.mark.parametrize("M", [1, 7, 16])
-@pytest.mark.parametrize("N,K,split", [(640, 1024, 1), (264, 2304, 1), (1152, 5120, 2), (128, 12288, 6), (1000, 512, 1)])
+@pytest.mark.parametrize("N,K,split", [(640, 1024, 1), (264, 2304, 1), (1152, 5120, 2), (128, 12288, 6), (1000, 512, 1),
+                                       (200, 1408, 1), (136, 128, 1), (520, 2432, 2), (264, 11008, 3)])
 def test_block_scaled_stream_wide(device, M, N, K, split, in_flight):
     case = W.block_scaled_case(M, N, K, seed=M + N)
     ref = R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16)
@@ -456,7 +458,7 @@ def test_block_scaled_stream_wide(device, M, N, K, split, in_flight):
 
 
 @pytest.mark.parametrize("M", [17, 24, 32])
-@pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 2), (72, 512, 1), (4096, 3072, 3)])
+@pytest.mark.parametrize("N,K,split", [(1000, 1024, 1), (520, 4096, 2), (72, 512, 1), (4096, 3072, 3), (200, 1408, 1), (264, 2432, 2)])
 def test_stream_wide_two_row_tiles(device, M, N, K, split):
     """17 .. 32 activation rows: two tiles of 16 in the wide form's activation piece (per-tensor and block-scaled)."""
     g = _g(M * 7 + N + K)

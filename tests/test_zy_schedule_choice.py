@@ -23,6 +23,7 @@ SHAPES = [
     (18432, 3072, False), (3584, 18432, False), (9728, 5120, False), (6656, 6656, False), (14336, 4096, False),
     (1024, 49152, False), (12288, 2048, False), (5120, 5120, False), (8192, 3072, False), (2048, 14336, False),
     (4608, 12288, True), (11264, 6144, True), (7680, 7680, True), (2560, 20480, True), (14336, 4096, True),
+    (4096, 11008, False), (4096, 11008, True), (12288, 5248, True),   # K with a short last 512-byte piece
 ]
 
 

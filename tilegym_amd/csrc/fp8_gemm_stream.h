@@ -361,7 +361,8 @@ __device__ __forceinline__ float stream_uniform_f32(const float* p) {
 
 // The wide variant with two half-size buffers per wave: pieces of 512 bytes of K (four K steps), piece c+1 in flight
 // while piece c is multiplied, piece c+2 requested as soon as piece c's fragments are in registers.  A load instruction
-// covers two rows x 512 bytes (lanes 0 - 31 one row, lanes 32 - 63 the next).  Needs K % 512 == 0: every wave issues a
+// covers two rows x 512 bytes (lanes 0 - 31 one row, lanes 32 - 63 the next).  Needs K % 128 == 0 (a last piece of one to
+// three K steps is loaded with the same number of instructions and multiplied over its valid steps): every wave issues a
 // fixed number of loads per piece (eight for its weight rows, two per 16 activation rows for its share of those, one per
 // 16 activation rows for their block scales), which the vmcnt waits count.
 // Workgroup b starts at piece b % (pieces) of its K range and wraps around: with all workgroups at the same K offset of
@@ -394,7 +395,8 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
     const int li = lane & 15, lg = lane >> 4;
     const int K = p.K, N = p.N, M = p.M;
     const int n_base = blockIdx.x * (16 * NW) + wave * 16;
-    const int npieces = K / PIECE;
+    const int npieces = (K + PIECE - 1) / PIECE;
+    const int tail_steps = (K % PIECE) / kKBlock;  // K steps of the last piece when K is no multiple of 512 (0: every piece is whole)
     int c_begin = 0, c_end = npieces;
     if (p.split_k > 1) {  // ksteps_per_split counts 1 KiB of K: two pieces
         c_begin = blockIdx.y * p.ksteps_per_split * 2;
@@ -407,28 +409,51 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
 
     // lane l of a load: row 2i + l/32, LDS position l%32 of the row's 32 chunks, which holds logical chunk (l%32) ^ (row % 16)
     const int half = lane >> 5, pos = lane & 31;
-    uint32_t w_off[8], a_off[A_LOADS];
+    // (the *_tail offsets are those of the short last piece: a load that would pass the end of its row fetches the piece's
+    // first chunk again instead; the MFMAs of that piece stop at its valid steps)
+    uint32_t w_off[8], a_off[A_LOADS], w_tail[8], a_tail[A_LOADS];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int r = 2 * i + half;
-        w_off[i] = (uint32_t)min(n_base + r, N - 1) * (uint32_t)K + (uint32_t)((pos ^ r) << 4);
+        const int r = 2 * i + half, chunk = pos ^ r;
+        const uint32_t row = (uint32_t)min(n_base + r, N - 1) * (uint32_t)K;
+        w_off[i] = row + (uint32_t)(chunk << 4);
+        w_tail[i] = row + (uint32_t)((chunk < tail_steps * 8 ? chunk : 0) << 4);
     }
     // wave w issues loads w, w + 4, w + 8, ... of the activation piece
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
-        const int r = 2 * (wave + i * NW) + half;
-        a_off[i] = (uint32_t)min(r, rows_a - 1) * (uint32_t)K + (uint32_t)((pos ^ (r & 15)) << 4);  // (rows past M: a copy of the last row, never stored)
+        const int r = 2 * (wave + i * NW) + half, chunk = pos ^ (r & 15);
+        const uint32_t row = (uint32_t)min(r, rows_a - 1) * (uint32_t)K;  // (rows past M: a copy of the last row, never stored)
+        a_off[i] = row + (uint32_t)(chunk << 4);
+        a_tail[i] = row + (uint32_t)((chunk < tail_steps * 8 ? chunk : 0) << 4);
     }
     // lane l of scale load mt: activation row 16 mt + l / 4, K step l % 4 of the piece
     const bool has_as = BLOCKSCALE && p.As != nullptr;
     const float* bs_ptr = BLOCKSCALE && p.Bs ? p.Bs + (int64_t)min(n_base / 128, p.nblocks - 1) * p.kblocks : nullptr;
     const v4i rsrc_as = make_rsrc(p.As);
     const uint32_t s_lds = lds_address(sS) + (BLOCKSCALE ? wave * (2 * MT * 256) : 0);
-    uint32_t as_off[MT];
+    uint32_t as_off[MT], as_tail[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) as_off[mt] = ((uint32_t)min(mt * 16 + (lane >> 2), rows_a - 1) * (uint32_t)p.kblocks + (lane & 3)) * 4u;
+    for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t row = (uint32_t)min(mt * 16 + (lane >> 2), rows_a - 1) * (uint32_t)p.kblocks;
+        as_off[mt] = (row + (lane & 3)) * 4u;
+        as_tail[mt] = (row + ((lane & 3) < tail_steps ? (lane & 3) : 0)) * 4u;
+    }
     auto issue = [&](int c, int buf) {
         const int k0 = c * PIECE;
+        if (tail_steps != 0 && c == npieces - 1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) direct_load_b128_nt(rsrc_b, my_lds + buf * BUF + i * 1024, w_tail[i], k0);
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) direct_load_b128(rsrc_a, a_lds + buf * ABUF + (wave + i * NW) * 1024, a_tail[i], k0);
+            if constexpr (BLOCKSCALE) {
+                if (has_as) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) direct_load_b32(rsrc_as, s_lds + (buf * MT + mt) * 256, as_tail[mt], c * (SPC * 4));
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) direct_load_b128_nt(rsrc_b, my_lds + buf * BUF + i * 1024, w_off[i], k0);
 #pragma unroll
@@ -457,10 +482,11 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
     for (int it = 0; it < n_pieces; ++it) {
         const int c = piece(it);
         const int buf = it & 1;
+        const int steps = (tail_steps != 0 && c == npieces - 1) ? tail_steps : SPC;
         float bsc[BLOCKSCALE ? SPC : 1];
         if constexpr (BLOCKSCALE) {  // the weight scales are the same in every lane: scalar loads, not counted by vmcnt
 #pragma unroll
-            for (int s = 0; s < SPC; ++s) bsc[s] = bs_ptr ? stream_uniform_f32(bs_ptr + c * SPC + s) : 1.0f;
+            for (int s = 0; s < SPC; ++s) bsc[s] = bs_ptr ? stream_uniform_f32(bs_ptr + min(c * SPC + s, p.kblocks - 1)) : 1.0f;
         }
         // my loads of piece c have landed (those of piece c+1 may be in flight) ...
         if (it + 1 >= n_pieces) __builtin_amdgcn_s_waitcnt(kWaitAll);
@@ -502,6 +528,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
         for (int s = 0; s < SPC; ++s) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
+                if (s >= steps) continue;
                 if constexpr (BLOCKSCALE) acc[mt] += mfma_e4m3(wf[s], af[mt][s], v4f{0.f, 0.f, 0.f, 0.f}) * (as4[mt][s] * bsc[s]);
                 else acc[mt] = mfma_e4m3(wf[s], af[mt][s], acc[mt]);
             }
@@ -527,7 +554,7 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
 // grid_x = ceil(N / 64); M <= 16 MT
 template <bool BLOCKSCALE, int MT>
 inline hipError_t launch_stream_wide_db(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
-    if (p.K % 512 != 0 || p.M > 16 * MT) return hipErrorInvalidValue;
+    if (p.K % kKBlock != 0 || p.K <= 0 || p.M > 16 * MT) return hipErrorInvalidValue;
     hipLaunchKernelGGL((fp8_gemm_stream_wide_db_kernel<BLOCKSCALE, MT>), dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
     return hipGetLastError();
 }

@@ -20,7 +20,7 @@ hipError_t run_stream_ragged(const GemmParams& p, hipStream_t s) { return launch
 
 hipError_t run_stream_wide(bool bs, const GemmParams& p, int gy, hipStream_t s, bool two_buffers, int mt) {
     const int gx = (p.N + 63) / 64;
-    if (two_buffers && p.K % 512 == 0) {
+    if (two_buffers && p.K % 128 == 0) {
         if (mt == 1) return bs ? launch_stream_wide_db<true, 1>(p, gx, gy, s) : launch_stream_wide_db<false, 1>(p, gx, gy, s);
         if (mt == 2) return bs ? launch_stream_wide_db<true, 2>(p, gx, gy, s) : launch_stream_wide_db<false, 2>(p, gx, gy, s);
         return hipErrorInvalidConfiguration;

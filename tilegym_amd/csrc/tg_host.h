@@ -47,7 +47,7 @@ hipError_t run_stream(int mt, int nbuf, int waves, bool blockscale, const GemmPa
 // 64 weight rows per workgroup, activation piece shared through LDS: M <= 16
 // ragged block-scaled GEMM, a handful of rows per expert: one grid row per expert, weights streamed once per 16 rows
 hipError_t run_stream_ragged(const GemmParams& p, hipStream_t s);
-// two_buffers (needs K % 512 == 0): two 512-byte-per-row pieces per wave in flight, staggered over K; else one 1 KiB piece
+// two_buffers (needs K % 128 == 0): two 512-byte-per-row pieces per wave in flight, staggered over K; else one 1 KiB piece
 // mt = 1, 2: tiles of 16 activation rows (M <= 16 mt; two only with two_buffers)
 hipError_t run_stream_wide(bool blockscale, const GemmParams& p, int gy, hipStream_t s, bool two_buffers, int mt);
 // C <- epilogue(sum_z partials[z]) for the split-K schedules (fixed z order: bit-reproducible)

@@ -197,7 +197,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     if (want_kernel == 1 && tile_ok) skinny = false;
     if ((want_kernel == 2 || want_kernel == 3) && M <= 64) skinny = true;
     // 17 .. 32 rows over a large weight: candidates for the wide streaming form (decided below; otherwise the tile kernels)
-    const bool try_wide = !skinny && want_kernel < 0 && M <= 32 && (K % 512) == 0 && N * K >= ((int64_t)48 << 20);
+    const bool try_wide = !skinny && want_kernel < 0 && M <= 32 && (K % 128) == 0 && N * K >= ((int64_t)48 << 20);
     if (try_wide) skinny = true;
     if (!skinny && !tile_ok) return s;
     const int want_split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
@@ -242,12 +242,12 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // 12288 x 5120 block-scaled: 17.7 us against 24.3 for the 64 x 128 tile kernel with split-K; 4096 x 14336: 16.0
         // against 16.9; 6144 x 4096: 10.6 against 8.4).  Four tiles (to 64 rows) were measured too and lose everywhere
         // (28672 x 4096 at M = 64: 30.4 against 26.3): every wave reads the whole activation piece from LDS.
-        const bool wide_rows = M <= 16 || (M <= 32 && (K % 512) == 0);
+        const bool wide_rows = M <= 16 || (M <= 32 && (K % 128) == 0);
         if (wide_rows && (want_rg == 4 || (want_rg < 0 && wide_auto && (M <= 16 || N * K >= ((int64_t)48 << 20))))) {
             s.row_groups = 4;
-            // K % 512 == 0: the form with two half pieces per wave in flight (reported as WAVES = 4); else, or with
+            // K % 128 == 0: the form with two half pieces per wave in flight (reported as WAVES = 4); else, or with
             // WAVES = 1, one 1 KiB piece per wave (reported as WAVES = 1)
-            s.waves = (K % 512) != 0 || (want_waves == 1 && M <= 16) ? 1 : 4;
+            s.waves = (K % 128) != 0 || (want_waves == 1 && M <= 16) ? 1 : 4;
             if (want_split > 1) s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, want_split);
             else if (want_split < 0 && wide_split > 1)
                 s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, (int)wide_split);
