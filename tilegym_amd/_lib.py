@@ -10,6 +10,7 @@ The descriptor / return-code conventions follow the reference's own C-ABI preced
 from __future__ import annotations
 
 import ctypes
+import struct
 import weakref
 import os
 from typing import Dict, Optional, Sequence, Tuple
@@ -84,7 +85,7 @@ def load():
             f"libtilegym_hip.so not found at {path}; build it with "
             f"`python -m tilegym_amd.build` (hipcc, gfx950). There is no fallback implementation.")
     L = ctypes.CDLL(path)
-    P = ctypes.POINTER(TgTensor)
+    P = ctypes.c_void_p  # const tg_tensor*: a packed descriptor (bytes, see _desc) or ctypes.byref(TgTensor)
     I32P = ctypes.POINTER(ctypes.c_int32)
     L.tg_abi_version.restype = ctypes.c_int32
     L.tg_rc_message.restype = ctypes.c_char_p
@@ -123,7 +124,7 @@ def load():
     L.tg_silu_mul_quant_1x128.argtypes = [P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_moe_sum.restype = ctypes.c_int32
     L.tg_moe_sum.argtypes = [P, P, ctypes.c_int32, ctypes.c_uint64]
-    PP = ctypes.POINTER(P)
+    PP = ctypes.POINTER(ctypes.POINTER(TgTensor))
     L.tg_fp8_group_gemm.restype = ctypes.c_int32
     L.tg_fp8_group_gemm.argtypes = [PP, PP, PP, PP, PP, ctypes.c_int32, ctypes.c_int32, P, I32P, ctypes.c_int32,
                                     ctypes.c_int32, ctypes.c_uint64]
@@ -156,8 +157,36 @@ def make_tensor_desc(t: Optional[torch.Tensor]) -> Optional[TgTensor]:
     return d
 
 
-def _ref(d: Optional[TgTensor]):
-    return None if d is None else ctypes.byref(d)
+_DESC_PACK = struct.Struct("=Qi4x5q5qi4x")  # the bytes of a TgTensor: ptr, ndim, pad, shape[5], strides[5], dtype, pad
+assert _DESC_PACK.size == ctypes.sizeof(TgTensor)
+
+
+def _desc(t: Optional[torch.Tensor]) -> Optional[bytes]:
+    """make_tensor_desc for the call paths: the same descriptor as packed bytes (ctypes passes a bytes object to a
+    ``const tg_tensor*`` parameter as a pointer to its buffer), built in one struct.pack instead of a dozen ctypes field
+    assignments -- 0.75 us against 1.9 us, on calls that take up to nine of them."""
+    if t is None:
+        return None
+    code = _DTYPE_CODES.get(t.dtype)
+    if code is None:
+        raise TypeError(f"dtype {t.dtype} has no ABI code")
+    sh, st = t.shape, t.stride()
+    nd = len(sh)
+    if nd == 2:
+        return _DESC_PACK.pack(t.data_ptr(), 2, sh[0], sh[1], 0, 0, 0, st[0], st[1], 0, 0, 0, code)
+    if nd == 1:
+        return _DESC_PACK.pack(t.data_ptr(), 1, sh[0], 0, 0, 0, 0, st[0], 0, 0, 0, 0, code)
+    if nd == 3:
+        return _DESC_PACK.pack(t.data_ptr(), 3, sh[0], sh[1], sh[2], 0, 0, st[0], st[1], st[2], 0, 0, code)
+    if nd > TG_MAX_DIMS:
+        raise ValueError(f"tensor rank {nd} exceeds {TG_MAX_DIMS}")
+    pad = (0,) * (TG_MAX_DIMS - nd)
+    return _DESC_PACK.pack(t.data_ptr(), nd, *sh, *pad, *st, *pad, code)
+
+
+def _ref(d):
+    """What to hand to a ``const tg_tensor*`` parameter: packed bytes as they are, a TgTensor by reference."""
+    return d if d is None or isinstance(d, bytes) else ctypes.byref(d)
 
 
 def make_cfg(kernel_configs: Optional[dict]):
@@ -286,7 +315,7 @@ def _weight_desc(t):
     hit = _weight_descs.get(id(t))
     if hit is not None and hit[0]() is t and t.data_ptr() == hit[1] and t.shape == hit[2]:
         return hit[3]
-    d = make_tensor_desc(t)
+    d = _desc(t)
     if len(_weight_descs) >= _CACHE_MAX:
         _weight_descs.clear()
     _weight_descs[id(t)] = (weakref.ref(t), t.data_ptr(), t.shape, d)
@@ -326,10 +355,10 @@ def _prepared_gemm(c, a, b, scale_a, scale_b, trans_a, trans_b, use_workspace):
     cfg, ncfg, ws_bytes = _gemm_constants(a, b, trans_a, trans_b, use_workspace)
     if hit is _VOLATILE or (hit is not None and hit[4][0] >= 2):
         _gemm_calls[key] = _VOLATILE
-        descs = (make_tensor_desc(c), make_tensor_desc(a), _weight_desc(b), make_tensor_desc(scale_a), _weight_desc(scale_b))
+        descs = (_desc(c), _desc(a), _weight_desc(b), _desc(scale_a), _weight_desc(scale_b))
         return tuple(_ref(d) for d in descs), cfg, ncfg, dev, ws_bytes, a.device, descs
     tensors = (c, a, b, scale_a, scale_b)
-    descs = (make_tensor_desc(c), make_tensor_desc(a), _weight_desc(b), make_tensor_desc(scale_a), _weight_desc(scale_b))
+    descs = (_desc(c), _desc(a), _weight_desc(b), _desc(scale_a), _weight_desc(scale_b))
     prepared = (tuple(_ref(d) for d in descs), cfg, ncfg, dev, ws_bytes, a.device, descs)
     if len(_gemm_calls) >= _CACHE_MAX:
         _gemm_calls.clear()
@@ -370,8 +399,8 @@ def fp8_gemm(c, a, b, scale_a=None, scale_b=None, trans_a=False, trans_b=True, a
     ws = None
     if use_workspace and M > 0 and N > 0 and K > 0:
         ws = workspace_for(a.device, workspace_bytes(M, N, K, trans_b, cfg, ncfg))
-    dc, da, db = make_tensor_desc(c), make_tensor_desc(a), make_tensor_desc(b)
-    dsa, dsb, dws = make_tensor_desc(scale_a), make_tensor_desc(scale_b), make_tensor_desc(ws)
+    dc, da, db = _desc(c), _desc(a), _desc(b)
+    dsa, dsb, dws = _desc(scale_a), _desc(scale_b), _desc(ws)
     rc = L.tg_fp8_gemm(_ref(dc), _ref(da), _ref(db), _ref(dsa), _ref(dsb), int(bool(trans_a)),
                        int(bool(trans_b)), float(alpha), float(beta), _ref(dws), cfg, ncfg, dev,
                        _stream_handle(a))
@@ -388,8 +417,8 @@ def fp8_gemm_static_scratch(c, a, b, scale_a=None, scale_b=None, trans_a=False, 
     L = load()
     dev = _device_index(a)
     cfg, ncfg = make_cfg(kernel_configs)
-    dc, da, db = make_tensor_desc(c), make_tensor_desc(a), make_tensor_desc(b)
-    dsa, dsb = make_tensor_desc(scale_a), make_tensor_desc(scale_b)
+    dc, da, db = _desc(c), _desc(a), _desc(b)
+    dsa, dsb = _desc(scale_a), _desc(scale_b)
     rc = L.tg_fp8_gemm_static_scratch(_ref(dc), _ref(da), _ref(db), _ref(dsa), _ref(dsb), int(bool(trans_a)),
                                       int(bool(trans_b)), float(alpha), float(beta), cfg, ncfg, dev, _stream_handle(a))
     check_rc(rc, "tg_fp8_gemm_static_scratch")
@@ -399,7 +428,7 @@ def fp8_ragged_gemm(c, a, b, a_scale, b_scale, m_indptr, kernel_configs=None) ->
     L = load()
     dev = _device_index(a)
     cfg, ncfg = make_cfg(kernel_configs)
-    ds = [make_tensor_desc(t) for t in (c, a, b, a_scale, b_scale, m_indptr)]
+    ds = [_desc(t) for t in (c, a, b, a_scale, b_scale, m_indptr)]
     rc = L.tg_fp8_ragged_gemm(*[_ref(d) for d in ds], cfg, ncfg, dev, _stream_handle(a))
     check_rc(rc, "tg_fp8_ragged_gemm")
 
@@ -409,7 +438,7 @@ def fp8_moe_gemm(c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids, expe
     L = load()
     dev = _device_index(a)
     cfg, ncfg = make_cfg(kernel_configs)
-    ds = [make_tensor_desc(t) for t in (c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids,
+    ds = [_desc(t) for t in (c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids,
                                         expert_ids, num_tokens_post_padded)]
     rc = L.tg_fp8_moe_gemm(*[_ref(d) for d in ds], int(bool(mul_routed_weight)), int(top_k),
                            int(block_m), cfg, ncfg, dev, _stream_handle(a))
@@ -431,7 +460,7 @@ def fp8_moe_gemm_silu_quant(a, b, a_scale, b_scale, sorted_token_ids, expert_ids
     inter = b.shape[1] // 2
     q = torch.empty((num_valid, inter), dtype=torch.float8_e4m3fn, device=a.device)
     scales = torch.empty((num_valid, inter // 128), dtype=torch.float32, device=a.device)
-    ds = [make_tensor_desc(t) for t in (q, scales, a, b, a_scale, b_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)]
+    ds = [_desc(t) for t in (q, scales, a, b, a_scale, b_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)]
     rc = L.tg_fp8_moe_gemm_silu_quant(*[_ref(d) for d in ds], int(top_k), int(block_m), _DTYPE_CODES[act_dtype], dev,
                                       _stream_handle(a))
     check_rc(rc, "tg_fp8_moe_gemm_silu_quant")
@@ -456,9 +485,9 @@ def moe_align_block_size(topk_ids, block_size: int, num_experts: int):
     post = torch.empty(1, dtype=torch.int32, device=dev)
     cumsum = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
     mx = torch.empty(1, dtype=torch.int32, device=dev)
-    rc = L.tg_moe_align_block_size(_ref(make_tensor_desc(ids)), int(block_size), int(num_experts),
-                                   _ref(make_tensor_desc(sorted_ids)), _ref(make_tensor_desc(expert_ids)),
-                                   _ref(make_tensor_desc(post)), _ref(make_tensor_desc(cumsum)), _ref(make_tensor_desc(mx)),
+    rc = L.tg_moe_align_block_size(_ref(_desc(ids)), int(block_size), int(num_experts),
+                                   _ref(_desc(sorted_ids)), _ref(_desc(expert_ids)),
+                                   _ref(_desc(post)), _ref(_desc(cumsum)), _ref(_desc(mx)),
                                    _device_index(ids), _stream_handle(ids))
     check_rc(rc, "tg_moe_align_block_size")
     return sorted_ids, expert_ids, post, cumsum, mx
@@ -482,10 +511,10 @@ def moe_align_quant_1x128(topk_ids, block_size: int, num_experts: int, x: torch.
     mx = torch.empty(1, dtype=torch.int32, device=dev)
     q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
     scales = torch.empty(x.shape[:-1] + (x.shape[-1] // 128,), dtype=torch.float32, device=x.device)
-    rc = L.tg_moe_align_quant_1x128(_ref(make_tensor_desc(ids)), int(block_size), int(num_experts),
-                                    _ref(make_tensor_desc(sorted_ids)), _ref(make_tensor_desc(expert_ids)),
-                                    _ref(make_tensor_desc(post)), _ref(make_tensor_desc(cumsum)), _ref(make_tensor_desc(mx)),
-                                    _ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+    rc = L.tg_moe_align_quant_1x128(_ref(_desc(ids)), int(block_size), int(num_experts),
+                                    _ref(_desc(sorted_ids)), _ref(_desc(expert_ids)),
+                                    _ref(_desc(post)), _ref(_desc(cumsum)), _ref(_desc(mx)),
+                                    _ref(_desc(q)), _ref(_desc(scales)), _ref(_desc(x)),
                                     _device_index(ids), _stream_handle(ids))
     check_rc(rc, "tg_moe_align_quant_1x128")
     return sorted_ids, expert_ids, post, cumsum, mx, q, scales
@@ -500,7 +529,7 @@ def fp8_quant_1x128(x: torch.Tensor, eps: float = 0.0, flashinfer_rule: bool = F
         q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
     if scales is None:
         scales = torch.empty(x.shape[:-1] + (x.shape[-1] // 128,), dtype=torch.float32, device=x.device)
-    rc = L.tg_fp8_quant_1x128(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+    rc = L.tg_fp8_quant_1x128(_ref(_desc(q)), _ref(_desc(scales)), _ref(_desc(x)),
                               float(eps), 1 if flashinfer_rule else 0, _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_fp8_quant_1x128")
     return q, scales
@@ -517,7 +546,7 @@ def fp8_quant_group(x: torch.Tensor, group_size: int, eps: float, rule: int, sca
     q = torch.empty(x.shape, dtype=dst_dtype, device=x.device)
     if scales is None:
         scales = torch.empty(x.shape[:-1] + (x.shape[-1] // group_size,), dtype=torch.float32, device=x.device)
-    rc = L.tg_fp8_quant_group(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+    rc = L.tg_fp8_quant_group(_ref(_desc(q)), _ref(_desc(scales)), _ref(_desc(x)),
                               int(group_size), float(eps), int(rule), _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_fp8_quant_group")
     return q, scales
@@ -529,7 +558,7 @@ def fp8_weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, dtype:
     L = load()
     x, s = x.contiguous(), s.contiguous()
     y = out if out is not None else torch.empty(x.shape, dtype=dtype, device=x.device)
-    rc = L.tg_fp8_weight_dequant(_ref(make_tensor_desc(y)), _ref(make_tensor_desc(x)), _ref(make_tensor_desc(s)),
+    rc = L.tg_fp8_weight_dequant(_ref(_desc(y)), _ref(_desc(x)), _ref(_desc(s)),
                                  int(block_size), _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_fp8_weight_dequant")
     return y
@@ -542,7 +571,7 @@ def silu_mul_quant_1x128(x: torch.Tensor):
     inter = two_i // 2
     q = torch.empty(R, inter, dtype=torch.float8_e4m3fn, device=x.device)
     scales = torch.empty(R, -(-inter // 128), dtype=torch.float32, device=x.device)
-    rc = L.tg_silu_mul_quant_1x128(_ref(make_tensor_desc(q)), _ref(make_tensor_desc(scales)), _ref(make_tensor_desc(x)),
+    rc = L.tg_silu_mul_quant_1x128(_ref(_desc(q)), _ref(_desc(scales)), _ref(_desc(x)),
                                    _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_silu_mul_quant_1x128")
     return q, scales
@@ -551,7 +580,7 @@ def silu_mul_quant_1x128(x: torch.Tensor):
 def moe_sum(x: torch.Tensor, out: torch.Tensor) -> None:
     """out (T, H) <- sum over axis 1 of x (T, top_k, H) through tg_moe_sum."""
     L = load()
-    rc = L.tg_moe_sum(_ref(make_tensor_desc(out)), _ref(make_tensor_desc(x)), _device_index(x), _stream_handle(x))
+    rc = L.tg_moe_sum(_ref(_desc(out)), _ref(_desc(x)), _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_moe_sum")
 
 
@@ -583,7 +612,7 @@ def fp8_group_gemm(cs, As, Bs, scales_a=None, scales_b=None, trans_b=True, kerne
     rc = L.tg_fp8_group_gemm(ctypes.cast(c_arr, PP), ctypes.cast(a_arr, PP), ctypes.cast(b_arr, PP),
                              ctypes.cast(sa_arr, PP) if sa_arr is not None else None,
                              ctypes.cast(sb_arr, PP) if sb_arr is not None else None,
-                             n, 1 if trans_b else 0, _ref(make_tensor_desc(ws)), cfg, ncfg, dev, _stream_handle(As[0]))
+                             n, 1 if trans_b else 0, _ref(_desc(ws)), cfg, ncfg, dev, _stream_handle(As[0]))
     del k1, k2, k3, k4, k5
     check_rc(rc, "tg_fp8_group_gemm")
 
@@ -593,13 +622,13 @@ def fp8_group_gemm(cs, As, Bs, scales_a=None, scales_b=None, trans_b=True, kerne
 def diag_read(x: torch.Tensor, scratch: torch.Tensor, workgroups: int = 0, loads_in_flight: int = 0) -> None:
     """tg_diag_read: enqueue a plain read of all bytes of x (scratch: int32, >= workgroups elements; 0 = the defaults,
     2048 workgroups and 4 loads per lane in flight)."""
-    rc = load().tg_diag_read(_ref(make_tensor_desc(x)), _ref(make_tensor_desc(scratch)), int(workgroups), int(loads_in_flight),
+    rc = load().tg_diag_read(_ref(_desc(x)), _ref(_desc(scratch)), int(workgroups), int(loads_in_flight),
                              _device_index(x), _stream_handle(x))
     check_rc(rc, "tg_diag_read")
 
 
 def diag_mfma(fmas: int, iters: int, workgroups: int, scratch: torch.Tensor) -> None:
     """tg_diag_mfma: enqueue the MFMA (+ scale-and-add FMA) issue-rate kernel (scratch: f32, >= workgroups * 512)."""
-    rc = load().tg_diag_mfma(int(fmas), int(iters), int(workgroups), _ref(make_tensor_desc(scratch)), _device_index(scratch),
+    rc = load().tg_diag_mfma(int(fmas), int(iters), int(workgroups), _ref(_desc(scratch)), _device_index(scratch),
                              _stream_handle(scratch))
     check_rc(rc, "tg_diag_mfma")

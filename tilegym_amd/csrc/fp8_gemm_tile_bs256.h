@@ -414,7 +414,6 @@ __global__ void __launch_bounds__(512, 1) fp8_gemm_bs256_kernel(const GemmParams
         // (Every wave computes all four of its row groups, also those without a valid row: a copy of the loop per number
         // of row groups, as fp8_gemm_tile_kernel has, was built and gave wrong results in a way that was not understood;
         // the step keeps NTM as a parameter.)
-        constexpr int n_tm = TM;
         k_loop(std::integral_constant<int, TM>{});
 
         // ---------------------------------------------------------------- epilogue, straight from the accumulators
