@@ -282,6 +282,28 @@ int32_t tg_silu_mul_quant_1x128(const tg_tensor* q, const tg_tensor* scales, con
  */
 int32_t tg_moe_sum(const tg_tensor* out, const tg_tensor* x, int32_t device_id, uint64_t hip_stream);
 
+/*
+ * The FP8 MoE layer in one call: what src/tilegym/ops/moe_interface.py:116-322 (fused_experts_impl, use_fp8_w8a8) does
+ * for one chunk of tokens, as the four launches tg_moe_align_quant_1x128 -> tg_fp8_moe_gemm_silu_quant -> tg_fp8_moe_gemm
+ * (x routed weight) -> tg_moe_sum on the caller's stream, with every intermediate in `workspace`.  The results are the
+ * bits the four calls give one by one; what the call saves is the host time of four bindings and nine allocations, which at
+ * one to sixteen tokens is more than the kernels run.
+ *   hidden (T, H) bf16 / f16, H % 128 == 0; w1 (E, 2I, H), w2 (E, H, I) e4m3fn with w1_scale (E, 2I/128, H/128) and
+ *   w2_scale (E, H/128, ceil(I/128)) f32; topk_weights (T, k) f32 and topk_ids (T, k) int32 / int64, contiguous;
+ *   out (T, H) of hidden's type.  E <= 512, 2I % 256 == 0, block_m 128 or 256 (the alignment block = the row tile of the
+ *   grouped GEMMs); T * k + E * (block_m - 1) slots must fit int32.
+ *   workspace: uint8, 256-byte aligned, at least tg_fp8_fused_moe_workspace_bytes(...) bytes; it needs no initialisation
+ *   and holds nothing between calls.
+ * Layers outside these limits (more tokens than one chunk, other intermediate sizes, fp8 activations with their own scales)
+ * are run call by call, as the Python layer does.
+ */
+int64_t tg_fp8_fused_moe_workspace_bytes(int64_t tokens, int64_t top_k, int64_t experts, int64_t hidden, int64_t inter,
+                                         int32_t block_m);
+int32_t tg_fp8_fused_moe(const tg_tensor* out, const tg_tensor* hidden, const tg_tensor* w1, const tg_tensor* w2,
+                         const tg_tensor* w1_scale, const tg_tensor* w2_scale, const tg_tensor* topk_weights,
+                         const tg_tensor* topk_ids, const tg_tensor* workspace, int32_t block_m, int32_t device_id,
+                         uint64_t hip_stream);
+
 /* The schedule the most recent GEMM call on this host thread chose: fills out[0..n) with the
  * TG_CFG_* slots (kernel, BLOCK_M, BLOCK_N, SPLIT_K, ROW_GROUPS, WAVES).  Returns slots written. */
 int32_t tg_last_config(int32_t* out, int32_t n);

