@@ -165,6 +165,11 @@ def test_ops_are_registered_with_torchs_dispatcher():
         assert tuple(r.shape) == (8, 384)
         q, s = torch.ops.tilegym_hip.fp8_quant_1x128(torch.empty(4, 3, 256, dtype=torch.bfloat16, device="cuda"))
         assert q.dtype == fp8 and tuple(q.shape) == (4, 3, 256) and tuple(s.shape) == (4, 3, 2)
+        y = torch.ops.tilegym_hip.fp8_fused_moe(torch.empty(5, 256, dtype=torch.float16, device="cuda"), torch.empty(4, 512, 256, dtype=fp8, device="cuda"),
+                                                torch.empty(4, 256, 256, dtype=fp8, device="cuda"), torch.empty(4, 4, 2, device="cuda"),
+                                                torch.empty(4, 2, 2, device="cuda"), torch.empty(5, 2, device="cuda"),
+                                                torch.empty(5, 2, dtype=torch.int64, device="cuda"))
+        assert tuple(y.shape) == (5, 256) and y.dtype == torch.float16
     x = torch.zeros(8, 256).to(fp8)
     import pytest
     with pytest.raises(NotImplementedError):

@@ -1752,6 +1752,16 @@ def test_ops_through_torchs_dispatcher(device):
     q, s = torch.ops.tilegym_hip.fp8_quant_1x128(x)
     q2, s2 = _lib.fp8_quant_1x128(x, 0.0, False)
     assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+    from tilegym_amd.ops import fused_moe
+    T, H, I, E, k = 9, 256, 128, 4, 2
+    hidden = (torch.randn(T, H, generator=g) * 0.5).to(torch.bfloat16).to(device)
+    w1q, w1s = R.quantize_weight_128x128(torch.randn(E * 2 * I, H, generator=g) * 0.1)
+    w2q, w2s = R.quantize_weight_128x128(torch.randn(E * H, I, generator=g) * 0.1)
+    w1q, w1s = w1q.reshape(E, 2 * I, H).to(device), w1s.reshape(E, 2 * I // 128, H // 128).to(device)
+    w2q, w2s = w2q.reshape(E, H, I).to(device), w2s.reshape(E, H // 128, 1).to(device)
+    ids, tw = torch.randint(0, E, (T, k), generator=g).to(device), torch.softmax(torch.randn(T, k, generator=g), dim=-1).to(device)
+    assert torch.equal(torch.ops.tilegym_hip.fp8_fused_moe(hidden, w1q, w2q, w1s, w2s, tw, ids),
+                       fused_moe(hidden, w1q, w2q, tw, ids, w1_scale=w1s, w2_scale=w2s))
 
 
 def test_config1_full(device):

@@ -13,6 +13,8 @@ They are registered for device tensors only: with CPU tensors the dispatcher rai
     fp8_moe_gemm_out(c, a, b, a_scale, b_scale, topk_weights, sorted_token_ids, expert_ids,
                      num_tokens_post_padded, mul_routed_weight, top_k, block_m) -> ()  tg_fp8_moe_gemm
     fp8_quant_1x128(x) -> (q, scales)                                                   tg_fp8_quant_1x128
+    fp8_fused_moe(hidden, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids) -> out   the FP8 MoE layer (tg_fp8_fused_moe
+                                                                                        when it fits one chunk)
 """
 
 from __future__ import annotations
@@ -24,7 +26,7 @@ import torch
 from . import _lib
 
 NAMESPACE = "tilegym_hip"
-OP_NAMES = ("fp8_gemm", "fp8_gemm_out", "fp8_ragged_gemm", "fp8_moe_gemm_out", "fp8_quant_1x128")
+OP_NAMES = ("fp8_gemm", "fp8_gemm_out", "fp8_ragged_gemm", "fp8_moe_gemm_out", "fp8_quant_1x128", "fp8_fused_moe")
 
 
 def _mnk(a: torch.Tensor, b: torch.Tensor, trans_a: bool, trans_b: bool) -> Tuple[int, int, int]:
@@ -108,6 +110,21 @@ def _(x):
     if x.shape[-1] % 128 != 0:
         raise ValueError("the last dimension must be a multiple of 128")
     return x.new_empty(x.shape, dtype=torch.float8_e4m3fn), x.new_empty(x.shape[:-1] + (x.shape[-1] // 128,), dtype=torch.float32)
+
+
+@torch.library.custom_op(f"{NAMESPACE}::fp8_fused_moe", mutates_args=(), device_types="cuda")
+def fp8_fused_moe(hidden: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w1_scale: torch.Tensor, w2_scale: torch.Tensor,
+                  topk_weights: torch.Tensor, topk_ids: torch.Tensor) -> torch.Tensor:
+    from .ops.moe_interface import fused_experts_impl
+    return fused_experts_impl(hidden, w1, w2, topk_weights, topk_ids, inplace=False, use_fp8_w8a8=True, w1_scale=w1_scale,
+                              w2_scale=w2_scale)
+
+
+@fp8_fused_moe.register_fake
+def _(hidden, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids):
+    if hidden.dim() != 2 or w1.dim() != 3 or w2.dim() != 3 or w1.shape[2] != hidden.shape[1] or w2.shape[1] != hidden.shape[1]:
+        raise ValueError("fp8_fused_moe expects hidden (T, H), w1 (E, 2I, H) and w2 (E, H, I)")
+    return hidden.new_empty(hidden.shape, dtype=torch.bfloat16 if hidden.dtype == torch.bfloat16 else torch.float16)
 
 
 def registered_ops():
