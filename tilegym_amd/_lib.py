@@ -307,7 +307,7 @@ def _stream_handle(t: torch.Tensor) -> int:
 # a decode loop, and building six descriptors, the cfg array and the workspace size costs more host time (~15 us) than a
 # small decode kernel runs (6 - 20 us).  Two caches take most of that away:
 #   * per call: the prepared arguments of a call whose five tensors are the very objects of an earlier call, keyed by
-#     their identities.  A hit is checked on every use (weak references to the tensors, their data pointers and shapes),
+#     their identities.  A hit is checked on every use (weak references to the tensors, their data pointers, shapes and strides),
 #     so a tensor that was freed, resized or given new storage is described afresh; a key whose entry keeps failing that
 #     check (Python hands the address of a freed tensor object to the next one, so fresh outputs repeat ids) is marked
 #     volatile and no longer kept;
@@ -318,7 +318,6 @@ _weight_descs: Dict[int, tuple] = {}
 _ws_bytes: Dict[tuple, int] = {}
 _CACHE_MAX = 4096
 _VOLATILE = object()
-_default_cfg = None
 
 
 def _same(ref, ptr, t) -> bool:
@@ -341,10 +340,7 @@ def _weight_desc(t):
 
 
 def _gemm_constants(a, b, trans_a, trans_b, use_workspace):
-    global _default_cfg
-    if _default_cfg is None:
-        _default_cfg = make_cfg(None)
-    cfg, ncfg = _default_cfg
+    cfg, ncfg = _cfg(None)
     M = a.shape[1] if trans_a else a.shape[0]
     K = a.shape[0] if trans_a else a.shape[1]
     N = b.shape[0] if trans_b else b.shape[1]
@@ -366,7 +362,8 @@ def _prepared_gemm(c, a, b, scale_a, scale_b, trans_a, trans_b, use_workspace):
         refs, ptrs, shapes = hit[0], hit[1], hit[2]
         if (_same(refs[0], ptrs[0], c) and _same(refs[1], ptrs[1], a) and _same(refs[2], ptrs[2], b)
                 and _same(refs[3], ptrs[3], scale_a) and _same(refs[4], ptrs[4], scale_b)
-                and c.shape == shapes[0] and a.shape == shapes[1] and b.shape == shapes[2]):
+                and c.shape == shapes[0] and a.shape == shapes[1] and b.shape == shapes[2]
+                and c.stride() == shapes[3] and a.stride() == shapes[4] and b.stride() == shapes[5]):
             return hit[3]
         hit[4][0] += 1
     dev = _device_index(a)
@@ -381,7 +378,8 @@ def _prepared_gemm(c, a, b, scale_a, scale_b, trans_a, trans_b, use_workspace):
     if len(_gemm_calls) >= _CACHE_MAX:
         _gemm_calls.clear()
     _gemm_calls[key] = (tuple(None if t is None else weakref.ref(t) for t in tensors),
-                        tuple(0 if t is None else t.data_ptr() for t in tensors), (c.shape, a.shape, b.shape), prepared,
+                        tuple(0 if t is None else t.data_ptr() for t in tensors),
+                        (c.shape, a.shape, b.shape, c.stride(), a.stride(), b.stride()), prepared,
                         hit[4] if hit is not None else [0])
     return prepared
 
