@@ -70,9 +70,12 @@ enum {
                             * chooses it by itself for K <= 1536 */
     TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup, and with ROW_GROUPS = 4 (the wide form) 1 = one 1 KiB piece per wave in flight instead of two half pieces; tiled 256x256 kernels: 8 = the generic eight-wave tile kernel (one workgroup per tile) instead of the persistent one */
     TG_CFG_QUANT_BLOCK_N = 6, /* block-scaled tg_fp8_gemm: weight rows per scale (default 128) */
-    TG_CFG_QUANT_BLOCK_K = 7, /* block-scaled tg_fp8_gemm: K elements per scale (default 128); blocks other than 128 x 128
-                               * run on the fallback kernel (no MFMA): the reference's block_size=[bn, bk] argument,
-                               * src/tilegym/suites/unsloth/cutile/fp8.py:388-446 */
+    TG_CFG_QUANT_BLOCK_K = 7, /* block-scaled tg_fp8_gemm: K elements per scale (default 128): the reference's
+                               * block_size=[bn, bk] argument, src/tilegym/suites/unsloth/cutile/fp8.py:388-446.  Blocks that
+                               * are multiples of 128 x 128 (256 x 128, 128 x 256, 256 x 256, ...) run on the MFMA kernels: with
+                               * a workspace (tg_fp8_gemm_workspace_bytes counts the room) tg_fp8_gemm first writes the scales
+                               * out per 128 x 128 block; finer blocks, and coarse ones without that room, run on the fallback
+                               * kernel (no MFMA) */
     TG_CFG_PIECES = 8,  /* reported by tg_last_config only: 1, or the number of separately scheduled pieces the call ran as
                          * (column chunks of a weight of 2 GiB and more; the columns or rows that fill whole rounds of the chip
                          * with 256x256 tiles and the rest): the other slots then describe the first piece.  Ignored in cfg[]. */

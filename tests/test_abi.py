@@ -154,6 +154,16 @@ def test_moe_gemm_silu_quant_argument_validation():
     assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * 200, K), 256)
 
 
+def test_workspace_bytes_count_the_room_for_coarse_block_scales():
+    """Quantization blocks that are multiples of 128 x 128 need room to write the scales out per 128 x 128 block."""
+    L = _lib.load()
+    M, N, K = 64, 1024, 2048
+    base = L.tg_fp8_gemm_workspace_bytes(M, N, K, 1, *_lib.make_cfg(None))
+    coarse = L.tg_fp8_gemm_workspace_bytes(M, N, K, 1, *_lib.make_cfg({"QUANT_BLOCK_N": 256, "QUANT_BLOCK_K": 256}))
+    fine = L.tg_fp8_gemm_workspace_bytes(M, N, K, 1, *_lib.make_cfg({"QUANT_BLOCK_N": 64, "QUANT_BLOCK_K": 64}))
+    assert fine == base and coarse == base + M * (K // 128) * 4 + (N // 128) * (K // 128) * 4
+
+
 def test_fused_moe_argument_validation():
     """tg_fp8_fused_moe checks shapes, types, block size and workspace before any device call."""
     L = _lib.load()

@@ -229,12 +229,13 @@ def test_column_piece_with_more_than_one_row_chunk(device):
     del codes, a_dev, out
 
 
-@pytest.mark.parametrize("block_size", [[64, 64], [64, 128], [256, 32], [128, 256], [48, 80]])
-@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 256, 256), (33, 200, 328)])
+@pytest.mark.parametrize("block_size", [[64, 64], [64, 128], [256, 32], [128, 256], [48, 80], [256, 128], [256, 256], [384, 512]])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 256, 256), (33, 200, 328), (16, 1000, 1536), (700, 520, 1024)])
 def test_block_scaled_quantization_blocks_other_than_128(device, block_size, M, N, K):
     """w8a8_block_fp8_matmul with the reference's block_size=[block_n, block_k] argument
-    (src/tilegym/suites/unsloth/cutile/fp8.py:388-446) for blocks other than 128 x 128, ragged at both edges: these run
-    on the software-decode kernel and must match the oracle like every other form."""
+    (src/tilegym/suites/unsloth/cutile/fp8.py:388-446) for blocks other than 128 x 128, ragged at both edges.  Blocks that
+    are multiples of 128 x 128 run on the MFMA kernels (their scales are written out per 128 x 128 block first), the others
+    on the software-decode kernel; all must match the oracle like every other form."""
     bn, bk = block_size
     g = _g(M + N + K + bn * 3 + bk)
     A, B = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
@@ -242,7 +243,11 @@ def test_block_scaled_quantization_blocks_other_than_128(device, block_size, M, 
     Bs = torch.rand(-(-N // bn), -(-K // bk), generator=g) * 0.05 + 0.01
     ref = R.ref_w8a8_block_fp8_matmul(A, B, As, Bs, block_size, torch.bfloat16)
     out = w8a8_block_fp8_matmul(A.to(device), B.to(device), As.to(device), Bs.to(device), block_size, torch.bfloat16)
-    used("fallback")
+    cfg = _lib.last_config()
+    if bn % 128 == 0 and bk % 128 == 0 and K % 128 == 0:
+        assert cfg["KERNEL_NAME"] in ("tiled", "stream", "skinny") and (cfg["QUANT_BLOCK_N"], cfg["QUANT_BLOCK_K"]) == (bn, bk), cfg
+    else:
+        assert cfg["KERNEL_NAME"] == "fallback", cfg
     check(out, ref, what=f"block_size={block_size} M={M} N={N} K={K}")
     # the same problem described with 128 x 128 scales has other shapes: the library must refuse the mismatch
     if (As.shape[1], Bs.shape) != (-(-K // 128), (-(-N // 128), -(-K // 128))):

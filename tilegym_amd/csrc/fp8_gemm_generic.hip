@@ -148,6 +148,23 @@ hipError_t run_splitk_reduce(const GemmParams& p, bool block_scaled, hipStream_t
     return hipGetLastError();
 }
 
+// Block scales given per (qbn x qbk) block, qbn and qbk multiples of 128, written out per 128 x 128 block: out[r][kb] =
+// in[r / rdiv][kb / kdiv] (rdiv = qbn / 128 for weight scales, 1 for the activations' per-row scales; kdiv = qbk / 128).
+__global__ void __launch_bounds__(256) expand_scales_kernel(const float* __restrict__ in, float* __restrict__ out, int rows_out, int cols_out,
+                                                            int in_cols, int rdiv, int kdiv) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)rows_out * cols_out) return;
+    const int r = (int)(idx / cols_out), kb = (int)(idx % cols_out);
+    out[idx] = in[(int64_t)(r / rdiv) * in_cols + kb / kdiv];
+}
+
+hipError_t run_expand_scales(const float* in, float* out, int rows_out, int cols_out, int in_cols, int rdiv, int kdiv, hipStream_t s) {
+    const int64_t work = (int64_t)rows_out * cols_out;
+    if (work <= 0) return hipSuccess;
+    hipLaunchKernelGGL(expand_scales_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, in, out, rows_out, cols_out, in_cols, rdiv, kdiv);
+    return hipGetLastError();
+}
+
 hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s) {
     if (rows <= 0 || cols <= 0) return hipSuccess;
     dim3 grid((cols + 63) / 64, (rows + 63) / 64, 1);

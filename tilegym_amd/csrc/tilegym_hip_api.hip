@@ -126,6 +126,17 @@ hipError_t scratch_address(int dev, uint8_t** out) {
     return hipSuccess;
 }
 
+// Bytes of the block scales of a (M, N, K) problem written out per 128 x 128 block, when cfg[] names quantization blocks that are
+// larger multiples of 128 (else 0: nothing to write out)
+int64_t expanded_scale_bytes(int64_t M, int64_t N, int64_t K, const int32_t* cfg, int32_t ncfg) {
+    int64_t qbn = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_N), qbk = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_K);
+    if (qbn <= 0) qbn = 128;
+    if (qbk <= 0) qbk = 128;
+    if ((qbn == 128 && qbk == 128) || qbn % 128 != 0 || qbk % 128 != 0) return 0;
+    const int64_t kblocks = cdiv(K, 128), nblocks = cdiv(N, 128);
+    return (M * kblocks * 4 + 255) / 256 * 256 + (nblocks * kblocks * 4 + 255) / 256 * 256;
+}
+
 struct Schedule {
     int kernel;  // 0 fallback, 1 tiled, 2 skinny, 3 stream
     int bm, bn, split_k, row_groups, mt, waves;
@@ -394,6 +405,7 @@ int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t tra
     if (partial > cap) partial = cap;
     bytes += (partial + 255) / 256 * 256;
     if (!trans_b) bytes += (N * K + 255) / 256 * 256;
+    bytes += expanded_scale_bytes(M, N, K, cfg, ncfg);
     return bytes;
 }
 
@@ -401,6 +413,46 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
                     const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
                     int32_t trans_b, float alpha, float beta, const tg_tensor* workspace,
                     const int32_t* cfg, int32_t ncfg, int32_t device_id, uint64_t hip_stream) {
+    // Quantization blocks that are multiples of 128 x 128 (cfg[] slots QUANT_BLOCK_N / _K: 256 x 128, 128 x 256, 256 x 256,
+    // ...): the scales are written out per 128 x 128 block at the tail of the workspace (one small launch each) and the
+    // problem runs on the MFMA kernels like any 128 x 128 one -- the same products times the same scales, added in the
+    // same order.  Without a workspace that holds them, and for finer blocks, the fallback kernel takes the problem.
+    const int64_t qbn = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_N), qbk = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_K);
+    if (a && b && c && scale_a && scale_b && workspace && a->ndim == 2 && b->ndim == 2 && !trans_a && trans_b &&
+        cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0) {
+        const int64_t M = a->shape[0], K = a->shape[1], N = b->shape[0];
+        const int64_t need = expanded_scale_bytes(M, N, K, cfg, ncfg);
+        const int64_t bn = qbn > 0 ? qbn : 128, bk = qbk > 0 ? qbk : 128;
+        const int64_t kblocks = cdiv(K, 128), nblocks = cdiv(N, 128), in_cols = cdiv(K, bk);
+        const int64_t ws_bytes = workspace->ptr ? numel(workspace) * elem_size(workspace->dtype) : 0;
+        const bool shapes_ok = scale_a->dtype == TG_F32 && scale_b->dtype == TG_F32 && scale_a->ndim == 2 && scale_b->ndim == 2 &&
+                               scale_a->shape[0] == M && scale_a->shape[1] == in_cols && scale_b->shape[0] == cdiv(N, bn) &&
+                               scale_b->shape[1] == in_cols && contiguous(scale_a) && contiguous(scale_b) && scale_a->ptr && scale_b->ptr;
+        if (need > 0 && shapes_ok && ws_bytes >= need && M > 0 && N > 0 && K > 0 && M <= INT32_MAX && N <= INT32_MAX && K <= INT32_MAX) {
+            g_err[0] = 0;
+            DeviceGuard guard(device_id);
+            if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+            hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+            const int64_t a_bytes = (M * kblocks * 4 + 255) / 256 * 256;
+            uint8_t* tail = reinterpret_cast<uint8_t*>(workspace->ptr) + (ws_bytes - need) / 256 * 256;
+            float* ea = reinterpret_cast<float*>(tail);
+            float* eb = reinterpret_cast<float*>(tail + a_bytes);
+            if (tg::run_expand_scales(reinterpret_cast<const float*>(scale_a->ptr), ea, (int)M, (int)kblocks, (int)in_cols, 1, (int)(bk / 128), stream) != hipSuccess ||
+                tg::run_expand_scales(reinterpret_cast<const float*>(scale_b->ptr), eb, (int)nblocks, (int)kblocks, (int)in_cols, (int)(bn / 128), (int)(bk / 128), stream) != hipSuccess)
+                return fail(TG_ERR_LAUNCH, "scale expansion launch failed");
+            tg_tensor sa2 = *scale_a, sb2 = *scale_b, ws2 = *workspace;
+            sa2.ptr = reinterpret_cast<uint64_t>(ea); sa2.shape[1] = kblocks; sa2.strides[0] = kblocks;
+            sb2.ptr = reinterpret_cast<uint64_t>(eb); sb2.shape[0] = nblocks; sb2.shape[1] = kblocks; sb2.strides[0] = kblocks;
+            ws2.ndim = 1; ws2.shape[0] = (int64_t)(tail - reinterpret_cast<uint8_t*>(workspace->ptr)) / elem_size(workspace->dtype); ws2.strides[0] = 1;
+            int32_t cfg2[TG_CFG_COUNT];
+            for (int i = 0; i < TG_CFG_COUNT; ++i) cfg2[i] = cfg_get(cfg, ncfg, i);
+            cfg2[TG_CFG_QUANT_BLOCK_N] = cfg2[TG_CFG_QUANT_BLOCK_K] = -1;
+            const int32_t rc = fp8_gemm_impl(c, a, b, &sa2, &sb2, trans_a, trans_b, alpha, beta, &ws2, false, cfg2, TG_CFG_COUNT, device_id, hip_stream);
+            g_last_cfg[TG_CFG_QUANT_BLOCK_N] = (int32_t)bn;
+            g_last_cfg[TG_CFG_QUANT_BLOCK_K] = (int32_t)bk;
+            return rc;
+        }
+    }
     return fp8_gemm_impl(c, a, b, scale_a, scale_b, trans_a, trans_b, alpha, beta, workspace, false, cfg, ncfg,
                          device_id, hip_stream);
 }
