@@ -180,3 +180,29 @@ def test_release_workspaces_empties_the_cache():
     from tilegym_amd import _lib
     _lib._workspaces[(0, 0, False)] = [__import__("torch").empty(1024, dtype=__import__("torch").uint8)]
     assert _lib.release_workspaces() == 1024 and not _lib._workspaces
+
+
+def test_recorded_schedule_table_round_trip(tmp_path):
+    """tilegym_amd.tune writes a table, _lib reads it: entries are kernel_configs per (M, N, K, block-scaled?), entries
+    whose best schedule is the automatic one are dropped, a later run merges, and an unknown shape gets the automatic cfg."""
+    from tilegym_amd import _lib, tune
+
+    path = str(tmp_path / "tune.json")
+    tune.write_table([{"M": 16, "N": 5120, "K": 12288, "block_scaled": False, "kernel_configs": {"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": 6},
+                       "us": 14.5, "auto_us": 16.0, "auto_schedule": {}},
+                      {"M": 1, "N": 4096, "K": 4096, "block_scaled": True, "kernel_configs": {}, "us": 6.3, "auto_us": 6.3, "auto_schedule": {}}], path)
+    tune.write_table([{"M": 8, "N": 4096, "K": 11008, "block_scaled": True, "kernel_configs": {"KERNEL": "stream", "WAVES": 8},
+                       "us": 14.0, "auto_us": 14.6, "auto_schedule": {}}], path)
+    try:
+        table = _lib.load_tune_table(path)
+        assert set(table) == {(16, 5120, 12288, False), (8, 4096, 11008, True)}
+        cfg, n = _lib._tuned_cfg(16, 5120, 12288, False)
+        assert n == _lib.TG_CFG_COUNT and cfg[_lib.CFG_SLOTS["KERNEL"]] == 3 and cfg[_lib.CFG_SLOTS["SPLIT_K"]] == 6
+        assert cfg[_lib.CFG_SLOTS["ROW_GROUPS"]] == 4 and cfg[_lib.CFG_SLOTS["WAVES"]] == -1
+        auto, _ = _lib._tuned_cfg(16, 5120, 12288, True)   # same shape, other scaling: not in the table
+        assert all(auto[i] == -1 for i in range(_lib.TG_CFG_COUNT))
+    finally:
+        assert _lib.load_tune_table("") == {}
+    assert [c for c in tune.candidates(1, 4096, 4096, False) if c["KERNEL"] == "tiled"] == []
+    assert {"KERNEL": "tiled", "BLOCK_M": 256, "BLOCK_N": 256, "SPLIT_K": 1} in tune.candidates(4096, 4096, 4096, True)
+    assert tune._parse_shape("8,4096,11008,block") == (8, 4096, 11008, True) and tune._parse_shape("8,4096,11008") == (8, 4096, 11008, False)

@@ -1621,6 +1621,41 @@ def test_config5_fused_experts_decode_regime(device, T):
     assert rep["matched"] >= 0.999 and rep["max_rel_to_sigma"] <= 0.1, rep
 
 
+def test_recorded_schedule_is_used_when_no_kernel_configs_are_given(device, tmp_path):
+    """A table written by tilegym_amd.tune (here: by hand, and by tune_shape on a small shape) decides the schedule of calls
+    that bring no kernel_configs; explicit kernel_configs still win; unloading the table restores the automatic choice."""
+    from tilegym_amd import tune
+
+    g = _g(321)
+    M, N, K = 8, 4096, 4096
+    a, b = fp8_randn((M, K), g).to(device), fp8_randn((N, K), g, 0.02).to(device)
+    sa, sb = torch.tensor([0.5], device=device), torch.tensor([0.25], device=device)
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+    ref = ((a.float() * 0.5) @ (b.float() * 0.25).t()).to(torch.bfloat16).cpu()
+    _lib.fp8_gemm(c, a, b, sa, sb)
+    auto = _lib.last_config()
+    assert (auto["ROW_GROUPS"], auto["SPLIT_K"]) == (1, 1), auto       # the narrow form
+    path = str(tmp_path / "tune.json")
+    tune.write_table([{"M": M, "N": N, "K": K, "block_scaled": False, "kernel_configs": {"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": 2},
+                       "us": 0.0, "auto_us": 0.0, "auto_schedule": {}}], path)
+    try:
+        _lib.load_tune_table(path)
+        for _ in range(2):                                             # the second call comes from the prepared-call cache
+            _lib.fp8_gemm(c, a, b, sa, sb)
+            got = _lib.last_config()
+            assert (got["KERNEL_NAME"], got["ROW_GROUPS"], got["SPLIT_K"]) == ("stream", 4, 2), got
+            check(c, ref, what="recorded schedule")
+        _lib.fp8_gemm(c, a, b, sa, sb, kernel_configs={"KERNEL": "stream", "WAVES": 8})
+        assert _lib.last_config()["WAVES"] == 8
+    finally:
+        _lib.load_tune_table("")
+    _lib.fp8_gemm(c, a, b, sa, sb)
+    assert _lib.last_config() == auto
+    entry = tune.tune_shape(4, 1024, 2048, False)
+    assert entry["us"] <= entry["auto_us"] and entry["auto_schedule"]["KERNEL_NAME"] == "stream"
+    assert entry["kernel_configs"] == {} or entry["us"] <= 0.97 * entry["auto_us"]
+
+
 def test_prepared_call_cache_follows_the_tensors(device):
     """The binding keeps the prepared arguments of a call by the identity of its tensors.  The same objects again: same
     result; an operand given new storage, a resized output, fresh outputs whose Python ids repeat, a dead weight whose id

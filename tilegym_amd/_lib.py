@@ -339,18 +339,57 @@ def _weight_desc(t):
     return d
 
 
-def _gemm_constants(a, b, trans_a, trans_b, use_workspace):
-    cfg, ncfg = _cfg(None)
+# ---- recorded schedules: TILEGYM_HIP_TUNE names a JSON file written by ``python -m tilegym_amd.tune`` that maps
+# (M, N, K, block-scaled?) to the kernel_configs that measured fastest on this GPU; a call without kernel_configs of its own
+# takes the recorded ones (the reference keeps per-architecture config tables and a search for the same purpose,
+# src/tilegym/ops/cutile/matmul.py:47-141,327-418).  Without the variable nothing is looked up.
+TUNE_ENV = "TILEGYM_HIP_TUNE"
+_tune_table: Optional[Dict[tuple, dict]] = None
+
+
+def load_tune_table(path: Optional[str] = None) -> Dict[tuple, dict]:
+    """(Re)load the schedule table from ``path`` (default: the file TILEGYM_HIP_TUNE names; no file -> empty table) and forget
+    the prepared calls that were made under the previous one."""
+    global _tune_table
+    import json
+    path = path if path is not None else os.environ.get(TUNE_ENV)
+    table: Dict[tuple, dict] = {}
+    if path:
+        with open(path) as f:
+            doc = json.load(f)
+        for e in doc.get("entries", []):
+            table[(int(e["M"]), int(e["N"]), int(e["K"]), bool(e.get("block_scaled", False)))] = dict(e["kernel_configs"])
+    _tune_table = table
+    _gemm_calls.clear()
+    _ws_bytes.clear()
+    return table
+
+
+def _tuned_cfg(M: int, N: int, K: int, block_scaled: bool):
+    """(cfg array, length) for a dense problem: the recorded schedule if there is one, else all-automatic."""
+    table = _tune_table if _tune_table is not None else load_tune_table()
+    if table:
+        kc = table.get((M, N, K, block_scaled))
+        if kc:
+            return make_cfg(kc)
+    return _cfg(None)
+
+
+def _gemm_constants(a, b, scale_b, trans_a, trans_b, use_workspace):
     M = a.shape[1] if trans_a else a.shape[0]
     K = a.shape[0] if trans_a else a.shape[1]
     N = b.shape[0] if trans_b else b.shape[1]
+    cfg, ncfg = _tuned_cfg(M, N, K, scale_b is not None and scale_b.numel() > 1)
     ws_bytes = 0
     if use_workspace and M > 0 and N > 0 and K > 0:
-        ws_bytes = _ws_bytes.get((M, N, K, trans_b))
+        key = (M, N, K, trans_b, cfg is _cfg(None)[0])
+        ws_bytes = _ws_bytes.get(key) if key[4] else None   # (a recorded schedule may ask for another split)
         if ws_bytes is None:
             if len(_ws_bytes) >= _CACHE_MAX:
                 _ws_bytes.clear()
-            ws_bytes = _ws_bytes[(M, N, K, trans_b)] = workspace_bytes(M, N, K, trans_b, cfg, ncfg)
+            ws_bytes = workspace_bytes(M, N, K, trans_b, cfg, ncfg)
+            if key[4]:
+                _ws_bytes[key] = ws_bytes
     return cfg, ncfg, ws_bytes
 
 
@@ -367,7 +406,7 @@ def _prepared_gemm(c, a, b, scale_a, scale_b, trans_a, trans_b, use_workspace):
             return hit[3]
         hit[4][0] += 1
     dev = _device_index(a)
-    cfg, ncfg, ws_bytes = _gemm_constants(a, b, trans_a, trans_b, use_workspace)
+    cfg, ncfg, ws_bytes = _gemm_constants(a, b, scale_b, trans_a, trans_b, use_workspace)
     if hit is _VOLATILE or (hit is not None and hit[4][0] >= 2):
         _gemm_calls[key] = _VOLATILE
         descs = (_desc(c), _desc(a), _weight_desc(b), _desc(scale_a), _weight_desc(scale_b))
