@@ -195,6 +195,54 @@ int pick_split(int64_t units, int64_t target_units, int64_t kblocks, int min_ste
     return (int)cdiv(kblocks, kps);
 }
 
+// Cost model of the LDS-tiled kernels above 64 rows.  Per tile kind: microseconds per K step of a tile while its compute
+// unit holds one workgroup (`alone`: the launch has at most 256 tiles) or two (`shared`), and per tile for set-up, first
+// loads and epilogue (`fixed`).  A launch takes rounds x (K steps x step + fixed), rounds = tiles / 256 or tiles / 512
+// rounded up, plus, with split-K, the reduction launch (kReduceUs + kReduceUsPerMB x the partial sums).  The numbers are a
+// least-squares fit to 9 600 measurements on MI355X: 360 shapes (M = 96 ... 8192, 18 weight shapes, both scalings) x every
+// tile x 1 / 2 / 4 / 8 splits, weights rotated past the caches, launches replayed from a graph.  The schedule it picks is
+// within 1 % of the best measured one on average (worst case 12 %; the rules it replaces: 7 - 8 % and 2.0 x).
+struct TileCost { int bm, bn; float alone, shared, fixed; };
+constexpr TileCost kPerTensorTiles[] = {{32, 32, 0.132f, 0.332f, 2.80f},   {64, 32, 0.178f, 0.405f, 3.46f},
+                                        {64, 64, 0.249f, 0.596f, 4.43f},   {64, 128, 0.414f, 0.811f, 4.02f},
+                                        {128, 128, 0.650f, 0.929f, 3.70f}, {128, 256, 0.874f, 1.782f, 6.88f},
+                                        {256, 256, 1.150f, 1.150f, 8.19f}};
+// (block-scaled 128 x 256 exists and can be forced; leaving it out of the automatic choice measured better)
+constexpr TileCost kBlockScaledTiles[] = {{64, 128, 0.685f, 0.851f, 3.50f}, {128, 128, 0.690f, 1.016f, 4.23f},
+                                          {256, 256, 1.496f, 1.496f, 8.11f}};
+constexpr float kReduceUs = 6.0f, kReduceUsPerMB = 0.235f;
+constexpr float kSplitMargin = 1.05f;  // a split schedule must be predicted this much faster than the best unsplit one
+
+float tile_cost_us(const TileCost& t, int64_t M, int64_t N, int64_t kblocks, int split) {
+    const int64_t tiles = cdiv(M, t.bm) * cdiv(N, t.bn) * split, ksteps = cdiv(kblocks, split);
+    const bool one_per_cu = t.bm == 256 && t.bn == 256;
+    float us = (one_per_cu || tiles <= 256) ? (float)cdiv(tiles, 256) * ((float)ksteps * t.alone + t.fixed)
+                                            : (float)cdiv(tiles, 512) * ((float)ksteps * t.shared + t.fixed);
+    if (split > 1) us += kReduceUs + kReduceUsPerMB * (float)(M * N * 4 * split) * 1e-6f;
+    return us;
+}
+
+// The cheapest (tile, split) by the model; a tile (bm > 0) or a split (want_split > 0) given by the caller is kept.
+void pick_tile_by_cost(int64_t M, int64_t N, int64_t kblocks, bool block_scaled, int64_t partial_bytes_avail, int want_split,
+                       int* bm, int* bn, int* split) {
+    const TileCost* kinds = block_scaled ? kBlockScaledTiles : kPerTensorTiles;
+    const int n_kinds = block_scaled ? (int)(sizeof(kBlockScaledTiles) / sizeof(TileCost)) : (int)(sizeof(kPerTensorTiles) / sizeof(TileCost));
+    float best = 0.f;
+    int best_bm = -1, best_bn = -1, best_split = 1;
+    for (int i = 0; i < n_kinds; ++i) {
+        const TileCost& t = kinds[i];
+        if (*bm > 0 && (t.bm != *bm || t.bn != *bn)) continue;
+        if (want_split > 1 && is_mid_tile(t.bm, t.bn)) continue;  // these split K inside the workgroup only
+        for (int sp = 1; sp <= 8; sp *= 2) {
+            if (want_split > 0 && sp != 1) break;          // the caller's split is applied by the caller
+            if (sp > 1 && (is_mid_tile(t.bm, t.bn) || kblocks / sp < 4 || (int64_t)sp * M * N * 4 > partial_bytes_avail)) break;
+            const float us = tile_cost_us(t, M, N, kblocks, want_split > 0 ? want_split : sp) * (sp > 1 ? kSplitMargin : 1.f);
+            if (best_bm < 0 || us < best) { best = us; best_bm = t.bm; best_bn = t.bn; best_split = sp; }
+        }
+    }
+    if (best_bm > 0) { *bm = best_bm; *bn = best_bn; *split = best_split; }
+}
+
 Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
                       const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
     Schedule s{0, -1, -1, 1, -1, -1, -1};
@@ -294,31 +342,19 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     }
     s.kernel = 1;
     int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
-    if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, block_scaled))) {
+    if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, block_scaled))) bm = bn = -1;
+    int model_split = 1;
+    if (M > 64) {
+        pick_tile_by_cost(M, N, kblocks, block_scaled, partial_bytes_avail, want_split, &bm, &bn, &model_split);
+    } else if (bm < 0) {
         auto tiles = [&](int64_t a, int64_t b) { return cdiv(M, a) * cdiv(N, b); };
-        // Measured on MI355X (256 CUs): the 256x256 tile (one workgroup per CU) moves half the bytes
-        // per FLOP into a CU and runs ~1.2x faster than 128x128 (two workgroups per CU) when its tile
-        // count fills whole rounds of the chip; a last round that is mostly empty costs more than
-        // that, so compare the two by (fraction of the rounds' slots that hold a tile) x (tile rate).
-        auto fill = [&](int64_t n, int64_t slots) { return (double)n / (double)(cdiv(n, slots) * slots); };
-        // (per-tensor: the persistent four-wave 256x256 kernel is another 8 % ahead of its eight-wave form, hence 0.77)
-        const double s256 = fill(tiles(256, 256), 256) * 1.0, s128 = fill(tiles(128, 128), 512) * (block_scaled ? 0.83 : 0.77);
-        // the three-stage 64x128 kernel (per-tensor) also wins above 64 rows while its tiles fit one round of the
-        // chip: 13.3 / 14.5 / 17.8 / 18.1 us against 17.1 / 18.8 / 18.7 / 21.6 for M = 96 / 128 / 256 / 512 at
-        // N = K = 4096; with more tiles the larger tiles' operand reuse wins (M = 1024: 32 vs 23 us)
-        // small weights at 16 < M <= 256: narrow tiles whose four waves split K inside the workgroup fill the chip in
-        // one launch, where the 64x128 tile needs split-K and a reduction launch (4096 x 4096 weight: 7.9 / 7.9 / 9.8 /
-        // 12.5 us at M = 32 / 64 / 128 / 256 against 10.4 / 12.0 / 14.7 / 17.6; 6144 x 4096: 9.4 / 10.2 / 12.9 against
-        // 11.8 / 13.3 / 16.7 at M = 32 / 64 / 128).  Beyond one round of workgroups, or when the weights dominate
-        // (>= 32 MiB), the activation re-reads cost more.
-        const bool small_w = !block_scaled && M <= 256 && N * K <= ((int64_t)32 << 20) && cfg_get(cfg, ncfg, TG_CFG_SPLIT_K) <= 1;
-        if (small_w && M <= 64 && tiles(32, 32) <= 256) { bm = 32; bn = 32; }
-        else if (small_w && M <= 128 && tiles(64, 32) <= 256) { bm = 64; bn = 32; }
-        else if (small_w && M > 64 && tiles(64, 64) <= 256) { bm = 64; bn = 64; }
-        else if (M <= 64 || (!block_scaled && tiles(64, 128) <= 256)) { bm = 64; bn = 128; }
-        else if (tiles(256, 256) >= 200 && s256 >= s128) { bm = 256; bn = 256; }
-        else if (!block_scaled && tiles(128, 256) >= 200 && tiles(256, 256) < 200) { bm = 128; bn = 256; }
-        else if (tiles(128, 128) >= 128 || M > 64) { bm = 128; bn = 128; }
+        // small weights at 16 < M <= 64: narrow tiles whose four waves split K inside the workgroup fill the chip in
+        // one launch, where the 64x128 tile needs split-K and a reduction launch (4096 x 4096 weight: 7.9 / 7.9 us at
+        // M = 32 / 64 against 10.4 / 12.0; 6144 x 4096: 9.4 / 10.2 against 11.8 / 13.3).  Beyond one round of
+        // workgroups, or when the weights dominate (>= 32 MiB), the activation re-reads cost more.
+        const bool small_w = !block_scaled && N * K <= ((int64_t)32 << 20) && want_split <= 1;
+        if (small_w && tiles(32, 32) <= 256) { bm = 32; bn = 32; }
+        else if (small_w && tiles(64, 32) <= 256) { bm = 64; bn = 32; }
         else { bm = 64; bn = 128; }
     }
     s.bm = bm;
@@ -328,6 +364,8 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     if (is_mid_tile(bm, bn)) return s;  // K is split inside the workgroup: one launch
     if (want_split > 1) {
         s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
+    } else if (M > 64) {
+        if (want_split < 0 && model_split > 1) s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, model_split);
     } else if (want_split < 0 && bm == 64 && bn == 128 && !block_scaled) {
         // weight-streaming regime, four-stage 64x128 kernel (one workgroup per compute unit): the largest
         // power-of-two split that keeps the grid within one round of the chip and >= 8 K steps per split
@@ -343,8 +381,6 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         int want = 1;
         while (want * wgs < units && want < 16) want *= 2;
         if (want > 1) s.split_k = pick_split(wgs, units, kblocks, 4, M, N, partial_bytes_avail, want);
-    } else if (want_split < 0 && wgs <= 128) {
-        s.split_k = pick_split(wgs, 256, kblocks, 4, M, N, partial_bytes_avail, want_split);
     }
     return s;
 }
@@ -525,7 +561,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
 
     // ---- column chunks.  The columns of C (rows of an (N, K) weight) can be computed in pieces, each a call of its own on
     // the same stream and workspace; the pieces take C's real row stride as an argument.
-    auto run_columns = [&](int64_t n0, int64_t cn) -> int32_t {
+    auto run_columns = [&](int64_t n0, int64_t cn, const int32_t* piece_cfg, int32_t piece_ncfg) -> int32_t {
         tg_tensor bs = *b, cs = *c, sbs;
         bs.ptr = b->ptr + (uint64_t)(n0 * K);
         bs.shape[0] = cn;
@@ -539,7 +575,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
             sbs.shape[0] = cdiv(cn, 128);
             sb = &sbs;
         }
-        return fp8_gemm_impl(&cs, a, &bs, scale_a, sb, trans_a, trans_b, alpha, beta, workspace, static_scratch, cfg, ncfg, device_id, hip_stream, N);
+        return fp8_gemm_impl(&cs, a, &bs, scale_a, sb, trans_a, trans_b, alpha, beta, workspace, static_scratch, piece_cfg, piece_ncfg, device_id, hip_stream, N);
     };
     const bool can_chunk = !chunk_ldc && std_blocks && trans_b && !trans_a && K > 0 && (K % 16) == 0 && aligned16(a->ptr) &&
                            aligned16(b->ptr) && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0;
@@ -548,7 +584,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         const int64_t chunk_n = ((kOffsetLimit - 1) / K) / 256 * 256;
         PieceRecord pieces;
         for (int64_t n0 = 0; n0 < N; n0 += chunk_n) {
-            if ((rc = run_columns(n0, (N - n0) < chunk_n ? (N - n0) : chunk_n))) return rc;
+            if ((rc = run_columns(n0, (N - n0) < chunk_n ? (N - n0) : chunk_n, cfg, ncfg))) return rc;
             pieces.after_piece();
         }
         pieces.publish();
@@ -565,10 +601,16 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
             const int64_t n1 = ((total / 256) * 256) / tm;   // column tiles that fit the whole rounds
             const int64_t m1 = ((total / 256) * 256) / tn;   // or row tiles
             PieceRecord pieces;
+            // the piece that fills whole rounds runs with 256 x 256 tiles whatever the cost model would say of it alone
+            int32_t full_cfg[TG_CFG_COUNT];
+            for (int i = 0; i < TG_CFG_COUNT; ++i) full_cfg[i] = cfg_get(cfg, ncfg, i);
+            full_cfg[TG_CFG_KERNEL] = 1;
+            full_cfg[TG_CFG_BLOCK_M] = full_cfg[TG_CFG_BLOCK_N] = 256;
+            full_cfg[TG_CFG_SPLIT_K] = 1;
             if (n1 >= 1 && n1 < tn && fills(tm * n1)) {
-                if ((rc = run_columns(0, n1 * 256))) return rc;
+                if ((rc = run_columns(0, n1 * 256, full_cfg, TG_CFG_COUNT))) return rc;
                 pieces.after_piece();
-                if ((rc = run_columns(n1 * 256, N - n1 * 256))) return rc;
+                if ((rc = run_columns(n1 * 256, N - n1 * 256, cfg, ncfg))) return rc;
                 pieces.after_piece();
                 pieces.publish();
                 return TG_OK;
@@ -590,7 +632,8 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
                         sa = &sas;
                     }
                     // (piece_ldc = N marks the call as a piece: no further splitting)
-                    rc = fp8_gemm_impl(&cs, &as, b, sa, scale_b, trans_a, trans_b, alpha, beta, workspace, static_scratch, cfg, ncfg, device_id, hip_stream, N);
+                    rc = fp8_gemm_impl(&cs, &as, b, sa, scale_b, trans_a, trans_b, alpha, beta, workspace, static_scratch,
+                                       piece ? cfg : full_cfg, piece ? ncfg : TG_CFG_COUNT, device_id, hip_stream, N);
                     if (rc) return rc;
                     pieces.after_piece();
                 }

@@ -24,6 +24,7 @@ import torch
 from . import _lib
 
 ROTATE_BYTES = 768 << 20
+REPORTED = ("KERNEL_NAME", "BLOCK_M", "BLOCK_N", "SPLIT_K", "ROW_GROUPS", "WAVES")
 
 
 def candidates(M: int, N: int, K: int, block_scaled: bool) -> List[dict]:
@@ -36,7 +37,7 @@ def candidates(M: int, N: int, K: int, block_scaled: bool) -> List[dict]:
     if M <= 64:
         out += [{"KERNEL": "skinny"}]
     if M > 16 and K % 128 == 0:
-        tiles = [(64, 128), (128, 128), (256, 256)] + ([] if block_scaled else [(32, 32), (64, 32), (64, 64)])
+        tiles = [(64, 128), (128, 128), (128, 256), (256, 256)] + ([] if block_scaled else [(32, 32), (64, 32), (64, 64)])
         for bm, bn in tiles:
             for s in (1, 2, 4, 8):
                 if s > 1 and (bm, bn) in ((32, 32), (64, 32), (64, 64)):
@@ -77,8 +78,10 @@ def _graph_us(fn, launches: int) -> float:
     return best
 
 
-def tune_shape(M: int, N: int, K: int, block_scaled: bool = False, device: Optional[torch.device] = None) -> dict:
-    """Time the automatic schedule and every candidate; returns a table entry (kernel_configs = {} when automatic wins)."""
+def tune_shape(M: int, N: int, K: int, block_scaled: bool = False, device: Optional[torch.device] = None,
+               keep_timings: bool = False) -> dict:
+    """Time the automatic schedule and every candidate; returns a table entry (kernel_configs = {} when automatic wins;
+    with keep_timings every candidate's time and the schedule it ran as, under "timings")."""
     device = device or torch.device("cuda", torch.cuda.current_device())
     gen = torch.Generator(device=device)
     gen.manual_seed(M * 7 + N + K)
@@ -104,17 +107,28 @@ def tune_shape(M: int, N: int, K: int, block_scaled: bool = False, device: Optio
         ran = _lib.last_config()
         return _graph_us(fn, copies), ran
 
-    auto_us, auto_ran = timed({"KERNEL": -1})   # an explicit all-automatic cfg: a loaded table is not consulted
-    best_kc, best_us = {}, auto_us
+    automatic = {"KERNEL": -1}                   # an explicit all-automatic cfg: a loaded table is not consulted
+    timed(automatic)                             # clocks and caches settle on the first graph; its time is not used
+    auto_us, auto_ran = timed(automatic)
+    best_kc, best_us, timings = {}, float("inf"), []
     for kc in candidates(M, N, K, block_scaled):
         us, ran = timed(kc)
-        if us is not None and ran["KERNEL_NAME"] == (kc["KERNEL"] if isinstance(kc["KERNEL"], str) else ran["KERNEL_NAME"]) and us < best_us:
+        if us is None or ran["KERNEL_NAME"] != kc["KERNEL"]:
+            continue
+        timings.append([kc, round(us, 2), {k: ran[k] for k in REPORTED}])
+        if us < best_us:
             best_kc, best_us = kc, us
+    auto_us = min(auto_us, timed(automatic)[0])  # and once more behind the candidates
+    if best_kc:
+        best_us = min(best_us, timed(best_kc)[0])
     # a forced schedule must beat the automatic one by more than the noise of the measurement to be recorded
     if best_us > 0.97 * auto_us:
         best_kc, best_us = {}, auto_us
-    return {"M": M, "N": N, "K": K, "block_scaled": bool(block_scaled), "kernel_configs": best_kc, "us": round(best_us, 2),
-            "auto_us": round(auto_us, 2), "auto_schedule": {k: auto_ran[k] for k in ("KERNEL_NAME", "BLOCK_M", "BLOCK_N", "SPLIT_K", "ROW_GROUPS", "WAVES")}}
+    entry = {"M": M, "N": N, "K": K, "block_scaled": bool(block_scaled), "kernel_configs": best_kc, "us": round(best_us, 2),
+             "auto_us": round(auto_us, 2), "auto_schedule": {k: auto_ran[k] for k in REPORTED}}
+    if keep_timings:
+        entry["timings"] = timings
+    return entry
 
 
 def write_table(entries: Iterable[dict], path: str) -> None:
@@ -146,17 +160,21 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--shape", type=_parse_shape, action="append", required=True, help="M,N,K[,block|tensor] (repeatable)")
     ap.add_argument("--out", required=True, help="JSON table to create or merge into")
+    ap.add_argument("--timings", help="also write every candidate's time per shape to this JSON file")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         raise SystemExit("tilegym_amd.tune measures on the GPU; none is visible")
     _lib.load()
     entries = []
     for M, N, K, bs in args.shape:
-        e = tune_shape(M, N, K, bs)
+        e = tune_shape(M, N, K, bs, keep_timings=bool(args.timings))
         entries.append(e)
         print(f"M={M} N={N} K={K} {'block' if bs else 'tensor'}: automatic {e['auto_us']} us ({e['auto_schedule']}), "
               f"best {e['us']} us {e['kernel_configs'] or '(automatic)'}", flush=True)
-    write_table(entries, args.out)
+    if args.timings:
+        with open(args.timings, "w") as f:
+            json.dump(entries, f, indent=1)
+    write_table([{k: v for k, v in e.items() if k != "timings"} for e in entries], args.out)
     return 0
 
 
