@@ -484,17 +484,25 @@ def test_stream_wide_two_row_tiles(device, M, N, K, split):
           what=f"block-scaled stream wide, two row tiles M={M} N={N} K={K}")
 
 
-def test_stream_wide_is_the_default_for_32_rows_over_a_large_weight(device):
-    """4096 x 14336 (58 MB) at M = 32 streams; 6144 x 4096 (25 MB) stays with the tile kernels."""
+def test_kernel_choice_at_32_rows_follows_the_cost_model(device):
+    """17 .. 64 rows: the cheapest of tile kernels, wide streaming form and skinny kernel by the fitted cost model.
+    16384 x 1024 at M = 32 streams (256 workgroups, one 1 KiB piece each); 4096 x 14336 takes 64 x 128 tiles with eight
+    splits (16.7 us against 18.1 for the streaming form with four); 6144 x 4096 takes tiles that split K inside the workgroup."""
     g = _g(41)
-    a, b = fp8_randn((32, 14336), g), fp8_randn((4096, 14336), g, 0.02)
+    a, b = fp8_randn((32, 1024), g), fp8_randn((16384, 1024), g, 0.02)
     out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
     cfg = used("stream")
-    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == 4, cfg
+    assert cfg["ROW_GROUPS"] == 4 and cfg["SPLIT_K"] == 1, cfg
+    check(out, R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True), what="16384 x 1024, M=32")
+    a, b = fp8_randn((32, 14336), g), fp8_randn((4096, 14336), g, 0.02)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["SPLIT_K"]) == (64, 128, 8), cfg
     check(out, R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True), what="down projection, M=32")
     a, b = fp8_randn((32, 4096), g), fp8_randn((6144, 4096), g, 0.02)
     out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
-    used("tiled")
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"]) in ((32, 32), (64, 32)), cfg
     check(out, R.ref_gemm_per_tensor(a, b, 0.01, 0.02, trans_b=True), what="qkv projection, M=32")
 
 

@@ -103,12 +103,17 @@ MID_SHAPES = [(160, 7168, 3584), (448, 3584, 7168), (1152, 9216, 4608), (2304, 4
               (5000, 2560, 6912), (272, 13824, 5120), (1792, 6912, 2560)]
 
 
+# 17 .. 64 rows: tile kernels, wide streaming form and skinny kernel compete
+SMALL_ROW_SHAPES = [(28, 7168, 3584), (28, 3584, 7168), (44, 9216, 4608), (60, 4608, 9216), (36, 5120, 13824),
+                    (52, 2560, 6912), (18, 13824, 5120), (62, 20480, 2560)]
+
+
 @pytest.mark.parametrize("block_scaled", [False, True])
-@pytest.mark.parametrize("M,N,K", MID_SHAPES)
+@pytest.mark.parametrize("M,N,K", MID_SHAPES + SMALL_ROW_SHAPES)
 def test_tile_cost_model_is_close_to_the_best_forced_tile(device, M, N, K, block_scaled):
     entry = tune.tune_shape(M, N, K, block_scaled, device)
     if entry["auto_us"] > 1.25 * entry["us"]:
         entry = tune.tune_shape(M, N, K, block_scaled, device)   # one more look before calling it a wrong choice
     print(f"M={M} N={N} K={K} bs={block_scaled}: auto {entry['auto_us']} us {entry['auto_schedule']}; best {entry['us']} us {entry['kernel_configs']}")
-    assert entry["auto_schedule"]["KERNEL_NAME"] == "tiled", entry
+    assert M <= 64 or entry["auto_schedule"]["KERNEL_NAME"] == "tiled", entry
     assert entry["auto_us"] <= 1.25 * entry["us"], entry

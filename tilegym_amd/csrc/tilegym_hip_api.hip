@@ -243,6 +243,29 @@ void pick_tile_by_cost(int64_t M, int64_t N, int64_t kblocks, bool block_scaled,
     if (best_bm > 0) { *bm = best_bm; *bn = best_bn; *split = best_split; }
 }
 
+// 17 .. 64 rows: the same form of model over more kinds of kernel, with constants of its own (here the weights stream from
+// HBM and a tile's step is shorter than above 64 rows; 4 000 measurements, 72 weight x row combinations x both scalings):
+// the tile kernels, the wide streaming form (to 32 rows; its "tile" is 64 weight rows x all activation rows, its K step a
+// 1 KiB piece) and the skinny kernel (cost proportional to the weight bytes x row tiles, plus a constant).  Against the
+// best forced schedule on 72 held-out combinations: 0.4 % (per-tensor) and 0.9 % (block-scaled) behind on average, worst
+// 7 % and 16 %; the rules it replaces: 7 % on average, worst 1.4 x and 1.7 x.
+struct SmallRowsCosts {
+    TileCost tiles[5];
+    int n_tiles;
+    TileCost wide;                         // bm, bn unused
+    float skinny_step, skinny_fixed;       // us per (256 workgroups x K step x row tile), us per launch
+    float reduce_us, reduce_us_per_mb;
+};
+constexpr SmallRowsCosts kSmallPerTensor = {{{32, 32, 0.133f, 0.324f, 3.66f}, {64, 32, 0.167f, 0.426f, 3.98f}, {64, 64, 0.242f, 0.689f, 4.66f},
+                                             {64, 128, 0.457f, 1.111f, 3.44f}, {128, 128, 0.714f, 1.192f, 2.38f}}, 5,
+                                            {0, 0, 2.446f, 5.599f, 3.54f}, 0.077f, 5.43f, 2.47f, 0.593f};
+constexpr SmallRowsCosts kSmallBlockScaled = {{{64, 128, 0.728f, 1.066f, 3.40f}, {128, 128, 0.743f, 1.235f, 3.31f}, {}, {}, {}}, 2,
+                                              {0, 0, 3.209f, 6.771f, 3.21f}, 0.102f, 5.42f, 2.47f, 0.549f};
+
+inline float rounds_cost_us(const TileCost& t, int64_t units, int64_t steps) {
+    return units <= 256 ? (float)steps * t.alone + t.fixed : (float)cdiv(units, 512) * ((float)steps * t.shared + t.fixed);
+}
+
 Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
                       const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
     Schedule s{0, -1, -1, 1, -1, -1, -1};
@@ -261,6 +284,68 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
     if (try_wide) skinny = true;
     if (!skinny && !tile_ok) return s;
     const int want_split = cfg_get(cfg, ncfg, TG_CFG_SPLIT_K);
+    auto skinny_schedule = [&]() {
+        Schedule k{2, -1, -1, 1, -1, -1, -1};
+        k.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+        int rg = cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS);
+        if (!(rg == 1 || rg == 2 || (rg == 4 && k.mt == 1))) rg = (N >= 16384 && k.mt <= 2) ? 2 : 1;
+        k.row_groups = rg;
+        const int64_t wgs = cdiv(N, 16 * rg);
+        // waves per workgroup: they split K inside the workgroup, no traffic between workgroups
+        int nw = cfg_get(cfg, ncfg, TG_CFG_WAVES);
+        if (nw != 4 && nw != 8 && nw != 16) {
+            nw = wgs * 4 >= kTargetWaves ? 4 : wgs * 8 >= kTargetWaves ? 8 : 16;
+            while (nw > 4 && kblocks < nw) nw /= 2;
+        }
+        k.waves = nw;
+        if (want_split > 1 || (want_split < 0 && wgs * nw * 2 <= kTargetWaves))
+            k.split_k = pick_split(wgs * nw, kTargetWaves, kblocks, 2 * nw, M, N, partial_bytes_avail, want_split);
+        return k;
+    };
+    // 17 .. 64 rows, nothing but (possibly) the split given by the caller: the cheapest kernel and split by the cost model
+    if (want_kernel < 0 && M > 16 && M <= 64 && tile_ok && K >= 1024 && cfg_get(cfg, ncfg, TG_CFG_BLOCK_M) <= 0 &&
+        cfg_get(cfg, ncfg, TG_CFG_BLOCK_N) <= 0 && cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS) < 0 && cfg_get(cfg, ncfg, TG_CFG_WAVES) < 0) {
+        const SmallRowsCosts& c = block_scaled ? kSmallBlockScaled : kSmallPerTensor;
+        auto reduce = [&](int split) { return split > 1 ? c.reduce_us + c.reduce_us_per_mb * (float)(M * N * 4 * split) * 1e-6f : 0.f; };
+        auto fits = [&](int split) { return split == 1 || (int64_t)split * M * N * 4 <= partial_bytes_avail; };
+        Schedule best{0, -1, -1, 1, -1, -1, -1};
+        float best_us = 0.f;
+        auto offer = [&](const Schedule& cand, float us) {
+            if (best.kernel == 0 || us < best_us) { best = cand; best_us = us; }  // (no margin against splits here: measured better)
+        };
+        for (int i = 0; i < c.n_tiles; ++i) {
+            const TileCost& t = c.tiles[i];
+            const bool mid = is_mid_tile(t.bm, t.bn);
+            if (mid && want_split > 1) continue;
+            for (int sp = 1; sp <= 8; sp *= 2) {
+                const int split = want_split > 0 ? want_split : sp;
+                if (split > 1 && (mid || kblocks / split < 4 || !fits(split))) break;
+                Schedule cand{1, t.bm, t.bn, 1, -1, -1, -1};
+                if (split > 1) cand.split_k = pick_split(cdiv(M, t.bm) * cdiv(N, t.bn), 256, kblocks, 4, M, N, partial_bytes_avail, split);
+                offer(cand, rounds_cost_us(t, cdiv(M, t.bm) * cdiv(N, t.bn) * cand.split_k, cdiv(kblocks, cand.split_k)) + reduce(cand.split_k));
+                if (want_split > 0) break;
+            }
+        }
+        if (M <= 32) {
+            const int64_t pieces = cdiv(K, 1024), wide_wgs = cdiv(N, 64);
+            static const int kWideSplits[] = {1, 2, 3, 4, 6, 8};
+            for (int sp : kWideSplits) {
+                const int split = want_split > 0 ? want_split : sp;
+                if (split > pieces || !fits(split)) break;
+                Schedule cand{3, -1, -1, 1, 4, 2, 4};
+                if (split > 1) cand.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, split);
+                offer(cand, rounds_cost_us(c.wide, wide_wgs * cand.split_k, cdiv(pieces, cand.split_k)) + reduce(cand.split_k));
+                if (want_split > 0) break;
+            }
+        }
+        // (the skinny kernel's time is the least regular of the three; it is the best only for weights of a few MB or
+        // very few weight rows, and is offered only there: 2048 x 7168 at M = 32 takes 13.5 us where the model said 9.7)
+        if (N * K <= ((int64_t)10 << 20) || N <= 1024) {
+            const Schedule cand = skinny_schedule();
+            offer(cand, (float)cdiv(N, 16) / 256.f * (float)kblocks * c.skinny_step * (float)cand.mt + c.skinny_fixed + reduce(cand.split_k));
+        }
+        return best;
+    }
     if (skinny && want_kernel != 2 && (want_kernel == 3 || K >= 1024)) {
         // weight streaming through LDS, 1 KiB of a row per load instruction
         s.kernel = 3;
@@ -321,25 +406,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         s = Schedule{0, -1, -1, 1, -1, -1, -1};  // not taken by the wide form: on to the tile kernels
         skinny = false;
     }
-    if (skinny) {
-        s.kernel = 2;
-        s.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-        int rg = cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS);
-        if (!(rg == 1 || rg == 2 || (rg == 4 && s.mt == 1))) rg = (N >= 16384 && s.mt <= 2) ? 2 : 1;
-        s.row_groups = rg;
-        const int64_t wgs = cdiv(N, 16 * rg);
-        // waves per workgroup: they split K inside the workgroup, no traffic between workgroups
-        int nw = cfg_get(cfg, ncfg, TG_CFG_WAVES);
-        if (nw != 4 && nw != 8 && nw != 16) {
-            nw = wgs * 4 >= kTargetWaves ? 4 : wgs * 8 >= kTargetWaves ? 8 : 16;
-            while (nw > 4 && kblocks < nw) nw /= 2;
-        }
-        s.waves = nw;
-        s.split_k = 1;
-        if (want_split > 1 || (want_split < 0 && wgs * nw * 2 <= kTargetWaves))
-            s.split_k = pick_split(wgs * nw, kTargetWaves, kblocks, 2 * nw, M, N, partial_bytes_avail, want_split);
-        return s;
-    }
+    if (skinny) return skinny_schedule();
     s.kernel = 1;
     int bm = cfg_get(cfg, ncfg, TG_CFG_BLOCK_M), bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
     if (!(bm > 0 && bn > 0 && tile_exists(bm, bn, block_scaled))) bm = bn = -1;
