@@ -346,6 +346,10 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         }
         return best;
     }
+    const bool nothing_forced = want_kernel < 0 && want_split < 0 && cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS) < 0 && cfg_get(cfg, ncfg, TG_CFG_WAVES) < 0;
+    // up to four rows against a weight of a few MB: the skinny kernel (no LDS, no barrier) is 4 - 19 % ahead of the
+    // streaming one (2048 x 2048 block-scaled at M = 1: 4.17 against 4.94 us; per-tensor 4.21 against 4.53)
+    if (nothing_forced && M <= 4 && N * K <= ((int64_t)5 << 20)) return skinny_schedule();
     if (skinny && want_kernel != 2 && (want_kernel == 3 || K >= 1024)) {
         // weight streaming through LDS, 1 KiB of a row per load instruction
         s.kernel = 3;
@@ -379,6 +383,22 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // splits; at M = 8 it is 14.4 against 13.4, and with fewer or more workgroups than compute units it loses by
         // 20 - 35 %: 5120 x 12288, 2048 x 32768)
         const int want_waves = cfg_get(cfg, ncfg, TG_CFG_WAVES);
+        // Long K over fewer 16-row workgroups than compute units, the weight too small for the rule above: four waves per
+        // workgroup leave the chip idle.  From 112 workgroups on and up to eight rows, eight waves split K inside the workgroup
+        // (3072 x 8192 at M = 1: 7.4 us against 8.4; 2048 x 7168: 6.4 against 7.4); else the wide form with up to eight
+        // splits (1024 x 16384: 8.3 - 9.1 us against 10.0 - 11.8; 1280 x 8192 at M = 16: 7.7 against 9.1).
+        const bool short_of_workgroups = nothing_forced && M <= 16 && !wide_auto && pieces >= 7 && wgs < 224;
+        if (short_of_workgroups && wgs >= 112 && M <= 8) {
+            s.waves = 8;
+            return s;
+        }
+        if (short_of_workgroups) {
+            s.row_groups = 4;
+            s.waves = (K % 128) != 0 ? 1 : 4;
+            const int64_t want = wide_split < 8 ? wide_split : 8;
+            if (want > 1) s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, (int)want);
+            return s;
+        }
         if (want_rg != 4 && want_split <= 1 && ((want_waves == 8 && M <= 16) || (want_waves < 0 && want_rg < 0 && M <= 2 && pieces >= 8 && wgs >= 224 && wgs <= 256))) {
             s.waves = 8;
             return s;
