@@ -484,6 +484,46 @@ def test_stream_wide_two_row_tiles(device, M, N, K, split):
           what=f"block-scaled stream wide, two row tiles M={M} N={N} K={K}")
 
 
+def _random_shapes(count, seed):
+    """Seeded shapes across the regimes of the automatic choice: rows log-uniform in 1 .. 700, weight rows multiples of 16
+    up to 6000, K a multiple of 128 (three in four) or of 16; the CPU oracle's work is capped at 2 GFLOP per shape."""
+    g = _g(seed)
+    out = []
+    while len(out) < count:
+        M = int(round(math.exp(float(torch.rand(1, generator=g)) * math.log(700.0))))
+        N = 16 * int(torch.randint(1, 376, (1,), generator=g))
+        K = 128 * int(torch.randint(1, 72, (1,), generator=g)) if float(torch.rand(1, generator=g)) < 0.75 else 16 * int(torch.randint(8, 500, (1,), generator=g))
+        if M * N * K <= 1_000_000_000:
+            out.append((M, N, K))
+    return out
+
+
+@pytest.mark.parametrize("block_scaled", [False, True])
+def test_automatic_schedules_on_random_shapes(device, block_scaled):
+    """Whatever kernel, tile and split the library picks by itself (fixed rules to 16 rows, cost models above), the whole
+    output matches the oracle: 70 seeded shapes per scaling, and every kind of kernel must have been met on the way."""
+    seen = set()
+    for M, N, K in _random_shapes(70, 2024 + block_scaled):
+        g = _g(M * 31 + N * 7 + K)
+        a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
+        if block_scaled:
+            sa = torch.rand(M, -(-K // 128), generator=g) * 0.05 + 0.01
+            sb = torch.rand(-(-N // 128), -(-K // 128), generator=g) * 0.05 + 0.01
+            ref = R.ref_w8a8_block_fp8_matmul(a, b, sa, sb, [128, 128], torch.bfloat16)
+            out = w8a8_block_fp8_matmul(a.to(device), b.to(device), sa.to(device), sb.to(device), [128, 128], torch.bfloat16)
+        else:
+            ref = R.ref_gemm_per_tensor(a, b, 0.03, 0.02, trans_b=True)
+            out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.03, scale_b=0.02, out_dtype=torch.bfloat16)
+        cfg = _lib.last_config()
+        seen.add((cfg["KERNEL_NAME"], cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["SPLIT_K"] > 1, cfg["ROW_GROUPS"], cfg["WAVES"]))
+        if cfg["KERNEL_NAME"] == "fallback":   # the MFMA tile kernels step through K in whole 128-byte blocks
+            assert M > 64 and K % 128 != 0, (M, N, K, cfg)
+        check(out, ref, what=f"automatic schedule {cfg} for {M}x{N}x{K} block_scaled={block_scaled}")
+    kernels = {k[0] for k in seen}
+    assert {"tiled", "stream", "skinny"} <= kernels, seen
+    assert len({k[1:3] for k in seen if k[0] == "tiled"}) >= (2 if block_scaled else 3) and any(k[3] for k in seen), seen
+
+
 def test_kernel_choice_at_32_rows_follows_the_cost_model(device):
     """17 .. 64 rows: the cheapest of tile kernels, wide streaming form and skinny kernel by the fitted cost model.
     16384 x 1024 at M = 32 streams (256 workgroups, one 1 KiB piece each); 4096 x 14336 takes 64 x 128 tiles with eight
