@@ -100,10 +100,13 @@ enum {
  *        C[m,n] = sum_kb scale_a[m,kb] * scale_b[n/128,kb] * sum_{k in kb} A[m,k] * B[n,k]
  *     (both must be of the same kind; block form requires the NT layout.)
  * workspace: NULL, or a 16-byte-aligned scratch buffer (any dtype, contents irrelevant) of at
- *     least tg_fp8_gemm_workspace_bytes() bytes.  It holds split-K partial sums and, for
- *     (K,N) weights, a K-contiguous copy of b.  Calls that share a workspace must not overlap
- *     in time (calls on one stream never do).  Without a workspace the split-K schedules and
- *     the (K,N) fast path are not used.
+ *     least tg_fp8_gemm_workspace_bytes() bytes.  It holds split-K partial sums, for
+ *     (K,N) weights a K-contiguous copy of b, and for a K that the MFMA kernels cannot step
+ *     through (K % 16 != 0; K % 128 != 0 above 64 rows) copies of a and b with every row
+ *     zero-padded to the next multiple of 128.  Calls that share a workspace must not overlap
+ *     in time (calls on one stream never do).  Without a workspace the split-K schedules, the
+ *     (K,N) fast path and the padded copies are not used (such a K then runs on the fallback
+ *     kernel).
  */
 int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
                     const tg_tensor* scale_a, const tg_tensor* scale_b, int32_t trans_a,
@@ -129,8 +132,9 @@ int32_t tg_fp8_gemm_static_scratch(const tg_tensor* c, const tg_tensor* a, const
                                    int32_t device_id, uint64_t hip_stream);
 
 /* Bytes of workspace that let tg_fp8_gemm use every schedule for this problem
- * (trans_b == 0 adds room for a K-contiguous copy of B).  Never fails; returns 0 for
- * non-positive sizes. */
+ * (trans_b == 0 adds room for a K-contiguous copy of B; a K that is no multiple of 16, or
+ * no multiple of 128 above 64 rows, adds room for zero-padded copies of both operands).
+ * Never fails; returns 0 for non-positive sizes. */
 int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t trans_b,
                                     const int32_t* cfg, int32_t ncfg);
 

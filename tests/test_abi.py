@@ -154,6 +154,18 @@ def test_moe_gemm_silu_quant_argument_validation():
     assert not _lib.moe_gemm_silu_quant_ok(torch.zeros(E, 2 * 200, K), 256)
 
 
+def test_workspace_bytes_count_the_room_for_zero_padded_operands():
+    """K that the MFMA kernels cannot step through (no multiple of 128 above 64 rows, no multiple of 16 anywhere) is
+    padded into the workspace: room for (M + N) rows of the padded K; none when the kernels take K as it is."""
+    L = _lib.load()
+    cfg, n = _lib.make_cfg(None)
+    for M, N, K, padded in [(200, 264, 4104, True), (200, 264, 4096, False), (16, 264, 4112, False), (16, 264, 4100, True), (65, 264, 4112, True)]:
+        got = L.tg_fp8_gemm_workspace_bytes(M, N, K, 1, cfg, n)
+        same_with_k_aligned = L.tg_fp8_gemm_workspace_bytes(M, N, -(-K // 128) * 128, 1, cfg, n)
+        kp = -(-K // 128) * 128
+        assert got - same_with_k_aligned == ((-(-M * kp // 256) * 256 + -(-N * kp // 256) * 256) if padded else 0), (M, N, K)
+
+
 def test_workspace_bytes_count_the_room_for_coarse_block_scales():
     """Quantization blocks that are multiples of 128 x 128 need room to write the scales out per 128 x 128 block."""
     L = _lib.load()

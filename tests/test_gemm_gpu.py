@@ -244,7 +244,7 @@ def test_block_scaled_quantization_blocks_other_than_128(device, block_size, M, 
     ref = R.ref_w8a8_block_fp8_matmul(A, B, As, Bs, block_size, torch.bfloat16)
     out = w8a8_block_fp8_matmul(A.to(device), B.to(device), As.to(device), Bs.to(device), block_size, torch.bfloat16)
     cfg = _lib.last_config()
-    if bn % 128 == 0 and bk % 128 == 0 and K % 128 == 0:
+    if bn % 128 == 0 and bk % 128 == 0:   # (K = 328 runs zero-padded to 384)
         assert cfg["KERNEL_NAME"] in ("tiled", "stream", "skinny") and (cfg["QUANT_BLOCK_N"], cfg["QUANT_BLOCK_K"]) == (bn, bk), cfg
     else:
         assert cfg["KERNEL_NAME"] == "fallback", cfg
@@ -339,12 +339,12 @@ def test_rows_split_where_256_tiles_leave_the_last_round_mostly_empty(device, bl
 
 
 def test_fallback_kernel_takes_more_rows_than_one_grid_dimension_holds(device):
-    """The software-decode kernel walks rows grid-stride: 300 000 rows (above 4 x 65 535) of a K that no fast kernel
-    takes (K % 16 != 0)."""
+    """The software-decode kernel walks rows grid-stride: 300 000 rows (above 4 x 65 535)."""
     M, N, K = 300_000, 8, 24
     g = _g(78)
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
-    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.5, scale_b=0.25, out_dtype=torch.bfloat16)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.5, scale_b=0.25, out_dtype=torch.bfloat16,
+                 kernel_configs={"KERNEL": "fallback"})
     used("fallback")
     rows = torch.tensor([0, 1, 262139, 262140, 262143, 262144, 299_999] + torch.randint(0, M, (200,), generator=g).tolist())
     check(out[rows.to(device)], R.ref_gemm_per_tensor(a[rows], b, 0.5, 0.25, trans_b=True), what="fallback, 300000 rows")
@@ -516,8 +516,7 @@ def test_automatic_schedules_on_random_shapes(device, block_scaled):
             out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.03, scale_b=0.02, out_dtype=torch.bfloat16)
         cfg = _lib.last_config()
         seen.add((cfg["KERNEL_NAME"], cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["SPLIT_K"] > 1, cfg["ROW_GROUPS"], cfg["WAVES"]))
-        if cfg["KERNEL_NAME"] == "fallback":   # the MFMA tile kernels step through K in whole 128-byte blocks
-            assert M > 64 and K % 128 != 0, (M, N, K, cfg)
+        assert cfg["KERNEL_NAME"] != "fallback", (M, N, K, cfg)   # (a K tail runs zero-padded through the workspace)
         check(out, ref, what=f"automatic schedule {cfg} for {M}x{N}x{K} block_scaled={block_scaled}")
     kernels = {k[0] for k in seen}
     assert {"tiled", "stream", "skinny"} <= kernels, seen
@@ -588,15 +587,37 @@ def test_all_four_layouts_agree_with_the_oracle(device):
     used("fallback")
 
 
-@pytest.mark.parametrize("M,N,K", [(32, 64, 1023), (130, 70, 200), (5, 33, 17)])
-def test_odd_k_uses_the_fallback_and_is_correct(device, M, N, K):
-    """K=1023 is the case the reference skips (tests/ops/test_matmul.py:130-131)."""
+@pytest.mark.parametrize("trans_b", [True, False])
+@pytest.mark.parametrize("M,N,K", [(32, 64, 1023), (130, 70, 200), (5, 33, 17), (300, 520, 1040), (200, 264, 4104), (16, 4096, 1000)])
+def test_any_k_runs_on_the_mfma_kernels_through_zero_padded_copies(device, M, N, K, trans_b):
+    """K = 1023 is the case the reference skips (tests/ops/test_matmul.py:130-131).  A K that is no multiple of 16, or no
+    multiple of 128 above 64 rows, is padded with zeros into the workspace -- (K, N) weights transposed on the way -- and
+    runs on the MFMA kernels; without a workspace the software-decode kernel takes it.  Same oracle either way."""
     g = _g(K)
     a, b = fp8_randn((M, K), g), fp8_randn((N, K), g)
     ref = R.ref_gemm_per_tensor(a, b, 0.5, 2.0, trans_b=True)
-    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.5, scale_b=2.0, out_dtype=torch.bfloat16)
+    bd = b.to(device) if trans_b else b.view(torch.uint8).t().contiguous().view(FP8).to(device)
+    out = matmul(a.to(device), bd, trans_b=trans_b, scale_a=0.5, scale_b=2.0, out_dtype=torch.bfloat16)
+    assert _lib.last_config()["KERNEL_NAME"] in ("tiled", "stream", "skinny"), _lib.last_config()
+    check(out, ref, what=f"padded K={K}")
+    sa, sb = torch.tensor([0.5], device=device), torch.tensor([2.0], device=device)
+    plain = torch.empty_like(out)
+    _lib.fp8_gemm(plain, a.to(device), bd, sa, sb, False, trans_b, 1.0, 0.0, None, use_workspace=False)
     used("fallback")
-    check(out, ref, what=f"fallback K={K}")
+    check(plain, ref, what=f"fallback K={K}")
+
+
+def test_block_scaled_k_tail_above_64_rows_runs_padded(device):
+    """Block-scaled, M = 200, K = 1000: the last K block holds 104 values; padded to 1024 the scales keep their shape."""
+    M, N, K = 200, 392, 1000
+    g = _g(1000)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.5)
+    sa = torch.rand(M, 8, generator=g) * 0.05 + 0.01
+    sb = torch.rand(4, 8, generator=g) * 0.05 + 0.01
+    ref = R.ref_w8a8_block_fp8_matmul(a, b, sa, sb, [128, 128], torch.bfloat16)
+    out = w8a8_block_fp8_matmul(a.to(device), b.to(device), sa.to(device), sb.to(device), [128, 128], torch.bfloat16)
+    used("tiled")
+    check(out, ref, what="block-scaled, K = 1000")
 
 
 def test_k_tail_multiple_of_16_skinny(device):

@@ -87,9 +87,10 @@ hipError_t run_generic(const GenericParams& q, hipStream_t s) {
     return hipGetLastError();
 }
 
+// dst (cols x ld) = transpose of src (rows x cols); ld >= rows, and dst[c][rows .. ld) = 0.
 __global__ void __launch_bounds__(256) transpose_u8_kernel(const uint8_t* __restrict__ src,
                                                            uint8_t* __restrict__ dst, int rows,
-                                                           int cols) {
+                                                           int cols, int ld) {
     __shared__ uint8_t t[64][65];
     const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -100,8 +101,28 @@ __global__ void __launch_bounds__(256) transpose_u8_kernel(const uint8_t* __rest
     __syncthreads();
     for (int i = ty; i < 64; i += 4) {
         const int c = c0 + i, r = r0 + tx;
-        if (c < cols && r < rows) dst[(int64_t)c * rows + r] = t[tx][i];
+        if (c < cols && r < ld) dst[(int64_t)c * ld + r] = t[tx][i];
     }
+}
+
+// dst (rows x ld) = src (rows x cols) with dst[r][cols .. ld) = 0; ld % 16 == 0, dst 16-byte aligned.  One thread writes
+// 16 bytes; it reads them as one vector when the source rows are 16-byte aligned too (cols % 16 == 0), else byte by byte.
+__global__ void __launch_bounds__(256) pad_rows_u8_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                          int rows, int cols, int ld, int vec) {
+    const int per_row = ld / 16;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)rows * per_row) return;
+    const int r = (int)(idx / per_row), c0 = (int)(idx % per_row) * 16;
+    v4i out = v4i{0, 0, 0, 0};
+    if (vec && c0 + 16 <= cols) {
+        out = *reinterpret_cast<const v4i*>(src + (int64_t)r * cols + c0);
+    } else if (c0 < cols) {
+        uint8_t bytes[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) bytes[q] = c0 + q < cols ? src[(int64_t)r * cols + c0 + q] : (uint8_t)0;
+        __builtin_memcpy(&out, bytes, 16);
+    }
+    *reinterpret_cast<v4i*>(dst + (int64_t)r * ld + c0) = out;
 }
 
 // Second pass of the split-K schedules: one thread adds the split_k partial sums of four
@@ -165,10 +186,18 @@ hipError_t run_expand_scales(const float* in, float* out, int rows_out, int cols
     return hipGetLastError();
 }
 
-hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s) {
-    if (rows <= 0 || cols <= 0) return hipSuccess;
-    dim3 grid((cols + 63) / 64, (rows + 63) / 64, 1);
-    hipLaunchKernelGGL(transpose_u8_kernel, grid, dim3(256, 1, 1), 0, s, src, dst, rows, cols);
+hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, int ld, hipStream_t s) {
+    if (rows <= 0 || cols <= 0 || ld < rows) return hipSuccess;
+    dim3 grid((cols + 63) / 64, (ld + 63) / 64, 1);
+    hipLaunchKernelGGL(transpose_u8_kernel, grid, dim3(256, 1, 1), 0, s, src, dst, rows, cols, ld);
+    return hipGetLastError();
+}
+
+hipError_t run_pad_rows_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, int ld, hipStream_t s) {
+    if (rows <= 0 || cols <= 0 || ld < cols || (ld % 16) != 0) return hipSuccess;
+    const int64_t threads = (int64_t)rows * (ld / 16);
+    const int vec = (cols % 16) == 0 && (reinterpret_cast<uintptr_t>(src) % 16) == 0;
+    hipLaunchKernelGGL(pad_rows_u8_kernel, dim3((unsigned)((threads + 255) / 256), 1, 1), dim3(256, 1, 1), 0, s, src, dst, rows, cols, ld, vec);
     return hipGetLastError();
 }
 

@@ -73,7 +73,10 @@ hipError_t run_silu_mul_quant(const void* x, int x_type, uint8_t* q, float* scal
 // out (tokens, H) <- sum over the top_k axis of x (tokens, top_k, H); bf16/f16, H % 8 == 0
 hipError_t run_moe_sum(const void* x, void* out, int x_type, int64_t tokens, int top_k, int H, hipStream_t s);
 // dst (cols, rows) <- transpose of src (rows, cols), one byte per element
-hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, hipStream_t s);
+// dst (cols x ld) = transpose of src (rows x cols), zero beyond `rows` in every dst row
+hipError_t run_transpose_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, int ld, hipStream_t s);
+// dst (rows x ld) = src (rows x cols), zero beyond `cols` in every dst row
+hipError_t run_pad_rows_u8(const uint8_t* src, uint8_t* dst, int rows, int cols, int ld, hipStream_t s);
 // out (rows_out, cols_out) = in[r / rdiv][kb / kdiv] (in has in_cols columns): block scales of coarser blocks per 128 x 128 block
 hipError_t run_expand_scales(const float* in, float* out, int rows_out, int cols_out, int in_cols, int rdiv, int kdiv, hipStream_t s);
 

@@ -516,6 +516,15 @@ int32_t tg_last_config(int32_t* out, int32_t n) {
     return m;
 }
 
+// Bytes of the zero-padded operand copies that let a K the MFMA kernels cannot step through run on them anyway: K % 128 != 0
+// above 64 rows (the tile kernels take whole 128-byte K blocks), K % 16 != 0 at any row count (the streaming kernels take
+// 16-byte pieces).  0 when no padding is needed.
+static int64_t padded_k_bytes(int64_t M, int64_t N, int64_t K) {
+    if (K <= 0 || (K % 128) == 0 || ((K % 16) == 0 && M <= 64)) return 0;
+    const int64_t kp = cdiv(K, 128) * 128;
+    return (M * kp + 255) / 256 * 256 + (N * kp + 255) / 256 * 256;
+}
+
 int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t trans_b,
                                     const int32_t* cfg, int32_t ncfg) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
@@ -529,6 +538,7 @@ int64_t tg_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t tra
     bytes += (partial + 255) / 256 * 256;
     if (!trans_b) bytes += (N * K + 255) / 256 * 256;
     bytes += expanded_scale_bytes(M, N, K, cfg, ncfg);
+    bytes += padded_k_bytes(M, N, K);
     return bytes;
 }
 
@@ -540,6 +550,40 @@ int32_t tg_fp8_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b,
     // ...): the scales are written out per 128 x 128 block at the tail of the workspace (one small launch each) and the
     // problem runs on the MFMA kernels like any 128 x 128 one -- the same products times the same scales, added in the
     // same order.  Without a workspace that holds them, and for finer blocks, the fallback kernel takes the problem.
+    // A K that is no multiple of 128 (above 64 rows) or of 16 (any row count): both operands are copied into the tail of the
+    // workspace with their rows padded with zeros to the next multiple of 128 -- (K, N) weights are transposed on the way --
+    // and the problem runs on the MFMA kernels with the padded K: the same products plus zeros.  Block scales need no
+    // change (their last K block was already a partial one).  Without a workspace that holds the copies the fallback
+    // kernel takes the problem as before.
+    tg_tensor a_pad, b_pad, ws_pad;
+    if (a && b && c && workspace && workspace->ptr && a->ptr && b->ptr && a->ndim == 2 && b->ndim == 2 && !trans_a &&
+        a->dtype == TG_F8E4M3FN && b->dtype == TG_F8E4M3FN && contiguous(a) && contiguous(b) && cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0 &&
+        // (quantization blocks whose K extent is no multiple of 128 would count another number of blocks over the padded K)
+        (cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_K) <= 0 || cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_K) % 128 == 0)) {
+        const int64_t M = a->shape[0], K = a->shape[1], N = trans_b ? b->shape[0] : b->shape[1];
+        const int64_t need = padded_k_bytes(M, N, K), kp = cdiv(K, 128) * 128;
+        const int64_t ws_bytes = numel(workspace) * elem_size(workspace->dtype);
+        const bool shapes_ok = (trans_b ? b->shape[1] : b->shape[0]) == K && M > 0 && N > 0 && M <= INT32_MAX && N <= INT32_MAX &&
+                               kp <= INT32_MAX && aligned16(workspace->ptr);
+        if (need > 0 && shapes_ok && ws_bytes >= need) {
+            g_err[0] = 0;
+            DeviceGuard guard(device_id);
+            if (!guard.ok) return fail(TG_ERR_DEVICE, "cannot use HIP device %d", device_id);
+            hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+            uint8_t* tail = reinterpret_cast<uint8_t*>(workspace->ptr) + (ws_bytes - need) / 256 * 256;
+            uint8_t* pa = tail;
+            uint8_t* pb = tail + (M * kp + 255) / 256 * 256;
+            const hipError_t ea = tg::run_pad_rows_u8(reinterpret_cast<const uint8_t*>(a->ptr), pa, (int)M, (int)K, (int)kp, stream);
+            const hipError_t eb = trans_b ? tg::run_pad_rows_u8(reinterpret_cast<const uint8_t*>(b->ptr), pb, (int)N, (int)K, (int)kp, stream)
+                                          : tg::run_transpose_u8(reinterpret_cast<const uint8_t*>(b->ptr), pb, (int)K, (int)N, (int)kp, stream);
+            if (ea != hipSuccess || eb != hipSuccess) return fail(TG_ERR_LAUNCH, "operand padding launch failed");
+            a_pad = *a; a_pad.ptr = reinterpret_cast<uint64_t>(pa); a_pad.shape[1] = kp; a_pad.strides[0] = kp; a_pad.strides[1] = 1;
+            b_pad = *b; b_pad.ptr = reinterpret_cast<uint64_t>(pb); b_pad.shape[0] = N; b_pad.shape[1] = kp; b_pad.strides[0] = kp; b_pad.strides[1] = 1;
+            ws_pad = *workspace; ws_pad.ndim = 1; ws_pad.strides[0] = 1;
+            ws_pad.shape[0] = (int64_t)(tail - reinterpret_cast<uint8_t*>(workspace->ptr)) / elem_size(workspace->dtype);
+            a = &a_pad; b = &b_pad; workspace = &ws_pad; trans_b = 1;
+        }
+    }
     const int64_t qbn = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_N), qbk = cfg_get(cfg, ncfg, TG_CFG_QUANT_BLOCK_K);
     if (a && b && c && scale_a && scale_b && workspace && a->ndim == 2 && b->ndim == 2 && !trans_a && trans_b &&
         cfg_get(cfg, ncfg, TG_CFG_KERNEL) != 0) {
@@ -759,7 +803,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
             uint8_t* bt = ws + ws_bytes - need;
             bt = reinterpret_cast<uint8_t*>(reinterpret_cast<uintptr_t>(bt) & ~(uintptr_t)15);
             if (bt >= ws_cursor) {
-                if (tg::run_transpose_u8(Bnt, bt, (int)K, (int)N, stream) != hipSuccess)
+                if (tg::run_transpose_u8(Bnt, bt, (int)K, (int)N, (int)K, stream) != hipSuccess)
                     return fail(TG_ERR_LAUNCH, "transpose launch failed");
                 Bnt = bt;
                 b_is_nk = true;
