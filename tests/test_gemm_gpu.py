@@ -484,6 +484,44 @@ def test_stream_wide_two_row_tiles(device, M, N, K, split):
           what=f"block-scaled stream wide, two row tiles M={M} N={N} K={K}")
 
 
+@pytest.mark.parametrize("bn", [56, 48, 40, 24, 12])
+@pytest.mark.parametrize("M,N,K,split", [(5, 1000, 1024, 1), (16, 1000, 1152, 1), (30, 520, 2048, 2), (16, 4096, 640, 1)])
+def test_stream_wide_with_fewer_rows_per_workgroup(device, bn, M, N, K, split):
+    """BLOCK_N of the wide streaming form: 4 x the weight rows a wave owns (64 by default).  Rows a wave does not own are
+    neither loaded nor stored; with block scales a wave's rows may lie on both sides of a 128-row boundary of the weight
+    scales (bn = 56, 48, 40, 24: rows 112 .. 139 etc.) and every output takes the scale of its own block.  N that is no
+    multiple of bn, one and two tiles of activation rows, a short last piece, split-K."""
+    g = _g(bn * 11 + M + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    sa, sb = torch.tensor([0.011]), torch.tensor([0.0003])
+    kc = {"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": split, "BLOCK_N": bn}
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=sa.to(device), scale_b=sb.to(device),
+                 out_dtype=torch.bfloat16, kernel_configs=kc)
+    cfg = used("stream")
+    assert (cfg["ROW_GROUPS"], cfg["SPLIT_K"], cfg["WAVES"], cfg["BLOCK_N"]) == (4, split, 4, bn), cfg
+    check(out, R.ref_gemm_per_tensor(a, b, sa, sb, trans_b=True), what=f"stream wide, {bn} rows per workgroup, M={M} N={N} K={K}")
+    case = W.block_scaled_case(M, N, K, seed=M + N + bn)
+    d = case.to(device)
+    out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs=kc)
+    cfg = used("stream")
+    assert (cfg["ROW_GROUPS"], cfg["SPLIT_K"], cfg["BLOCK_N"]) == (4, split, bn), cfg
+    check(out, R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16),
+          what=f"block-scaled stream wide, {bn} rows per workgroup, M={M} N={N} K={K}")
+
+
+def test_stream_wide_picks_its_rows_per_workgroup(device):
+    """12288 weight rows in workgroups of 48 are one workgroup per compute unit (64: 192 workgroups, a quarter of the chip
+    idle); 8192 x 8192 takes 32 rows per workgroup in one launch instead of 64 and two K splits."""
+    g = _g(4848)
+    for N, K, bn in [(12288, 1024, 48), (8192, 8192, 32)]:
+        a, b = fp8_randn((16, K), g), fp8_randn((N, K), g, 0.02)
+        out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
+        cfg = used("stream")
+        assert (cfg["ROW_GROUPS"], cfg["SPLIT_K"], cfg["BLOCK_N"]) == (4, 1, bn), cfg
+        rows = torch.arange(0, N, 37)
+        check(out[:, rows.to(device)], R.ref_gemm_per_tensor(a, b[rows], 0.01, 0.02, trans_b=True), what=f"{N} x {K}, rows per workgroup")
+
+
 def _random_shapes(count, seed):
     """Seeded shapes across the regimes of the automatic choice: rows log-uniform in 1 .. 700, weight rows multiples of 16
     up to 6000, K a multiple of 128 (three in four) or of 16; the CPU oracle's work is capped at 2 GFLOP per shape."""

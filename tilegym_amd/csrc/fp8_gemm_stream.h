@@ -374,6 +374,20 @@ __device__ __forceinline__ float stream_uniform_f32(const float* p) {
 // compute unit).
 // MT tiles of 16 activation rows (M <= 16 MT): the activation piece in LDS grows to 16 MT rows, every wave multiplies
 // its weight fragments with all of them.  Built for MT = 1 and 2; MT = 4 works and is slower than the tile kernels.
+// The wide kernel's LDS table of activation scales: none at all for per-tensor scales, so that the per-tensor kernel's
+// 64 + 16 KiB of buffers are exactly half of a compute unit's 160 KiB and two workgroups share one.
+template <bool BLOCKSCALE, int FLOATS>
+struct StreamScaleTable {
+    __device__ static __forceinline__ float* get() {
+        __shared__ __align__(16) float table[FLOATS];
+        return table;
+    }
+};
+template <int FLOATS>
+struct StreamScaleTable<false, FLOATS> {
+    __device__ static __forceinline__ float* get() { return nullptr; }
+};
+
 template <bool BLOCKSCALE, int MT>
 __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -388,15 +402,20 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
     // block scales: every wave's own copy of the piece's 16 MT rows x 4 steps of activation scales, fetched by MT more direct
     // loads of the piece so that they are counted by the same vmcnt wait.  (An ordinary load here would make the compiler
     // wait for vmcnt(0) before its first use, i.e. for the next piece's loads as well: no overlap left.)
-    __shared__ __align__(16) float sS[BLOCKSCALE ? NW * 2 * MT * 64 : 4];
+    float* const sS = StreamScaleTable<BLOCKSCALE, NW * 2 * MT * 64>::get();
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int K = p.K, N = p.N, M = p.M;
-    const int n_base = blockIdx.x * (16 * NW) + wave * 16;
+    // weight rows per wave: 16, or fewer so that the workgroups (4 R rows each) come out as a whole number per compute unit
+    // (28672 rows: 448 workgroups of 64 rows are 1.75 per compute unit, 512 of 56 rows are two).  The rows a wave does
+    // not own are loaded from beyond the descriptor's range (no memory request, zeros) and never stored.
+    const int R = p.wave_rows > 0 ? p.wave_rows : 16;
+    const int n_base = (blockIdx.x * NW + wave) * R;
     const int npieces = (K + PIECE - 1) / PIECE;
     const int tail_steps = (K % PIECE) / kKBlock;  // K steps of the last piece when K is no multiple of 512 (0: every piece is whole)
+    constexpr uint32_t kOutOfRange = 0x80000000u;  // >= the descriptor's 2^31 - 1 bytes
     int c_begin = 0, c_end = npieces;
     if (p.split_k > 1) {  // ksteps_per_split counts 1 KiB of K: two pieces
         c_begin = blockIdx.y * p.ksteps_per_split * 2;
@@ -415,9 +434,10 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int r = 2 * i + half, chunk = pos ^ r;
+        const bool mine = r < R && n_base + r < N;
         const uint32_t row = (uint32_t)min(n_base + r, N - 1) * (uint32_t)K;
-        w_off[i] = row + (uint32_t)(chunk << 4);
-        w_tail[i] = row + (uint32_t)((chunk < tail_steps * 8 ? chunk : 0) << 4);
+        w_off[i] = mine ? row + (uint32_t)(chunk << 4) : kOutOfRange;
+        w_tail[i] = mine ? row + (uint32_t)((chunk < tail_steps * 8 ? chunk : 0) << 4) : kOutOfRange;
     }
     // wave w issues loads w, w + 4, w + 8, ... of the activation piece
 #pragma unroll
@@ -430,6 +450,12 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
     // lane l of scale load mt: activation row 16 mt + l / 4, K step l % 4 of the piece
     const bool has_as = BLOCKSCALE && p.As != nullptr;
     const float* bs_ptr = BLOCKSCALE && p.Bs ? p.Bs + (int64_t)min(n_base / 128, p.nblocks - 1) * p.kblocks : nullptr;
+    // with fewer than 16 rows per wave its rows may lie on both sides of a 128-row boundary of the weight scales: the scales of
+    // the next block row are fetched as well (scalar loads), and every lane picks per output which of the two is its own
+    const float* bs_ptr2 = BLOCKSCALE && p.Bs ? p.Bs + (int64_t)min(n_base / 128 + 1, p.nblocks - 1) * p.kblocks : nullptr;
+    bool next_block[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) next_block[q] = BLOCKSCALE && (n_base + lg * 4 + q) / 128 != n_base / 128;
     const v4i rsrc_as = make_rsrc(p.As);
     const uint32_t s_lds = lds_address(sS) + (BLOCKSCALE ? wave * (2 * MT * 256) : 0);
     uint32_t as_off[MT], as_tail[MT];
@@ -483,10 +509,13 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
         const int c = piece(it);
         const int buf = it & 1;
         const int steps = (tail_steps != 0 && c == npieces - 1) ? tail_steps : SPC;
-        float bsc[BLOCKSCALE ? SPC : 1];
+        float bsc[BLOCKSCALE ? SPC : 1], bsc2[BLOCKSCALE ? SPC : 1];
         if constexpr (BLOCKSCALE) {  // the weight scales are the same in every lane: scalar loads, not counted by vmcnt
 #pragma unroll
-            for (int s = 0; s < SPC; ++s) bsc[s] = bs_ptr ? stream_uniform_f32(bs_ptr + min(c * SPC + s, p.kblocks - 1)) : 1.0f;
+            for (int s = 0; s < SPC; ++s) {
+                bsc[s] = bs_ptr ? stream_uniform_f32(bs_ptr + min(c * SPC + s, p.kblocks - 1)) : 1.0f;
+                bsc2[s] = bs_ptr2 ? stream_uniform_f32(bs_ptr2 + min(c * SPC + s, p.kblocks - 1)) : 1.0f;
+            }
         }
         // my loads of piece c have landed (those of piece c+1 may be in flight) ...
         if (it + 1 >= n_pieces) __builtin_amdgcn_s_waitcnt(kWaitAll);
@@ -529,13 +558,21 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 if (s >= steps) continue;
-                if constexpr (BLOCKSCALE) acc[mt] += mfma_e4m3(wf[s], af[mt][s], v4f{0.f, 0.f, 0.f, 0.f}) * (as4[mt][s] * bsc[s]);
-                else acc[mt] = mfma_e4m3(wf[s], af[mt][s], acc[mt]);
+                if constexpr (BLOCKSCALE) {
+                    // (the same product of the two scales as with one scale per wave, then one multiply-add per output)
+                    const float lo = as4[mt][s] * bsc[s], hi = as4[mt][s] * bsc2[s];
+                    const v4f sc = v4f{next_block[0] ? hi : lo, next_block[1] ? hi : lo, next_block[2] ? hi : lo, next_block[3] ? hi : lo};
+                    acc[mt] += mfma_e4m3(wf[s], af[mt][s], v4f{0.f, 0.f, 0.f, 0.f}) * sc;
+                } else {
+                    acc[mt] = mfma_e4m3(wf[s], af[mt][s], acc[mt]);
+                }
             }
         }
     }
-    const bool vec_ok = p.vec_store != 0;
+    // a lane holds four consecutive weight rows' results: all of them, or (R % 4 != 0) only the first R - 4 lg, are the wave's
+    const bool vec_ok = p.vec_store != 0 && (R & 3) == 0;
     const int col = n_base + lg * 4;
+    const int n_end = min(n_base + R, N);  // (store4 writes single elements up to its N argument when four would pass it)
     float scale = p.alpha;
     if constexpr (!BLOCKSCALE) {
         if (p.As) scale *= p.As[0];
@@ -544,17 +581,17 @@ __global__ void __launch_bounds__(256) fp8_gemm_stream_wide_db_kernel(const Gemm
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + li;
-        if (m >= M || col >= N) continue;
-        if (p.split_k > 1) store4(p.partials + (int64_t)blockIdx.y * M * N, OUT_F32, m, col, N, N, acc[mt], 0.f, vec_ok);
-        else store4(p.C, p.out_type, m, col, N, p.ldc, acc[mt] * scale, p.beta, vec_ok);
+        if (m >= M || col >= n_end) continue;
+        if (p.split_k > 1) store4(p.partials + (int64_t)blockIdx.y * M * N, OUT_F32, m, col, n_end, N, acc[mt], 0.f, vec_ok);
+        else store4(p.C, p.out_type, m, col, n_end, p.ldc, acc[mt] * scale, p.beta, vec_ok);
     }
 #endif
 }
 
-// grid_x = ceil(N / 64); M <= 16 MT
+// grid_x = ceil(N / (4 R)) with R = p.wave_rows weight rows per wave (0: 16); M <= 16 MT
 template <bool BLOCKSCALE, int MT>
 inline hipError_t launch_stream_wide_db(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
-    if (p.K % kKBlock != 0 || p.K <= 0 || p.M > 16 * MT) return hipErrorInvalidValue;
+    if (p.K % kKBlock != 0 || p.K <= 0 || p.M > 16 * MT || p.wave_rows < 0 || p.wave_rows > 16) return hipErrorInvalidValue;
     hipLaunchKernelGGL((fp8_gemm_stream_wide_db_kernel<BLOCKSCALE, MT>), dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
     return hipGetLastError();
 }

@@ -19,13 +19,14 @@ hipError_t run_stream(int mt, int nbuf, int waves, bool bs, const GemmParams& p,
 hipError_t run_stream_ragged(const GemmParams& p, hipStream_t s) { return launch_stream_ragged(p, s); }
 
 hipError_t run_stream_wide(bool bs, const GemmParams& p, int gy, hipStream_t s, bool two_buffers, int mt) {
-    const int gx = (p.N + 63) / 64;
+    int gx = (p.N + 63) / 64;
     if (two_buffers && p.K % 128 == 0) {
+        if (p.wave_rows > 0) gx = (p.N + 4 * p.wave_rows - 1) / (4 * p.wave_rows);
         if (mt == 1) return bs ? launch_stream_wide_db<true, 1>(p, gx, gy, s) : launch_stream_wide_db<false, 1>(p, gx, gy, s);
         if (mt == 2) return bs ? launch_stream_wide_db<true, 2>(p, gx, gy, s) : launch_stream_wide_db<false, 2>(p, gx, gy, s);
         return hipErrorInvalidConfiguration;
     }
-    if (mt != 1) return hipErrorInvalidConfiguration;
+    if (mt != 1 || (p.wave_rows != 0 && p.wave_rows != 16)) return hipErrorInvalidConfiguration;
     return bs ? launch_stream_wide<true>(p, gx, gy, s) : launch_stream_wide<false>(p, gx, gy, s);
 }
 

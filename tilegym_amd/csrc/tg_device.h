@@ -52,6 +52,8 @@ struct GemmParams {
     int inter;
     float* act_scales;
     int act_is_bf16;
+    // wide streaming form: weight rows per wave (1 .. 16; 0 means 16).  Fewer than 16 make more, smaller workgroups
+    int wave_rows;
 };
 
 // A list of independent per-tensor-scaled NT GEMMs handed to one launch in the kernel arguments.

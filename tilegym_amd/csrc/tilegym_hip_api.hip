@@ -367,7 +367,7 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // compute unit (4096 x 14336, 64 row blocks, M = 1: 22.3 / 16.0 / 13.0 / 14.2 us with 1 / 2 / 4 / 7 splits;
         // 6144 x 8192, 96 row blocks: 14.7 / 12.2 / 12.9 with 1 / 2 / 4) -- counts between one and two per compute unit
         // leave some compute units with twice the work of the others.
-        int64_t wide_split = wide_wgs >= 136 ? 1 : 256 / wide_wgs;
+        int64_t wide_split = wide_wgs >= 136 ? 1 : 256 / wide_wgs;  // (may be set to 1 below)
         if (wide_split > pieces) wide_split = pieces;
         if (wide_split > 16) wide_split = 16;
         if (wide_wgs >= 112 && pieces < 6) wide_split = 1;  // (8192 x 3072 at M = 16: 7.9 us unsplit, 9.5 with two splits)
@@ -376,8 +376,33 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
         // eight rows where every narrow workgroup's own activation loads weigh more (6144 x 4096 at M = 16: 9.3 against
         // 9.6; 1536 x 24576: 10.4 - 11.9 against 13.5 - 19.4).  One to four rows over 96 - 135 row blocks stay narrow: its
         // 384 - 540 workgroups fill the chip without a reduction (8192 x 8192 at M = 1: 13.6 against 15.7).
-        const bool wide_auto = N >= 16384 || (wide_wgs >= 136 && K >= 2048) ||
-                               (N * K >= ((int64_t)(M > 8 || pieces >= 12 ? 24 : 32) << 20) && wide_wgs * wide_split >= 176 && !(M <= 4 && wide_wgs >= 96));
+        bool wide_auto = N >= 16384 || (wide_wgs >= 136 && K >= 2048) ||
+                         (N * K >= ((int64_t)(M > 8 || pieces >= 12 ? 24 : 32) << 20) && wide_wgs * wide_split >= 176 && !(M <= 4 && wide_wgs >= 96));
+        // Weight rows per workgroup of the two-piece wide form.  64 rows leave compute units idle when N / 64 is well below 256 or a little above it; fewer rows per
+        // workgroup fill the chip in one launch where split-K needed a second one.  Cost of a choice ~ rounds of 256
+        // workgroups x (rows + 16): 12288 x 5120 at M = 16 takes 12.6 us with 48 rows (256 workgroups) against 13.2 with
+        // 64 (192); 22016 x 4096: 17.3 (48 rows) against 19.9; 8192 x 8192: 13.9 (32 rows, unsplit) against 16.3 (64 rows,
+        // two splits); 6144 x 4096: 8.4 (24 rows) against 10.0.  Long K (more than eight 1 KiB pieces) stays with 64 rows
+        // and split-K: a workgroup walks its pieces one round trip after the other (4096 x 14336: 14.4 us with four
+        // splits, 19.8 unsplit with 24 rows).
+        int wide_bn = 64;
+        const bool rows_free = (K % 128) == 0 && cfg_get(cfg, ncfg, TG_CFG_BLOCK_N) <= 0 && cfg_get(cfg, ncfg, TG_CFG_WAVES) != 1;
+        if (rows_free && M <= 16 && (pieces <= 8 || wide_split == 1) && want_split <= 1) {
+            int64_t best_cost = 0;
+            int best_bn = 64;
+            for (int bn = 64; bn >= 24; bn -= 8) {
+                const int64_t cost = cdiv(cdiv(N, bn), 256) * (bn + 16);
+                if (bn == 64 || cost < best_cost) { best_cost = cost; best_bn = bn; }
+            }
+            // (too few weight rows to fill the chip even with 24 per workgroup: 64 rows and split-K as before)
+            if (cdiv(N, best_bn) >= 200) {
+                wide_bn = best_bn;
+                if (pieces <= 8) wide_split = 1;
+                // with its workgroups filling the chip the wide form also wins at nine rows and more over smaller weights
+                // (8192 x 3072 at M = 16: 7.3 against 8.0 us; 5120 x 5120: 9.4 against 11.9)
+                if (M > 8 && pieces <= 8) wide_auto = true;
+            }
+        }
         // long K over one 16-row workgroup per compute unit, one or two activation rows: eight waves split K inside the
         // workgroup, one launch, no partial sums (4096 x 14336: 12.6 us at M = 1 against 13.0 for the wide form with four
         // splits; at M = 8 it is 14.4 against 13.4, and with fewer or more workgroups than compute units it loses by
@@ -413,6 +438,10 @@ Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool f
             // K % 128 == 0: the form with two half pieces per wave in flight (reported as WAVES = 4); else, or with
             // WAVES = 1, one 1 KiB piece per wave (reported as WAVES = 1)
             s.waves = (K % 128) != 0 || (want_waves == 1 && M <= 16) ? 1 : 4;
+            // weight rows per workgroup of the two-piece form (BLOCK_N = 64, 56, ... 16: 4 x the rows per wave)
+            const int want_bn = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
+            if (s.waves == 4 && want_bn >= 4 && want_bn <= 64 && want_bn % 4 == 0) s.bn = want_bn;
+            else if (s.waves == 4 && M <= 16 && wide_bn != 64) s.bn = wide_bn;
             if (want_split > 1) s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, want_split);
             else if (want_split < 0 && wide_split > 1)
                 s.split_k = pick_split(wide_wgs, 512, pieces, 1, M, N, partial_bytes_avail, (int)wide_split);
@@ -873,6 +902,7 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         // one workgroup, except for long K where they tie
         if (nbuf != 1 && nbuf != 2) nbuf = (per_wave >= 3 && s.mt == 1 && !block_scaled) ? 2 : 1;
         if (s.mt != 1 || s.waves == 8) nbuf = 1;
+        if (s.row_groups == 4 && s.waves == 4 && s.bn > 0) p.wave_rows = s.bn / 4;
         hipError_t e = s.row_groups == 4 ? tg::run_stream_wide(block_scaled, p, s.split_k, stream, s.waves == 4, s.mt)
                                          : tg::run_stream(s.mt, nbuf, s.waves, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "stream kernel launch failed: %s", hipGetErrorString(e));

@@ -32,6 +32,8 @@ def candidates(M: int, N: int, K: int, block_scaled: bool) -> List[dict]:
     out: List[dict] = []
     if M <= 32:
         out += [{"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": s} for s in (1, 2, 3, 4, 6, 8)]
+        # fewer weight rows per workgroup of the wide form
+        out += [{"KERNEL": "stream", "ROW_GROUPS": 4, "SPLIT_K": s, "BLOCK_N": bn} for bn in (56, 48, 40, 32, 24) for s in (1, 2)]
     if M <= 16:
         out += [{"KERNEL": "stream", "ROW_GROUPS": 1, "SPLIT_K": 1, "WAVES": 4}, {"KERNEL": "stream", "WAVES": 8}]
     if M <= 64:
