@@ -69,7 +69,7 @@ enum {
                             * tiled 256x256 block-scaled kernels (dense and ragged): 1 = the persistent form (one workgroup per
                             * compute unit walks the tiles, three weight slabs in LDS, scales in registers); the ragged GEMM
                             * chooses it by itself for K <= 1536 */
-    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup, and with ROW_GROUPS = 4 (the wide form) 1 = one 1 KiB piece per wave in flight instead of two half pieces; tiled 256x256 kernels: 8 = the generic eight-wave tile kernel (one workgroup per tile) instead of the persistent one */
+    TG_CFG_WAVES = 5,   /* skinny kernel: waves per workgroup splitting K (4/8/16); stream kernel: 8 = eight waves split K inside a 16-row workgroup, and with ROW_GROUPS = 4 (the wide form) 1 = one 1 KiB piece per wave in flight instead of two half pieces; tiled 256x256 kernels: 8 = the generic eight-wave tile kernel (one workgroup per tile) instead of the persistent one; ragged GEMM, streaming form: 4 / 6 / 8 waves (64 / 96 / 128 weight rows) per workgroup */
     TG_CFG_QUANT_BLOCK_N = 6, /* block-scaled tg_fp8_gemm: weight rows per scale (default 128) */
     TG_CFG_QUANT_BLOCK_K = 7, /* block-scaled tg_fp8_gemm: K elements per scale (default 128): the reference's
                                * block_size=[bn, bk] argument, src/tilegym/suites/unsloth/cutile/fp8.py:388-446.  Blocks that

@@ -1627,26 +1627,32 @@ def _moe_base(which):
 def test_ragged_stream_form(device, T, E, H, I, k, which):
     """The streaming ragged kernel (one grid row per expert) forced at several row counts: empty experts, experts with more
     than 16 rows (several passes over their weights), K of 1 .. 3 steps past a multiple of 512 (the short last piece), N that
-    is no multiple of 64, against per-expert oracle GEMMs; untouched rows of the output do not exist."""
+    is no multiple of 64, against per-expert oracle GEMMs; untouched rows of the output do not exist.  With four, six
+    and eight waves (64 .. 128 weight rows) per workgroup."""
     base = W.moe_grouped_case(which, tokens=max(T, 8), experts=E, hidden=H, inter=I, top_k=k)
     case = W.moe_decode_case(base, T)
     d = case.to(device)
-    out = torch.full((case.a.shape[0], case.b.shape[1]), 7.0, dtype=torch.bfloat16, device=device)
-    _lib.fp8_ragged_gemm(out, d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, {"KERNEL": "stream"})
-    cfg = used("stream")
-    assert cfg["ROW_GROUPS"] == 4, cfg
-    for e in range(E):
-        lo, hi = int(case.m_indptr[e]), int(case.m_indptr[e + 1])
-        if hi > lo:
-            ref = R.ref_w8a8_block_fp8_matmul(case.a[lo:hi], case.b[e], case.a_scale[lo:hi], case.b_scale[e], None, torch.bfloat16)
-            check(out[lo:hi], ref, what=f"ragged stream {which} T={T} expert {e}")
+    for waves in (None, 4, 6, 8):
+        out = torch.full((case.a.shape[0], case.b.shape[1]), 7.0, dtype=torch.bfloat16, device=device)
+        _lib.fp8_ragged_gemm(out, d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, {"KERNEL": "stream"} if waves is None else {"KERNEL": "stream", "WAVES": waves})
+        cfg = used("stream")
+        assert cfg["ROW_GROUPS"] == 4 and (waves is None or cfg["WAVES"] == waves), cfg
+        for e in range(E):
+            lo, hi = int(case.m_indptr[e]), int(case.m_indptr[e + 1])
+            if hi > lo:
+                ref = R.ref_w8a8_block_fp8_matmul(case.a[lo:hi], case.b[e], case.a_scale[lo:hi], case.b_scale[e], None, torch.bfloat16)
+                check(out[lo:hi], ref, what=f"ragged stream {which} T={T} expert {e} waves {waves}")
 
 
 def test_ragged_stream_form_is_the_default_for_one_token(device):
     case = W.moe_decode_case(_moe_base("down"), 1)
     d = case.to(device)
     out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, 1)
-    used("stream")
+    assert used("stream")["WAVES"] == 4          # six rows x 32 workgroups of 64 weight rows: one per compute unit as it is
+    case = W.moe_decode_case(_moe_base("gate_up"), 1)
+    d = case.to(device)
+    out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, 1)
+    assert used("stream")["WAVES"] == 6          # six rows x 44 workgroups are 264: 96 weight rows per workgroup make it 180
     case = W.moe_decode_case(_moe_base("down"), 16)
     d = case.to(device)
     out = ragged_block_scaled_bmm(d.a, d.b, d.a_scale, d.b_scale, d.m_indptr, 16)

@@ -16,7 +16,14 @@ hipError_t run_stream(int mt, int nbuf, int waves, bool bs, const GemmParams& p,
     return hipErrorInvalidConfiguration;
 }
 
-hipError_t run_stream_ragged(const GemmParams& p, hipStream_t s) { return launch_stream_ragged(p, s); }
+hipError_t run_stream_ragged(const GemmParams& p, int waves, hipStream_t s) {
+    switch (waves) {
+        case 4: return launch_stream_ragged<4>(p, s);
+        case 6: return launch_stream_ragged<6>(p, s);
+        case 8: return launch_stream_ragged<8>(p, s);
+        default: return hipErrorInvalidConfiguration;
+    }
+}
 
 hipError_t run_stream_wide(bool bs, const GemmParams& p, int gy, hipStream_t s, bool two_buffers, int mt) {
     int gx = (p.N + 63) / 64;

@@ -46,7 +46,7 @@ hipError_t run_skinny(int mt, int rg, int nw, bool blockscale, const GemmParams&
 hipError_t run_stream(int mt, int nbuf, int waves, bool blockscale, const GemmParams& p, int gx, int gy, hipStream_t s);
 // 64 weight rows per workgroup, activation piece shared through LDS: M <= 16
 // ragged block-scaled GEMM, a handful of rows per expert: one grid row per expert, weights streamed once per 16 rows
-hipError_t run_stream_ragged(const GemmParams& p, hipStream_t s);
+hipError_t run_stream_ragged(const GemmParams& p, int waves, hipStream_t s);  // waves per workgroup: 4, 6 or 8 (16 weight rows each)
 // two_buffers (needs K % 128 == 0): two 512-byte-per-row pieces per wave in flight, staggered over K; else one 1 KiB piece
 // mt = 1, 2: tiles of 16 activation rows (M <= 16 mt; two only with two_buffers)
 hipError_t run_stream_wide(bool blockscale, const GemmParams& p, int gy, hipStream_t s, bool two_buffers, int mt);

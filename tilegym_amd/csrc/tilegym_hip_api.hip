@@ -1063,8 +1063,23 @@ int32_t tg_fp8_ragged_gemm(const tg_tensor* c, const tg_tensor* a, const tg_tens
     const bool stream_ok = p.As && p.Bs && N * K < ((int64_t)1 << 31) && E <= 65535;
     if (stream_ok && (want_kernel == 3 || (want_kernel < 0 && total_m <= kRaggedStreamRows))) {
         s.kernel = 3; s.row_groups = 4; s.waves = 4;
+        // Waves (16 weight rows each) per workgroup: WAVES = 4 / 6 / 8, else the fewest that give the fewest rounds of 256
+        // workgroups with rows -- at most one grid row per routed row.  One token of config 5 (six experts): gate+up
+        // 264 workgroups of 64 rows 11.5 us, 180 of 96 rows 9.7 us; two tokens, down: 384 of 64 rows 10.8 us, 192 of 128
+        // rows 9.3 us; with equal rounds fewer waves are faster (down, one token: 7.0 / 8.4 / 9.0 us for 4 / 6 / 8).
+        const int want_waves = cfg_get(cfg, ncfg, TG_CFG_WAVES);
+        if (want_waves == 4 || want_waves == 6 || want_waves == 8) {
+            s.waves = want_waves;
+        } else {
+            const int64_t live = total_m < E ? total_m : E;
+            int64_t best_rounds = 0;
+            for (int w : {4, 6, 8}) {
+                const int64_t rounds = cdiv(live * cdiv(N, 16 * w), 256);
+                if (w == 4 || rounds < best_rounds) { best_rounds = rounds; s.waves = w; }
+            }
+        }
         remember(s);
-        const hipError_t e = tg::run_stream_ragged(p, stream);
+        const hipError_t e = tg::run_stream_ragged(p, s.waves, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "ragged stream kernel launch failed: %s", hipGetErrorString(e));
         return TG_OK;
     }
