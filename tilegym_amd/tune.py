@@ -3,9 +3,10 @@
     python -m tilegym_amd.tune --shape 16,5120,12288 --shape 8,4096,11008,block --out tune.json
     TILEGYM_HIP_TUNE=tune.json python my_decode_loop.py
 
-The library picks its schedules in O(1) from rules fitted to a set of shapes (``choose_dense`` in
-csrc/tilegym_hip_api.hip) and a test holds them within 25 % of the best forced schedule on shapes they were not fitted
-to.  For a caller who wants the last few percent on the shapes of one model, this module does what the reference's
+The library picks its schedules in O(1): fixed rules up to 16 rows, cost models over kernels, tiles and split-K factors
+above (``choose_dense`` in csrc/tilegym_hip_api.hip; their constants were fitted to tables this module wrote), and a test
+holds the choice within 25 % of the best forced schedule on shapes outside the fit (measured: 1 - 2 % on average).
+For a caller who wants the last few percent on the shapes of one model, this module does what the reference's
 exhaustive search does (src/tilegym/ops/cutile/matmul.py:327-418): it times the candidates on this GPU -- weights
 rotated through more copies than the caches hold, launches replayed from a HIP graph, as in a decode step -- and writes
 a JSON table that ``tilegym_amd._lib`` reads when TILEGYM_HIP_TUNE names it.  A recorded entry is only a
