@@ -160,7 +160,7 @@ def test_per_tensor_mid_tiles(device, bm, bn, M, N, K):
 def test_mid_tiles_are_the_default_for_small_weights(device):
     g = _g(8)
     b = fp8_randn((4096, 4096), g, 0.02)
-    for M, want in ((32, (32, 32)), (64, (32, 32)), (128, (64, 32)), (192, (64, 64)), (256, (64, 64)), (320, (64, 128))):
+    for M, want in ((32, (32, 32)), (64, (32, 32)), (128, (64, 32)), (192, (64, 64)), (256, (64, 64)), (320, (64, 88))):   # (320 rows: five row tiles x 47 tiles of 88 columns fit one round, 32 of 128 leave 96 compute units idle)
         a = fp8_randn((M, 4096), g)
         out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
         cfg = used("tiled")
@@ -520,6 +520,35 @@ def test_stream_wide_picks_its_rows_per_workgroup(device):
         assert (cfg["ROW_GROUPS"], cfg["SPLIT_K"], cfg["BLOCK_N"]) == (4, 1, bn), cfg
         rows = torch.arange(0, N, 37)
         check(out[:, rows.to(device)], R.ref_gemm_per_tensor(a, b[rows], 0.01, 0.02, trans_b=True), what=f"{N} x {K}, rows per workgroup")
+
+
+@pytest.mark.parametrize("bn", [72, 96, 112, 120])
+@pytest.mark.parametrize("M,N,K,split", [(64, 1000, 1024, 1), (40, 2304, 512, 1), (130, 520, 2048, 2), (17, 4096, 640, 1)])
+def test_deep_tile_kernel_over_fewer_weight_rows_per_tile(device, bn, M, N, K, split):
+    """BLOCK_N = 72 .. 120 with BLOCK_M = 64: the 64 x 128 tile kernel with tiles that cover fewer weight rows (the rest of
+    the weight slab is neither loaded nor stored).  N that is no multiple of the tile, several row tiles, split-K."""
+    g = _g(bn * 13 + M + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    kc = {"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": bn, "SPLIT_K": split}
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.011, scale_b=0.0003, out_dtype=torch.bfloat16, kernel_configs=kc)
+    cfg = used("tiled")
+    assert (cfg["BLOCK_M"], cfg["BLOCK_N"], cfg["SPLIT_K"]) == (64, bn, split), cfg
+    check(out, R.ref_gemm_per_tensor(a, b, 0.011, 0.0003, trans_b=True), what=f"64 x {bn} tiles, M={M} N={N} K={K}")
+    full = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.011, scale_b=0.0003, out_dtype=torch.bfloat16,
+                  kernel_configs={"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": 128, "SPLIT_K": split})
+    assert torch.equal(out, full)     # the same products in the same order, whatever the tile's width
+
+
+def test_deep_tile_is_narrowed_to_fill_the_chip(device):
+    """28672 weight rows at M = 64: 224 tiles of 128 columns would leave an eighth of the compute units idle; 256 tiles of 112 run."""
+    g = _g(112)
+    a, b = fp8_randn((64, 512), g), fp8_randn((28672, 512), g, 0.02)
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.01, scale_b=0.02, out_dtype=torch.bfloat16)
+    cfg = _lib.last_config()
+    if cfg["KERNEL_NAME"] == "tiled" and cfg["BLOCK_M"] == 64 and cfg["BLOCK_N"] > 64:
+        assert cfg["BLOCK_N"] == 112, cfg
+    rows = torch.arange(0, 28672, 61)
+    check(out[:, rows.to(device)], R.ref_gemm_per_tensor(a, b[rows], 0.01, 0.02, trans_b=True), what="28672 x 512 at M = 64")
 
 
 def _random_shapes(count, seed):

@@ -9,6 +9,9 @@
 // Same slab layout, swizzles, fragment addressing, MFMA order per accumulator and epilogue arithmetic
 // as fp8_gemm_tile_kernel<64, 128, 1, 4, false, GROUP_DENSE, SPLIT>: identical results.
 // Steps past the end re-fetch the last one, which keeps the wait counts uniform.
+// A tile may cover fewer than 128 weight rows (p.tile_cols, a multiple of 8): the slab rows beyond them are requested from
+// beyond the buffer descriptor's range (no memory traffic, zeros) and their columns are not stored.  With 28672 weight
+// rows at M = 64, tiles of 112 are one per compute unit where tiles of 128 leave an eighth of the chip idle.
 #pragma once
 
 #include "fp8_gemm_tile.h"
@@ -32,14 +35,16 @@ __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmPa
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave;
     const int K = p.K;
-    const int tiles_n = (p.N + BN - 1) / BN, tiles_m = (p.M + BM - 1) / BM;
+    const int cols = p.tile_cols > 0 ? p.tile_cols : BN;   // weight rows (output columns) this tile covers
+    const int tiles_n = (p.N + cols - 1) / cols, tiles_m = (p.M + BM - 1) / BM;
     const int pid = xcd_remap((int)blockIdx.x, tiles_m * tiles_n);
     constexpr int GM = 8;
     const int width = GM * tiles_n;
     const int group = pid / width, first_m = group * GM;
     const int gsz = min(tiles_m - first_m, GM);
     const int tile_m = first_m + (pid % width) % gsz, tile_n = (pid % width) / gsz;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = tile_n * cols;
+    const int n_end = min(n0 + cols, p.N);
     const int rows_valid = min(BM, p.M - m0);
 
     int ks = 0, ks_end = p.kblocks;
@@ -62,7 +67,7 @@ __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmPa
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
         const int br = (i * NL + wave) * 8 + lrow;
-        b_off[i] = (uint32_t)min(n0 + br, p.N - 1) * (uint32_t)K + ljb * 16;
+        b_off[i] = n0 + br < n_end ? (uint32_t)(n0 + br) * (uint32_t)K + ljb * 16 : 0x80000000u;  // (>= the descriptor's 2^31 - 1 bytes)
     }
     const v4i rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(p.B);
     const uint32_t lds0 = lds_address(lds) + wave * 1024;
@@ -166,11 +171,11 @@ __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmPa
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
             const int rt = tm * 16 + li;
-            if (rt >= rows_valid || col >= p.N) continue;
+            if (rt >= rows_valid || col >= n_end) continue;
             if constexpr (SPLIT)
-                store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, m0 + rt, col, p.N, p.N, acc[0][tm], acc[1][tm], 0.f, vec_ok);
+                store8(p.partials + (int64_t)blockIdx.y * MN, OUT_F32, m0 + rt, col, n_end, p.N, acc[0][tm], acc[1][tm], 0.f, vec_ok);
             else
-                store8(p.C, OT, m0 + rt, col, p.N, p.ldc, acc[0][tm] * scale, acc[1][tm] * scale, p.beta, vec_ok);
+                store8(p.C, OT, m0 + rt, col, n_end, p.ldc, acc[0][tm] * scale, acc[1][tm] * scale, p.beta, vec_ok);
         }
     };
     if (SPLIT || p.out_type == OUT_BF16) emit(std::integral_constant<int, OUT_BF16>{});
@@ -182,6 +187,7 @@ __global__ void __launch_bounds__(256, 2) fp8_gemm_tile_deep_kernel(const GemmPa
 
 template <bool SPLIT>
 inline hipError_t launch_tile_deep(const GemmParams& p, int grid_x, int grid_y, hipStream_t stream) {
+    if (p.tile_cols != 0 && (p.tile_cols < 8 || p.tile_cols > 128 || (p.tile_cols % 8) != 0)) return hipErrorInvalidValue;
     hipLaunchKernelGGL(fp8_gemm_tile_deep_kernel<SPLIT>, dim3(grid_x, grid_y, 1), dim3(256, 1, 1), 0, stream, p);
     return hipGetLastError();
 }

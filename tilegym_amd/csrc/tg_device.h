@@ -54,6 +54,8 @@ struct GemmParams {
     int act_is_bf16;
     // wide streaming form: weight rows per wave (1 .. 16; 0 means 16).  Fewer than 16 make more, smaller workgroups
     int wave_rows;
+    // deep 64 x 128 tile kernel: weight rows a tile covers (a multiple of 8, 72 .. 128; 0 means 128).  Fewer make more tiles
+    int tile_cols;
 };
 
 // A list of independent per-tensor-scaled NT GEMMs handed to one launch in the kernel arguments.

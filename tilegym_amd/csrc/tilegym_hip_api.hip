@@ -170,8 +170,12 @@ struct PieceRecord {
 // Tiles of fp8_gemm_tile_mid_kernel.
 bool is_mid_tile(int bm, int bn) { return ((bm == 64 || bm == 32) && bn == 32) || (bm == 64 && bn == 64); }
 
+// Per-tensor 64-row tiles of 72 .. 120 weight rows: the deep 64 x 128 kernel with the rest of its weight slab unused.
+bool is_narrowed_deep_tile(int bm, int bn) { return bm == 64 && bn >= 72 && bn < 128 && bn % 8 == 0; }
+
 bool tile_exists(int bm, int bn, bool block_scaled) {
     if (is_mid_tile(bm, bn)) return !block_scaled;  // the four waves split K inside the workgroup (per-tensor only)
+    if (is_narrowed_deep_tile(bm, bn)) return !block_scaled;
     if (bm == 128 && bn == 128) return true;
     if (bm == 128 && bn == 256) return true;
     if (bm == 64 && bn == 128) return true;
@@ -266,8 +270,27 @@ inline float rounds_cost_us(const TileCost& t, int64_t units, int64_t steps) {
     return units <= 256 ? (float)steps * t.alone + t.fixed : (float)cdiv(units, 512) * ((float)steps * t.shared + t.fixed);
 }
 
+Schedule choose_dense_tile(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
+                           const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail);
+
+// The schedule of a dense problem: choose_dense_tile's, and for the per-tensor 64 x 128 tile kernel with fewer workgroups than
+// compute units the tile narrowed (120, 112, ... 72 weight rows) as far as the workgroups still fit one round: what a
+// workgroup of this weight-streaming regime takes in, (64 + columns) x K bytes, shrinks with it, and more compute units
+// take part (28672 x 4096 at M = 64: 224 tiles of 128 columns or 256 of 112).
 Schedule choose_dense(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
                       const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
+    Schedule s = choose_dense_tile(M, N, K, block_scaled, fast_layout, cfg, ncfg, partial_bytes_avail);
+    if (s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128 && cfg_get(cfg, ncfg, TG_CFG_BLOCK_N) <= 0) {
+        const int64_t tiles_m = cdiv(M, 64);
+        if (tiles_m * cdiv(N, 128) * s.split_k < 256) {
+            for (int bn = 120; bn >= 72 && tiles_m * cdiv(N, bn) * s.split_k <= 256; bn -= 8) s.bn = bn;
+        }
+    }
+    return s;
+}
+
+Schedule choose_dense_tile(int64_t M, int64_t N, int64_t K, bool block_scaled, bool fast_layout,
+                           const int32_t* cfg, int32_t ncfg, int64_t partial_bytes_avail) {
     Schedule s{0, -1, -1, 1, -1, -1, -1};
     const int want_kernel = cfg_get(cfg, ncfg, TG_CFG_KERNEL);
     const int64_t kblocks = cdiv(K, 128);
@@ -932,7 +955,8 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         if (rows != M && s.split_k > 1) { pc.split_k = 1; pc.ksteps_per_split = (int)kblocks; }
         int gx = (int)(cdiv(rows, s.bm) * cdiv(N, s.bn));
         const bool split = pc.split_k > 1;
-        const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && s.bn == 128;
+        const bool deep = s.kernel == 1 && !block_scaled && s.bm == 64 && (s.bn == 128 || is_narrowed_deep_tile(s.bm, s.bn));
+        if (deep) pc.tile_cols = s.bn;
         const bool mid = s.kernel == 1 && !block_scaled && is_mid_tile(s.bm, s.bn);
         // persistent kernel with the hand-ordered K loop for the dense per-tensor 256x256 tile, from two K steps up
         // (WAVES = 8 asks for the generic eight-wave tile kernel instead)

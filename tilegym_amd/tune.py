@@ -46,6 +46,9 @@ def candidates(M: int, N: int, K: int, block_scaled: bool) -> List[dict]:
                 if s > 1 and (bm, bn) in ((32, 32), (64, 32), (64, 64)):
                     continue
                 out.append({"KERNEL": "tiled", "BLOCK_M": bm, "BLOCK_N": bn, "SPLIT_K": s})
+        if not block_scaled and M <= 512:
+            # the 64 x 128 tile kernel over fewer weight rows per tile (more, lighter workgroups)
+            out += [{"KERNEL": "tiled", "BLOCK_M": 64, "BLOCK_N": bn, "SPLIT_K": s} for bn in (112, 96, 80) for s in (1, 2, 4, 8)]
     return out
 
 
