@@ -63,7 +63,7 @@ enum {
     TG_CFG_KERNEL = 0,  /* 0 fallback (no MFMA), 1 LDS-tiled MFMA kernel, 2 skinny (direct weight streaming), 3 stream (weight streaming through LDS) */
     TG_CFG_BLOCK_M = 1, /* tiled kernel: rows of A per workgroup (32/64/128/256; 32x32, 64x32 and 64x64 = in-workgroup K split, per-tensor only) */
     TG_CFG_BLOCK_N = 2, /* tiled kernel: rows of B per workgroup (32/64/128/256; per-tensor with BLOCK_M = 64 also 72 .. 120 in steps of 8); stream kernel, wide form (ROW_GROUPS = 4,
-                         * K % 128 == 0): rows of B per workgroup, a multiple of 4 up to 64 (four waves own a quarter each) */
+                         * K % 128 == 0): rows of B per workgroup, a multiple of 4 up to 64 (four waves own a quarter each); narrow form: 1 .. 16 */
     TG_CFG_SPLIT_K = 3, /* K partitions reduced through the workspace (1 = none)         */
     TG_CFG_ROW_GROUPS = 4, /* skinny kernel: 16-row groups of B per wave (1/2/4); stream kernel: LDS buffers per wave (1/2);
                             * tiled 256x256 block-scaled kernels (dense and ragged): 1 = the persistent form (one workgroup per

@@ -551,6 +551,28 @@ def test_deep_tile_is_narrowed_to_fill_the_chip(device):
     check(out[:, rows.to(device)], R.ref_gemm_per_tensor(a, b[rows], 0.01, 0.02, trans_b=True), what="28672 x 512 at M = 64")
 
 
+@pytest.mark.parametrize("rows", [14, 12, 8, 5])
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 1024), (8, 520, 4096), (16, 2050, 1152)])
+def test_narrow_stream_form_with_fewer_rows_per_workgroup(device, rows, M, N, K):
+    """BLOCK_N of the narrow streaming form: the weight rows a workgroup owns (16 by default).  Same bits as with 16."""
+    g = _g(rows * 17 + M + N + K)
+    a, b = fp8_randn((M, K), g), fp8_randn((N, K), g, 0.02)
+    kc = {"KERNEL": "stream", "ROW_GROUPS": 1, "WAVES": 4, "SPLIT_K": 1, "BLOCK_N": rows}
+    out = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.011, scale_b=0.0003, out_dtype=torch.bfloat16, kernel_configs=kc)
+    cfg = used("stream")
+    assert (cfg["ROW_GROUPS"], cfg["BLOCK_N"]) == (1, rows), cfg
+    check(out, R.ref_gemm_per_tensor(a, b, 0.011, 0.0003, trans_b=True), what=f"narrow stream, {rows} rows per workgroup, M={M} N={N} K={K}")
+    kc["BLOCK_N"] = 16
+    full = matmul(a.to(device), b.to(device), trans_b=True, scale_a=0.011, scale_b=0.0003, out_dtype=torch.bfloat16, kernel_configs=kc)
+    assert torch.equal(out, full)
+    if rows == 8:   # block-scaled: a workgroup's rows share one weight scale, so only divisors of 128
+        case = W.block_scaled_case(M, N, K, seed=M + N)
+        d = case.to(device)
+        out = w8a8_block_fp8_matmul(d.a, d.b, d.scale_a, d.scale_b, None, torch.bfloat16, kernel_configs=kc | {"BLOCK_N": 8})
+        assert used("stream")["BLOCK_N"] == 8
+        check(out, R.ref_w8a8_block_fp8_matmul(case.a, case.b, case.scale_a, case.scale_b, None, torch.bfloat16), what="block-scaled narrow stream, 8 rows")
+
+
 def _random_shapes(count, seed):
     """Seeded shapes across the regimes of the automatic choice: rows log-uniform in 1 .. 700, weight rows multiples of 16
     up to 6000, K a multiple of 128 (three in four) or of 16; the CPU oracle's work is capped at 2 GFLOP per shape."""

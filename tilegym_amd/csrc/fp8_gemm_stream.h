@@ -29,7 +29,12 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_kernel(const GemmPara
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int K = p.K, N = p.N, M = p.M;
-    const int n_base = blockIdx.x * 16;
+    // weight rows per workgroup: 16, or fewer so that the workgroups come out even over the compute units (6144 rows:
+    // 384 workgroups of 16 rows put two on half of the compute units and one on the others, 512 of 12 rows two on each).
+    // The rows a workgroup does not own are requested from beyond the descriptor's range (no memory request) and not stored.
+    const int R = p.wave_rows > 0 ? p.wave_rows : 16;
+    const int n_base = blockIdx.x * R;
+    const int n_end = min(n_base + R, N);
     const int nchunks_total = (K + kStreamChunk - 1) / kStreamChunk;
 
     int c_begin = 0, c_end = nchunks_total;
@@ -49,7 +54,7 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_kernel(const GemmPara
         for (int r = 0; r < 16; ++r) {
             const int n = min(n_base + r, N - 1);
             const int j = lane ^ r;
-            const uint32_t voff = (uint32_t)n * (uint32_t)K + j * 16;
+            const uint32_t voff = n_base + r < n_end ? (uint32_t)n * (uint32_t)K + j * 16 : 0x80000000u;
             const uint32_t dst = my_lds + buf * BUF + r * kStreamChunk;
             if (k0 + j * 16 < K) {
                 direct_load_b128_nt(rsrc_b, dst, voff, k0);
@@ -210,14 +215,14 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_kernel(const GemmPara
 #pragma unroll
         for (int w = 0; w < NW - 1; ++w) acc[mt] += red[(w * MT + mt) * 64 + lane];
 
-    const bool vec_ok = p.vec_store != 0;
+    const bool vec_ok = p.vec_store != 0 && (R & 3) == 0;  // (a lane's four outputs are all the workgroup's, or with R % 4 != 0 some of them)
     const int col = n_base + lg * 4;
     if (p.split_k > 1) {
         float* mine = p.partials + (int64_t)blockIdx.y * M * N;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + li;
-            if (m < M && col < N) store4(mine, OUT_F32, m, col, N, N, acc[mt], 0.f, vec_ok);
+            if (m < M && col < n_end) store4(mine, OUT_F32, m, col, n_end, N, acc[mt], 0.f, vec_ok);
         }
         return;
     }
@@ -229,7 +234,7 @@ __global__ void __launch_bounds__(64 * NW) fp8_gemm_stream_kernel(const GemmPara
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + li;
-        if (m < M && col < N) store4(p.C, p.out_type, m, col, N, p.ldc, acc[mt] * scale, p.beta, vec_ok);
+        if (m < M && col < n_end) store4(p.C, p.out_type, m, col, n_end, p.ldc, acc[mt] * scale, p.beta, vec_ok);
     }
 #endif
 }

@@ -5,6 +5,8 @@
 namespace tg {
 
 hipError_t run_stream(int mt, int nbuf, int waves, bool bs, const GemmParams& p, int gx, int gy, hipStream_t s) {
+    // rows per workgroup: 1 .. 16; with block scales a workgroup's rows share one weight scale
+    if (p.wave_rows < 0 || p.wave_rows > 16 || (bs && p.wave_rows > 0 && 128 % p.wave_rows != 0)) return hipErrorInvalidValue;
     // eight waves per workgroup (one 16 KiB buffer each, one workgroup per compute unit): long K over few weight rows
     if (waves == 8 && mt == 1 && nbuf == 1)
         return bs ? launch_stream<1, 1, true, 8>(p, gx, gy, s) : launch_stream<1, 1, false, 8>(p, gx, gy, s);

@@ -473,6 +473,14 @@ Schedule choose_dense_tile(int64_t M, int64_t N, int64_t K, bool block_scaled, b
         if (!try_wide) {
             if (want_split > 1 || (want_split < 0 && wgs * 4 * 4 <= kTargetWaves && pieces >= 16))
                 s.split_k = pick_split(wgs * 4, kTargetWaves / 2, pieces, want_split > 1 ? 1 : 8, M, N, partial_bytes_avail, want_split);
+            // weight rows per workgroup of the narrow form (BLOCK_N = 1 .. 16; block-scaled: a divisor of 128)
+            const int want_rows = cfg_get(cfg, ncfg, TG_CFG_BLOCK_N);
+            if (want_rows >= 1 && want_rows <= 16 && (!block_scaled || 128 % want_rows == 0)) s.bn = want_rows;
+            // between one and two workgroups of 16 rows per compute unit, half of the compute units take in twice what the
+            // others do; 12 rows per workgroup even that out (6144 x 4096 at M = 8: 8.1 against 8.7 us; 5120 x 5120 at
+            // M = 1: 8.9 against 9.5).  More than two per compute unit cost more than they even out (7168 rows: 14 rows
+            // per workgroup 6.4 against 6.0 us), and block-scaled workgroups must not straddle a row of weight scales.
+            else if (want_rows <= 0 && !block_scaled && s.split_k == 1 && wgs >= 272 && cdiv(N, 12) <= 512) s.bn = 12;
             return s;
         }
         s = Schedule{0, -1, -1, 1, -1, -1, -1};  // not taken by the wide form: on to the tile kernels
@@ -926,8 +934,9 @@ int32_t fp8_gemm_impl(const tg_tensor* c, const tg_tensor* a, const tg_tensor* b
         if (nbuf != 1 && nbuf != 2) nbuf = (per_wave >= 3 && s.mt == 1 && !block_scaled) ? 2 : 1;
         if (s.mt != 1 || s.waves == 8) nbuf = 1;
         if (s.row_groups == 4 && s.waves == 4 && s.bn > 0) p.wave_rows = s.bn / 4;
+        if (s.row_groups != 4 && s.bn > 0) p.wave_rows = s.bn;  // narrow form: weight rows per workgroup
         hipError_t e = s.row_groups == 4 ? tg::run_stream_wide(block_scaled, p, s.split_k, stream, s.waves == 4, s.mt)
-                                         : tg::run_stream(s.mt, nbuf, s.waves, block_scaled, p, (int)cdiv(N, 16), s.split_k, stream);
+                                         : tg::run_stream(s.mt, nbuf, s.waves, block_scaled, p, (int)cdiv(N, p.wave_rows > 0 ? p.wave_rows : 16), s.split_k, stream);
         if (e != hipSuccess) return fail(TG_ERR_LAUNCH, "stream kernel launch failed: %s", hipGetErrorString(e));
         if (s.split_k > 1 && tg::run_splitk_reduce(p, block_scaled, stream) != hipSuccess)
             return fail(TG_ERR_LAUNCH, "split-K reduction launch failed");
