@@ -410,20 +410,24 @@ Schedule choose_dense_tile(int64_t M, int64_t N, int64_t K, bool block_scaled, b
         // splits, 19.8 unsplit with 24 rows).
         int wide_bn = 64;
         const bool rows_free = (K % 128) == 0 && cfg_get(cfg, ncfg, TG_CFG_BLOCK_N) <= 0 && cfg_get(cfg, ncfg, TG_CFG_WAVES) != 1;
-        if (rows_free && M <= 16 && (pieces <= 8 || wide_split == 1) && want_split <= 1) {
+        // (block-scaled: to K = 5120 only -- a piece of its K loop takes longer, and from there on 64 rows with two or
+        // more splits win: 8192 x 8192 at M = 16 16.5 us against 19.1 unsplit with 32 rows)
+        const int64_t unsplit_pieces = block_scaled ? 5 : 8;
+        if (rows_free && M <= 16 && (pieces <= unsplit_pieces || wide_split == 1) && want_split <= 1) {
             int64_t best_cost = 0;
             int best_bn = 64;
-            for (int bn = 64; bn >= 24; bn -= 8) {
+            // (long K: 48 rows and more -- 9216 x 16384 takes 25.2 us with 48 rows and 32.5 with 40)
+            for (int bn = 64; bn >= (pieces > 8 ? 48 : 24); bn -= 8) {
                 const int64_t cost = cdiv(cdiv(N, bn), 256) * (bn + 16);
                 if (bn == 64 || cost < best_cost) { best_cost = cost; best_bn = bn; }
             }
             // (too few weight rows to fill the chip even with 24 per workgroup: 64 rows and split-K as before)
-            if (cdiv(N, best_bn) >= 200) {
+            if (cdiv(N, best_bn) >= 176) {
                 wide_bn = best_bn;
-                if (pieces <= 8) wide_split = 1;
+                if (pieces <= unsplit_pieces) wide_split = 1;
                 // with its workgroups filling the chip the wide form also wins at nine rows and more over smaller weights
                 // (8192 x 3072 at M = 16: 7.3 against 8.0 us; 5120 x 5120: 9.4 against 11.9)
-                if (M > 8 && pieces <= 8) wide_auto = true;
+                if (M > 8 && pieces <= unsplit_pieces) wide_auto = true;
             }
         }
         // long K over one 16-row workgroup per compute unit, one or two activation rows: eight waves split K inside the
