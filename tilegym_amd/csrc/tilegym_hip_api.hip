@@ -367,6 +367,16 @@ Schedule choose_dense_tile(int64_t M, int64_t N, int64_t K, bool block_scaled, b
             const Schedule cand = skinny_schedule();
             offer(cand, (float)cdiv(N, 16) / 256.f * (float)kblocks * c.skinny_step * (float)cand.mt + c.skinny_fixed + reduce(cand.split_k));
         }
+        // the wide form, unsplit: weight rows per workgroup so that the workgroups fill the chip, as for up to 16 rows
+        if (best.kernel == 3 && best.row_groups == 4 && best.split_k == 1) {
+            int64_t best_cost = 0;
+            int rows = 64;
+            for (int bn = 64; bn >= 32; bn -= 8) {
+                const int64_t cost = cdiv(cdiv(N, bn), 256) * (bn + 16);
+                if (bn == 64 || cost < best_cost) { best_cost = cost; rows = bn; }
+            }
+            if (rows != 64 && cdiv(N, rows) >= 176) best.bn = rows;
+        }
         return best;
     }
     const bool nothing_forced = want_kernel < 0 && want_split < 0 && cfg_get(cfg, ncfg, TG_CFG_ROW_GROUPS) < 0 && cfg_get(cfg, ncfg, TG_CFG_WAVES) < 0;
