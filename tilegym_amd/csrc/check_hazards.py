@@ -1,0 +1,153 @@
+#!/usr/bin/env python3
+"""Build check for one hardware rule that the compiler cannot enforce inside inline assembly.
+
+On gfx9-family hardware a vector-memory instruction must not read a scalar register within five
+wait states of a vector instruction writing it (v_readfirstlane, v_readlane, a VALU compare or
+carry into a scalar pair): the memory instruction would see the register's old value.  hipcc
+inserts the s_nops for the instructions it emits itself; the direct global->LDS loads and the
+register scale loads of these kernels are inline assembly, which its hazard recognizer does not
+look into.  Most of them carry their own wait states; the ones that do not (direct_load_b128_settled)
+rely on this check.
+
+    python3 check_hazards.py file.s [file.s ...]     # assembly from hipcc --cuda-device-only -S
+    python3 check_hazards.py --build [name.hip ...]   # compile the sources beside this file first
+
+Walks every kernel's control-flow graph backwards from each buffer_/global_/scratch_/flat_
+instruction over all paths, five wait states deep (s_nop N counts N + 1, everything else 1).
+Exit status 1 and one line per finding if a scalar operand was written by a vector instruction
+inside that window.
+"""
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+WAIT_STATES = 5
+VMEM_PREFIXES = ("buffer_", "global_", "scratch_", "flat_")
+CARRY_OPS = ("v_div_scale", "v_mad_u64_u32", "v_mad_i64_i32")
+HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
+               "-packed-fp32-ops", "--cuda-device-only", "-S"]
+# translation units with inline-assembly memory instructions
+DEFAULT_SOURCES = ["fp8_gemm_tile_pt.hip", "fp8_gemm_tile256.hip", "fp8_gemm_tile_bs.hip", "fp8_gemm_tile_bs256.hip",
+                   "fp8_gemm_tile_grouped.hip", "fp8_gemm_tile_list.hip", "fp8_gemm_stream.hip"]
+
+
+def scalar_regs(tok):
+    m = re.fullmatch(r"s\[(\d+):(\d+)\]", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.fullmatch(r"s(\d+)", tok)
+    if m:
+        return {int(m.group(1))}
+    if tok in ("vcc", "vcc_lo", "vcc_hi"):
+        return {"vcc"}
+    return set()
+
+
+def valu_scalar_writes(op, toks):
+    """Scalar registers a vector instruction writes."""
+    if not op.startswith("v_") or not toks:
+        return set()
+    dst = scalar_regs(toks[0])
+    if len(toks) > 1 and ("_co_" in op or op.startswith(CARRY_OPS)):
+        dst |= scalar_regs(toks[1])
+    if op.endswith("_e32") and (op.startswith("v_cmp") or "_co_" in op):
+        dst |= {"vcc"}
+    return dst
+
+
+def parse_kernels(path):
+    """{kernel: [(op, operand tokens, text)]} plus each kernel's label -> instruction index."""
+    kernels, labels, name = {}, {}, None
+    for raw in open(path):
+        line = raw.split(";")[0].strip()
+        if not line:
+            continue
+        if line.endswith(":"):
+            label = line[:-1]
+            if label.startswith(".L") or label.startswith("BB") or label.startswith(".BB"):
+                if name is not None:
+                    labels[name][label] = len(kernels[name])
+            else:
+                name = label
+                kernels[name], labels[name] = [], {}
+            continue
+        if line.startswith(".") or name is None:
+            continue
+        op, _, rest = line.partition(" ")
+        toks = [t.strip().split()[0] for t in rest.split(",") if t.strip()]
+        kernels[name].append((op, toks, line))
+    return kernels, labels
+
+
+def predecessors(insts, labels):
+    preds = [[] for _ in insts]
+    for i, (op, toks, _) in enumerate(insts):
+        falls = op not in ("s_branch", "s_endpgm", "s_setpc_b64")
+        if falls and i + 1 < len(insts):
+            preds[i + 1].append(i)
+        if op == "s_branch" or op.startswith("s_cbranch"):
+            target = labels.get(toks[-1] if toks else "")
+            if target is not None and target < len(insts):
+                preds[target].append(i)
+    return preds
+
+
+def scan(path):
+    findings = []
+    kernels, labels = parse_kernels(path)
+    for name, insts in kernels.items():
+        preds = predecessors(insts, labels[name])
+        writes = [valu_scalar_writes(op, toks) for op, toks, _ in insts]
+        for i, (op, toks, text) in enumerate(insts):
+            if not op.startswith(VMEM_PREFIXES):
+                continue
+            used = set()
+            for t in toks:
+                used |= scalar_regs(t)
+            if not used:
+                continue
+            stack, seen = [(j, 0) for j in preds[i]], set()
+            while stack:
+                j, waited = stack.pop()
+                if (j, waited) in seen:
+                    continue
+                seen.add((j, waited))
+                if writes[j] & used:
+                    findings.append(f"{os.path.basename(path)}: {name}: '{insts[j][2]}' -> '{text}' after {waited} wait states")
+                    continue
+                jop, jtoks, _ = insts[j]
+                waited += int(jtoks[0], 0) + 1 if jop == "s_nop" and jtoks else 1
+                if waited < WAIT_STATES:
+                    stack.extend((k, waited) for k in preds[j])
+    return findings
+
+
+def main(argv):
+    files = argv
+    tmp = None
+    if argv and argv[0] == "--build":
+        here = os.path.dirname(os.path.abspath(__file__))
+        hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+        tmp = tempfile.TemporaryDirectory()
+        files, procs = [], []
+        for src in argv[1:] or DEFAULT_SOURCES:
+            out = os.path.join(tmp.name, os.path.splitext(os.path.basename(src))[0] + ".s")
+            procs.append(subprocess.Popen([hipcc, *HIPCC_FLAGS, os.path.join(here, src), "-o", out],
+                                          stderr=subprocess.DEVNULL))
+            files.append(out)
+        if any(p.wait() != 0 for p in procs):
+            print("check_hazards: a source did not compile", file=sys.stderr)
+            return 2
+    findings = []
+    for f in files:
+        findings += scan(f)
+    for line in findings:
+        print(line)
+    print(f"check_hazards: {len(files)} file(s), {len(findings)} finding(s)")
+    return 1 if findings else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv[1:]))

@@ -51,14 +51,37 @@ __device__ __forceinline__ v4i make_rsrc(const void* base) {
 // flight as possibly aliasing every later LDS read and drains the whole memory pipeline
 // (vmcnt(0)) in front of it, which would undo the multi-step prefetch.  Completion is tracked by
 // hand with the vmcnt waits in the kernel; the "memory" clobber keeps LDS reads from being
-// cached across it.
+// cached across it.  The compiler's hazard recognizer does not look into inline assembly either:
+// a scalar operand that a vector instruction has just written (v_readfirstlane, when the
+// compiler keeps a wave-uniform offset in a vector register) must not be read by a memory
+// instruction within five wait states, or the instruction sees the register's old value.  The
+// M0 write and the s_nop in front of each load are those five.
 __device__ __forceinline__ void direct_load_b128(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
     lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);  // wave-uniform by construction
     soffset = __builtin_amdgcn_readfirstlane(soffset);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory");
+}
+
+// The same load without those wait states, for the one loop where they cost measurable time (a 256 x 256 tile's
+// sixteen loads per K step: 2-3% of the launch).  Only for scalar operands that no vector instruction can have written
+// shortly before: values that come out of settle() below and scalar arithmetic on them, in a kernel that spills no
+// scalar register (a spilled one comes back through v_readlane).  check_hazards.py verifies both on the kernel's assembly.
+__device__ __forceinline__ void direct_load_b128_settled(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
                  : "memory");
+}
+// A wave-uniform value in a scalar register written by a scalar instruction: what the compiler derives from it with
+// scalar arithmetic is never produced by v_readfirstlane right in front of its use.
+__device__ __forceinline__ int settle(int x) {
+    int r;
+    x = __builtin_amdgcn_readfirstlane(x);
+    asm volatile("s_mov_b32 %0, %1" : "=s"(r) : "s"(x));
+    return r;
 }
 
 // The same load marked non-temporal: for data a launch reads exactly once (the weights of a
@@ -67,7 +90,7 @@ __device__ __forceinline__ void direct_load_b128(v4i rsrc, uint32_t lds_addr, ui
 __device__ __forceinline__ void direct_load_b128_nt(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
     lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
     soffset = __builtin_amdgcn_readfirstlane(soffset);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
                  :
                  : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
                  : "memory");
@@ -77,7 +100,7 @@ __device__ __forceinline__ void direct_load_b128_nt(v4i rsrc, uint32_t lds_addr,
 __device__ __forceinline__ void direct_load_b32(v4i rsrc, uint32_t lds_addr, uint32_t voffset, int soffset) {
     lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
     soffset = __builtin_amdgcn_readfirstlane(soffset);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
                  : "memory");

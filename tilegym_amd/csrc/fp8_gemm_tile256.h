@@ -85,12 +85,14 @@ __global__ void __launch_bounds__(256, 1) fp8_gemm_tile256_kernel(const GemmPara
     };
     set_offsets(m0, n0);
     const v4i rsrc_a = make_rsrc(p.A), rsrc_b = make_rsrc(p.B);
-    const uint32_t ldsA = lds_address(sA) + wave * 1024, ldsB = lds_address(sB) + wave * 1024;
+    // (the loads of this kernel go without the wait states of direct_load_b128: their scalar operands are the two
+    // descriptors, these two settled addresses and the loop's own scalar counters)
+    const uint32_t ldsA = settle(lds_address(sA) + wave * 1024), ldsB = settle(lds_address(sB) + wave * 1024);
     auto load_a = [&](int i, int kstep, int stage) {
-        direct_load_b128(rsrc_a, ldsA + stage * SLAB + i * NW * 1024, a_off[i], kstep * kKBlock);
+        direct_load_b128_settled(rsrc_a, ldsA + stage * SLAB + i * NW * 1024, a_off[i], kstep * kKBlock);
     };
     auto load_b = [&](int i, int kstep, int stage) {
-        direct_load_b128(rsrc_b, ldsB + stage * SLAB + i * NW * 1024, b_off[i], kstep * kKBlock);
+        direct_load_b128_settled(rsrc_b, ldsB + stage * SLAB + i * NW * 1024, b_off[i], kstep * kKBlock);
     };
 
     // ---- fragment addresses (see fp8_gemm_tile.h)

@@ -42,10 +42,12 @@ __device__ __forceinline__ v4i make_rsrc_sized(const void* base, uint32_t bytes)
 }
 
 // 4 bytes per lane from a buffer into a register.  The caller orders its use behind a vmcnt wait by hand.
+// (s_nop 4: five wait states between a vector instruction that wrote the scalar offset and this read of it,
+// which the compiler does not insert in front of inline assembly.)
 __device__ __forceinline__ int buffer_load_b32_raw(v4i rsrc, uint32_t voffset, int soffset) {
     int r;
     soffset = __builtin_amdgcn_readfirstlane(soffset);
-    asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(r) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+    asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, %2, %3 offen" : "=v"(r) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
     return r;
 }
 
