@@ -16,6 +16,13 @@ Walks every kernel's control-flow graph backwards from each buffer_/global_/scra
 instruction over all paths, five wait states deep (s_nop N counts N + 1, everything else 1).
 Exit status 1 and one line per finding if a scalar operand was written by a vector instruction
 inside that window.
+
+Second rule, same reason: the compiler takes the result register of an inline-assembly
+buffer_load as written when the statement ends, while the data arrives later (the kernels wait
+with s_waitcnt vmcnt by hand).  A register copy that the compiler places between the load and
+that wait (at a loop's back edge, say) would copy the old contents.  Walks forwards from every
+buffer_load into registers: a finding if any path reads or overwrites the destination before an
+s_waitcnt with a vmcnt field.
 """
 import os
 import re
@@ -81,6 +88,57 @@ def parse_kernels(path):
     return kernels, labels
 
 
+def vector_regs(tok):
+    m = re.fullmatch(r"[va]\[(\d+):(\d+)\]", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.fullmatch(r"[va](\d+)", tok)
+    if m:
+        return {int(m.group(1))}
+    return set()
+
+
+def successors(insts, labels):
+    succs = [[] for _ in insts]
+    for i, (op, toks, _) in enumerate(insts):
+        if op not in ("s_branch", "s_endpgm", "s_setpc_b64") and i + 1 < len(insts):
+            succs[i].append(i + 1)
+        if op == "s_branch" or op.startswith("s_cbranch"):
+            target = labels.get(toks[-1] if toks else "")
+            if target is not None and target < len(insts):
+                succs[i].append(target)
+    return succs
+
+
+def scan_early_use(path):
+    """buffer loads into registers whose destination is touched before any vmcnt wait."""
+    findings = []
+    kernels, labels = parse_kernels(path)
+    for name, insts in kernels.items():
+        succs = successors(insts, labels[name])
+        for i, (op, toks, text) in enumerate(insts):
+            if not op.startswith("buffer_load") or " lds" in text or not toks:
+                continue
+            dst = vector_regs(toks[0])
+            stack, seen = list(succs[i]), set()
+            while stack:
+                j = stack.pop()
+                if j in seen:
+                    continue
+                seen.add(j)
+                jop, jtoks, jtext = insts[j]
+                if jop == "s_waitcnt" and "vmcnt(" in jtext:
+                    continue
+                touched = set()
+                for t in jtoks:
+                    touched |= vector_regs(t)
+                if touched & dst:
+                    findings.append(f"{os.path.basename(path)}: {name}: '{text}' then '{jtext}' with no vmcnt wait between")
+                    continue
+                stack.extend(succs[j])
+    return findings
+
+
 def predecessors(insts, labels):
     preds = [[] for _ in insts]
     for i, (op, toks, _) in enumerate(insts):
@@ -142,7 +200,7 @@ def main(argv):
             return 2
     findings = []
     for f in files:
-        findings += scan(f)
+        findings += scan(f) + scan_early_use(f)
     for line in findings:
         print(line)
     print(f"check_hazards: {len(files)} file(s), {len(findings)} finding(s)")

@@ -360,13 +360,15 @@ __global__ void __launch_bounds__(512, 1) fp8_gemm_bs256_kernel(const GemmParams
             }
             if constexpr (PH == 1) form_products();
             {
-                const bool from_next = PH == QUAD - 1 || (TAIL && k == last);
+                // (a chunk's first step is never a tile's last: the host gives this kernel no K with a last chunk of one
+                // step, and nothing that was requested in this step is read in it)
+                const bool from_next = PH == QUAD - 1 || (TAIL && PH != 0 && k == last);
                 const int src_lane_off = from_next ? 0 : (PH + 1) * 64;
 #pragma unroll
                 for (int tm = 0; tm < TM; ++tm) {
                     int v;
                     if constexpr (PH == QUAD - 1) v = s_nxt[tm];
-                    else if constexpr (TAIL) v = from_next ? s_nxt[tm] : __float_as_int(s_cur[tm]);
+                    else if constexpr (TAIL && PH != 0) v = from_next ? s_nxt[tm] : __float_as_int(s_cur[tm]);
                     else v = __float_as_int(s_cur[tm]);
                     sc_n[tm] = __int_as_float(__builtin_amdgcn_ds_bpermute(bp_base + src_lane_off, v));
                 }
@@ -403,7 +405,9 @@ __global__ void __launch_bounds__(512, 1) fp8_gemm_bs256_kernel(const GemmParams
             for (int k0 = 0; k0 < nsteps; k0 += QUAD) {
                 step(ntm_tag, std::integral_constant<int, 0>{}, k0);
                 if constexpr (TAIL) {
-                    if (k0 + 1 < nsteps) step(ntm_tag, std::integral_constant<int, 1>{}, k0 + 1);
+                    // the second step follows unconditionally (see from_next): its wait is the one that covers the scale
+                    // requests of the first, also in front of the epilogue
+                    step(ntm_tag, std::integral_constant<int, 1>{}, k0 + 1);
                     if (k0 + 2 < nsteps) step(ntm_tag, std::integral_constant<int, 2>{}, k0 + 2);
                     if (k0 + 3 < nsteps) step(ntm_tag, std::integral_constant<int, 3>{}, k0 + 3);
                 } else {
@@ -413,9 +417,9 @@ __global__ void __launch_bounds__(512, 1) fp8_gemm_bs256_kernel(const GemmParams
                 }
             }
         };
-        // (Every wave computes all four of its row groups, also those without a valid row: a copy of the loop per number
-        // of row groups, as fp8_gemm_tile_kernel has, was built and gave wrong results in a way that was not understood;
-        // the step keeps NTM as a parameter.)
+        // (Every wave computes all four of its row groups, also those without a valid row: a second copy of the loop
+        // for tiles of at most 128 rows measured no faster, and one copy per number of row groups, as
+        // fp8_gemm_tile_kernel has, spills; the step keeps NTM as a parameter.)
         k_loop(std::integral_constant<int, TM>{});
 
         // ---------------------------------------------------------------- epilogue, straight from the accumulators
