@@ -80,6 +80,15 @@ def test_loads_into_lds_have_no_destination_register(tmp_path):
     assert _early(tmp_path, "\tbuffer_load_dwordx4 v1, s[52:55], s18 offen lds\n\tv_mov_b32_e32 v2, v1") == []
 
 
+def test_spilled_registers_above_the_recorded_count_are_found(tmp_path):
+    path = tmp_path / "k.s"
+    meta = "    .name:           _ZN2tg23fp8_gemm_tile256_kernelENS_10GemmParamsE\n    .vgpr_spill_count: {n}\n"
+    path.write_text(meta.format(n=3))
+    assert len(check_hazards.scan_spills(str(path))) == 1
+    path.write_text(meta.format(n=0))
+    assert check_hazards.scan_spills(str(path)) == []
+
+
 @pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
 def test_no_kernel_breaks_either_rule():
     run = subprocess.run([sys.executable, os.path.join(CSRC, "check_hazards.py"), "--build"], capture_output=True, text=True,
